@@ -1,0 +1,142 @@
+"""ctypes binding of ``libhdit.so`` (the C ABI declared in ``include/hdit.h``).
+
+There is no fallback: if the library has not been built the first call raises.
+"""
+import ctypes as C
+import os
+import threading
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libhdit.so")
+
+HDIT_GEMM_MAX_PROBLEMS = 16
+EPI_BIAS, EPI_BIAS_GELU, EPI_GATE_RESIDUAL = 0, 1, 2
+
+
+class GemmProblem(C.Structure):
+    _fields_ = [
+        ("a", C.c_void_p),
+        ("b", C.c_void_p),
+        ("c", C.c_void_p),
+        ("bias", C.c_void_p),
+        ("resid", C.c_void_p),
+        ("gate", C.c_void_p),
+        ("lda", C.c_int64),
+        ("ldb", C.c_int64),
+        ("ldc", C.c_int64),
+        ("ldr", C.c_int64),
+        ("m", C.c_int32),
+        ("n", C.c_int32),
+        ("k", C.c_int32),
+        ("epilogue", C.c_int32),
+        ("rows_per_batch", C.c_int32),
+        ("gate_stride", C.c_int32),
+    ]
+
+
+class SeqSegment(C.Structure):
+    _fields_ = [
+        ("ptr", C.c_void_p),
+        ("stride_b", C.c_int64),
+        ("stride_s", C.c_int64),
+        ("stride_h", C.c_int64),
+        ("len", C.c_int32),
+        ("pad_", C.c_int32),
+    ]
+
+
+class AttnArgs(C.Structure):
+    _fields_ = [
+        ("q", SeqSegment * 2),
+        ("k", SeqSegment * 2),
+        ("v", SeqSegment * 2),
+        ("o", SeqSegment * 2),
+        ("batch", C.c_int32),
+        ("heads", C.c_int32),
+        ("head_dim", C.c_int32),
+        ("scale", C.c_float),
+    ]
+
+
+class QkNormJob(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p),
+        ("stride_b", C.c_int64),
+        ("stride_s", C.c_int64),
+        ("stride_h", C.c_int64),
+        ("weight", C.c_void_p),
+        ("bias", C.c_void_p),
+        ("cos_table", C.c_void_p),
+        ("sin_table", C.c_void_p),
+        ("seq", C.c_int32),
+        ("rope_row0", C.c_int32),
+        ("rope_rows", C.c_int32),
+        ("norm_kind", C.c_int32),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/hdit.h declares
+SIGNATURES = {
+    "hdit_abi_version": (C.c_int, []),
+    "hdit_last_error": (C.c_char_p, []),
+    "hdit_gemm_bf16": (C.c_int, [C.POINTER(GemmProblem), C.c_int, C.c_void_p]),
+    "hdit_attn_fwd_bf16": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p]),
+    "hdit_attn_absmax": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p]),
+    "hdit_attn_fwd_fp8": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p]),
+    "hdit_layernorm_modulate": (
+        C.c_int,
+        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
+         C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_void_p],
+    ),
+    "hdit_gate_residual": (
+        C.c_int,
+        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64,
+         C.c_int64, C.c_int64, C.c_void_p],
+    ),
+    "hdit_adaln_gemv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "hdit_gelu_tanh": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_void_p]),
+    "hdit_qk_norm_rope": (C.c_int, [C.POINTER(QkNormJob), C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p]),
+    "hdit_copy_rows": (
+        C.c_int,
+        [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_void_p],
+    ),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+def lib():
+    """Load (once) and return the bound library; raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise RuntimeError(
+                    f"{LIB_PATH} is missing: the HIP kernels are not built. Run "
+                    "`python -c 'import __graft_entry__ as g; g.build()'` (or hetu_dit_amd.build.build_library())."
+                )
+            handle = C.CDLL(LIB_PATH)
+            for name, (res, args) in SIGNATURES.items():
+                fn = getattr(handle, name)  # AttributeError if the library lacks a declared symbol
+                fn.restype = res
+                fn.argtypes = args
+            _lib = handle
+    return _lib
+
+
+class HditError(RuntimeError):
+    pass
+
+
+_CODES = {-1: "HDIT_EINVAL", -2: "HDIT_EUNSUPPORTED", -3: "HDIT_ELAUNCH"}
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        detail = ""
+        if rc == -3:
+            detail = ": " + lib().hdit_last_error().decode()
+        raise HditError(f"{what} failed with {_CODES.get(rc, rc)}{detail}")

@@ -1,0 +1,27 @@
+// Host-side plumbing shared by the C-ABI entry points: ABI version, per-thread
+// error string, launch check.
+#include <string.h>
+
+#include "hdit_common.h"
+
+namespace {
+thread_local char g_err[256] = "";
+}
+
+namespace hdit_host {
+void set_error(const char* msg) {
+  strncpy(g_err, msg ? msg : "", sizeof(g_err) - 1);
+  g_err[sizeof(g_err) - 1] = 0;
+}
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return HDIT_OK;
+  char buf[256];
+  snprintf(buf, sizeof(buf), "%s: %s", what, hipGetErrorString(e));
+  set_error(buf);
+  return HDIT_ELAUNCH;
+}
+}  // namespace hdit_host
+
+extern "C" __attribute__((visibility("default"))) int hdit_abi_version(void) { return 1; }
+extern "C" __attribute__((visibility("default"))) const char* hdit_last_error(void) { return g_err; }

@@ -1,0 +1,405 @@
+// Bandwidth-bound glue kernels for gfx950: every tensor is touched once, with
+// 16-byte accesses laid out so that a wave reads/writes contiguous 1 KiB runs,
+// statistics in fp32, wave64 cross-lane reductions.
+#include "hdit_common.h"
+
+namespace {
+
+using hdit::pack8;
+using hdit::unpack8;
+using hdit::wave_sum;
+
+// ---------------------------------------------------------------------------
+// LayerNorm (optional affine) + adaLN modulate.  One wave per row; the row
+// stays in registers between the statistics and the write.
+// ---------------------------------------------------------------------------
+template <int NCH>  // 16-byte chunks per lane (row has dim/8 chunks, NCH = ceil(dim/512))
+__global__ void __launch_bounds__(256) ln_modulate_kernel(const __bf16* __restrict__ x, __bf16* __restrict__ y,
+                                                          const float* __restrict__ shift,
+                                                          const float* __restrict__ scale,
+                                                          const __bf16* __restrict__ lw,
+                                                          const __bf16* __restrict__ lb, int64_t rows, int tokens,
+                                                          int dim, int64_t ldx, int64_t ldy, int64_t mod_stride,
+                                                          float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int nchunks = dim >> 3;
+  const __bf16* xr = x + row * ldx;
+  i32x4 raw[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    int c = lane + i * 64;
+    if (c < nchunks) raw[i] = __builtin_nontemporal_load((const i32x4*)(xr + c * 8));
+  }
+  float s = 0.f;
+  float f[NCH][8];
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    int c = lane + i * 64;
+    if (c < nchunks) {
+      unpack8(raw[i], f[i]);
+#pragma unroll
+      for (int e = 0; e < 8; e++) s += f[i][e];
+    }
+  }
+  const float inv_d = 1.0f / (float)dim;
+  const float mean = wave_sum(s) * inv_d;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    int c = lane + i * 64;
+    if (c < nchunks) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        f[i][e] -= mean;
+        q += f[i][e] * f[i][e];
+      }
+    }
+  }
+  const float rstd = rsqrtf(wave_sum(q) * inv_d + eps);
+  const int b = (int)(row / tokens);
+  const float* sh = shift ? shift + (int64_t)b * mod_stride : nullptr;
+  const float* sc = scale ? scale + (int64_t)b * mod_stride : nullptr;
+  __bf16* yr = y + row * ldy;
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    int c = lane + i * 64;
+    if (c < nchunks) {
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = f[i][e] * rstd;
+      if (lw) {
+        float w[8];
+        unpack8(*(const i32x4*)(lw + c * 8), w);
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] *= w[e];
+      }
+      if (lb) {
+        float w[8];
+        unpack8(*(const i32x4*)(lb + c * 8), w);
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] += w[e];
+      }
+      if (sc) {
+        f32x4 s0 = *(const f32x4*)(sc + c * 8), s1 = *(const f32x4*)(sc + c * 8 + 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          o[e] *= 1.0f + s0[e];
+          o[e + 4] *= 1.0f + s1[e];
+        }
+      }
+      if (sh) {
+        f32x4 s0 = *(const f32x4*)(sh + c * 8), s1 = *(const f32x4*)(sh + c * 8 + 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          o[e] += s0[e];
+          o[e + 4] += s1[e];
+        }
+      }
+      __builtin_nontemporal_store(pack8(o), (i32x4*)(yr + c * 8));
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// out = x + gate[b] * y
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) gate_residual_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ y,
+                                                            const float* __restrict__ gate, __bf16* __restrict__ out,
+                                                            int64_t total_chunks, int tokens, int chunks_per_row,
+                                                            int64_t ldx, int64_t ldy, int64_t ldo,
+                                                            int64_t gate_stride) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total_chunks) return;
+  int64_t row = i / chunks_per_row;
+  int c = (int)(i - row * chunks_per_row);
+  int b = (int)(row / tokens);
+  float fx[8], fy[8];
+  unpack8(__builtin_nontemporal_load((const i32x4*)(x + row * ldx + c * 8)), fx);
+  unpack8(__builtin_nontemporal_load((const i32x4*)(y + row * ldy + c * 8)), fy);
+  const float* g = gate + (int64_t)b * gate_stride + c * 8;
+  f32x4 g0 = *(const f32x4*)g, g1 = *(const f32x4*)(g + 4);
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    fx[e] += g0[e] * fy[e];
+    fx[e + 4] += g1[e] * fy[e + 4];
+  }
+  __builtin_nontemporal_store(pack8(fx), (i32x4*)(out + row * ldo + c * 8));
+}
+
+// ---------------------------------------------------------------------------
+// y = gelu_tanh(x + bias)
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) gelu_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ bias,
+                                                   __bf16* __restrict__ y, int64_t total_chunks, int chunks_per_row,
+                                                   int64_t ldx, int64_t ldy) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total_chunks) return;
+  int64_t row = i / chunks_per_row;
+  int c = (int)(i - row * chunks_per_row);
+  float f[8];
+  unpack8(__builtin_nontemporal_load((const i32x4*)(x + row * ldx + c * 8)), f);
+  if (bias) {
+    float w[8];
+    unpack8(*(const i32x4*)(bias + c * 8), w);
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] += w[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++) f[e] = hdit::gelu_tanh_f(f[e]);
+  __builtin_nontemporal_store(pack8(f), (i32x4*)(y + row * ldy + c * 8));
+}
+
+// ---------------------------------------------------------------------------
+// adaLN projection: out[b, n] = W[n, :] . silu(temb[b, :]) + bias[n]
+// One wave per output row; the weight row is streamed once for all batches.
+// ---------------------------------------------------------------------------
+template <int MAXB>
+__global__ void __launch_bounds__(256) adaln_gemv_kernel(const __bf16* __restrict__ temb, const __bf16* __restrict__ w,
+                                                         const __bf16* __restrict__ bias, float* __restrict__ out,
+                                                         int batch, int n, int k) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n) return;
+  const int nchunks = k >> 3;
+  float acc[MAXB];
+#pragma unroll
+  for (int b = 0; b < MAXB; b++) acc[b] = 0.f;
+  const __bf16* wr = w + (int64_t)row * k;
+  for (int c = lane; c < nchunks; c += 64) {
+    float fw[8];
+    unpack8(__builtin_nontemporal_load((const i32x4*)(wr + c * 8)), fw);
+#pragma unroll
+    for (int b = 0; b < MAXB; b++) {
+      if (b < batch) {
+        float ft[8];
+        unpack8(*(const i32x4*)(temb + (int64_t)b * k + c * 8), ft);
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[b] += fw[e] * hdit::silu_f(ft[e]);
+      }
+    }
+  }
+  float bv = bias ? (float)bias[row] : 0.f;
+#pragma unroll
+  for (int b = 0; b < MAXB; b++) {
+    if (b < batch) {
+      float r = wave_sum(acc[b]);
+      if (lane == 0) out[(int64_t)b * n + row] = r + bv;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Per-head QK norm (RMS / LayerNorm) + rotate-pairs RoPE, in place.
+// A head vector of HD elements is held by HD/8 adjacent lanes (8 elements each).
+// ---------------------------------------------------------------------------
+struct QkJobs {
+  int count;
+  hdit_qknorm_job j[4];
+};
+
+template <int HD>
+__global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkJobs jobs, int batch, int heads, float eps) {
+  constexpr int LPH = HD / 8;  // lanes per head vector
+  const hdit_qknorm_job& job = jobs.j[blockIdx.y];
+  const int64_t vec = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPH;
+  const int c = threadIdx.x % LPH;
+  const int64_t nvec = (int64_t)batch * job.seq * heads;
+  if (vec >= nvec) return;
+  const int h = (int)(vec % heads);
+  const int64_t bs = vec / heads;
+  const int s = (int)(bs % job.seq);
+  const int b = (int)(bs / job.seq);
+  __bf16* p = (__bf16*)job.x + b * job.stride_b + s * job.stride_s + h * job.stride_h + c * 8;
+  float f[8];
+  unpack8(*(const i32x4*)p, f);
+  if (job.norm_kind == 1) {
+    float q = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) q += f[e] * f[e];
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) q += __shfl_xor(q, off, 64);
+    float r = rsqrtf(q * (1.0f / HD) + eps);
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] *= r;
+  } else if (job.norm_kind == 2) {
+    float sm = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) sm += f[e];
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) sm += __shfl_xor(sm, off, 64);
+    float mean = sm * (1.0f / HD);
+    float q = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      f[e] -= mean;
+      q += f[e] * f[e];
+    }
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) q += __shfl_xor(q, off, 64);
+    float r = rsqrtf(q * (1.0f / HD) + eps);
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] *= r;
+  }
+  if (job.norm_kind != 0) {
+    if (job.weight) {
+      float w[8];
+      unpack8(*(const i32x4*)((const __bf16*)job.weight + c * 8), w);
+#pragma unroll
+      for (int e = 0; e < 8; e++) f[e] *= w[e];
+    }
+    if (job.bias) {
+      float w[8];
+      unpack8(*(const i32x4*)((const __bf16*)job.bias + c * 8), w);
+#pragma unroll
+      for (int e = 0; e < 8; e++) f[e] += w[e];
+    }
+  }
+  const int rr = s - job.rope_row0;
+  if (job.cos_table && rr >= 0 && rr < job.rope_rows) {
+    const float* cp = job.cos_table + (int64_t)rr * HD + c * 8;
+    const float* sp = job.sin_table + (int64_t)rr * HD + c * 8;
+    f32x4 c0 = *(const f32x4*)cp, c1 = *(const f32x4*)(cp + 4);
+    f32x4 s0 = *(const f32x4*)sp, s1 = *(const f32x4*)(sp + 4);
+    float cs[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+    float sn[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+      o[e] = f[e] * cs[e] - f[e + 1] * sn[e];
+      o[e + 1] = f[e + 1] * cs[e + 1] + f[e] * sn[e + 1];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] = o[e];
+  }
+  *(i32x4*)p = pack8(f);
+}
+
+__global__ void __launch_bounds__(256) copy_rows_kernel(const __bf16* __restrict__ src, __bf16* __restrict__ dst,
+                                                        int64_t total_chunks, int tokens, int chunks_per_row,
+                                                        int64_t src_sb, int64_t src_st, int64_t dst_sb,
+                                                        int64_t dst_st) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total_chunks) return;
+  int64_t row = i / chunks_per_row;
+  int c = (int)(i - row * chunks_per_row);
+  int64_t b = row / tokens, t = row - b * tokens;
+  i32x4 v = __builtin_nontemporal_load((const i32x4*)(src + b * src_sb + t * src_st + c * 8));
+  __builtin_nontemporal_store(v, (i32x4*)(dst + b * dst_sb + t * dst_st + c * 8));
+}
+
+inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate(const void* x, void* y, const float* shift, const float* scale,
+                                       const void* ln_weight, const void* ln_bias, int batch, int tokens, int dim,
+                                       int64_t ldx, int64_t ldy, int64_t mod_stride, float eps, void* stream) {
+  if (!x || !y || batch < 0 || tokens < 0 || dim <= 0) return HDIT_EINVAL;
+  if (dim % 8 || ldx % 8 || ldy % 8 || mod_stride % 4) return HDIT_EINVAL;
+  if (dim > 8192) return HDIT_EUNSUPPORTED;
+  if (!aligned16(x) || !aligned16(y) || !aligned16(shift) || !aligned16(scale) || !aligned16(ln_weight) ||
+      !aligned16(ln_bias))
+    return HDIT_EINVAL;
+  int64_t rows = (int64_t)batch * tokens;
+  if (rows == 0) return HDIT_OK;
+  dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  int nch = (dim / 8 + 63) / 64;
+#define LN_LAUNCH(N)                                                                                             \
+  hipLaunchKernelGGL(ln_modulate_kernel<N>, grid, block, 0, s, (const __bf16*)x, (__bf16*)y, shift, scale,      \
+                     (const __bf16*)ln_weight, (const __bf16*)ln_bias, rows, tokens, dim, ldx, ldy, mod_stride, \
+                     eps)
+  if (nch <= 1) LN_LAUNCH(1);
+  else if (nch <= 2) LN_LAUNCH(2);
+  else if (nch <= 3) LN_LAUNCH(3);
+  else if (nch <= 4) LN_LAUNCH(4);
+  else if (nch <= 6) LN_LAUNCH(6);
+  else if (nch <= 8) LN_LAUNCH(8);
+  else if (nch <= 12) LN_LAUNCH(12);
+  else LN_LAUNCH(16);
+#undef LN_LAUNCH
+  return hdit_host::check_launch("hdit_layernorm_modulate");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_gate_residual(const void* x, const void* y, const float* gate, void* out, int batch, int tokens,
+                                  int dim, int64_t ldx, int64_t ldy, int64_t ldo, int64_t gate_stride,
+                                  void* stream) {
+  if (!x || !y || !gate || !out || batch < 0 || tokens < 0 || dim <= 0) return HDIT_EINVAL;
+  if (dim % 8 || ldx % 8 || ldy % 8 || ldo % 8 || gate_stride % 4) return HDIT_EINVAL;
+  if (!aligned16(x) || !aligned16(y) || !aligned16(out) || !aligned16(gate)) return HDIT_EINVAL;
+  int64_t total = (int64_t)batch * tokens * (dim / 8);
+  if (total == 0) return HDIT_OK;
+  hipLaunchKernelGGL(gate_residual_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __bf16*)x, (const __bf16*)y, gate, (__bf16*)out, total, tokens, dim / 8, ldx, ldy, ldo,
+                     gate_stride);
+  return hdit_host::check_launch("hdit_gate_residual");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_gelu_tanh(const void* x, const void* bias, void* y, int64_t rows, int dim, int64_t ldx,
+                              int64_t ldy, void* stream) {
+  if (!x || !y || rows < 0 || dim <= 0 || dim % 8 || ldx % 8 || ldy % 8) return HDIT_EINVAL;
+  if (!aligned16(x) || !aligned16(y) || !aligned16(bias)) return HDIT_EINVAL;
+  int64_t total = rows * (dim / 8);
+  if (total == 0) return HDIT_OK;
+  hipLaunchKernelGGL(gelu_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __bf16*)x, (const __bf16*)bias, (__bf16*)y, total, dim / 8, ldx, ldy);
+  return hdit_host::check_launch("hdit_gelu_tanh");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_adaln_gemv(const void* temb, const void* w, const void* bias, float* out, int batch, int n, int k,
+                               void* stream) {
+  if (!temb || !w || !out || batch <= 0 || n <= 0 || k <= 0) return HDIT_EINVAL;
+  if (batch > 8) return HDIT_EUNSUPPORTED;
+  if (k % 8 || !aligned16(temb) || !aligned16(w)) return HDIT_EINVAL;
+  dim3 grid((n + 3) / 4), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  if (batch <= 2)
+    hipLaunchKernelGGL(adaln_gemv_kernel<2>, grid, block, 0, s, (const __bf16*)temb, (const __bf16*)w,
+                       (const __bf16*)bias, out, batch, n, k);
+  else
+    hipLaunchKernelGGL(adaln_gemv_kernel<8>, grid, block, 0, s, (const __bf16*)temb, (const __bf16*)w,
+                       (const __bf16*)bias, out, batch, n, k);
+  return hdit_host::check_launch("hdit_adaln_gemv");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_qk_norm_rope(const hdit_qknorm_job* jobs, int count, int batch, int heads, int head_dim, float eps,
+                                 void* stream) {
+  if (!jobs || count <= 0 || count > 4 || batch <= 0 || heads <= 0) return HDIT_EINVAL;
+  if (head_dim != 64 && head_dim != 128) return HDIT_EUNSUPPORTED;
+  QkJobs tab;
+  tab.count = count;
+  int64_t max_vec = 0;
+  for (int i = 0; i < count; i++) {
+    const hdit_qknorm_job& j = jobs[i];
+    if (!j.x || j.seq < 0 || j.norm_kind < 0 || j.norm_kind > 2) return HDIT_EINVAL;
+    if (j.stride_b % 8 || j.stride_s % 8 || j.stride_h % 8 || !aligned16(j.x)) return HDIT_EINVAL;
+    if (!aligned16(j.weight) || !aligned16(j.bias) || !aligned16(j.cos_table) || !aligned16(j.sin_table))
+      return HDIT_EINVAL;
+    if (j.cos_table && !j.sin_table) return HDIT_EINVAL;
+    tab.j[i] = j;
+    int64_t nv = (int64_t)batch * j.seq * heads;
+    if (nv > max_vec) max_vec = nv;
+  }
+  if (max_vec == 0) return HDIT_OK;
+  int lph = head_dim / 8;
+  int64_t threads = max_vec * lph;
+  dim3 grid((unsigned)((threads + 255) / 256), count), block(256);
+  if (head_dim == 64)
+    hipLaunchKernelGGL(qk_norm_rope_kernel<64>, grid, block, 0, (hipStream_t)stream, tab, batch, heads, eps);
+  else
+    hipLaunchKernelGGL(qk_norm_rope_kernel<128>, grid, block, 0, (hipStream_t)stream, tab, batch, heads, eps);
+  return hdit_host::check_launch("hdit_qk_norm_rope");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_copy_rows(const void* src, void* dst, int batch, int tokens, int dim, int64_t src_sb,
+                              int64_t src_st, int64_t dst_sb, int64_t dst_st, void* stream) {
+  if (!src || !dst || batch < 0 || tokens < 0 || dim <= 0 || dim % 8) return HDIT_EINVAL;
+  if (src_sb % 8 || src_st % 8 || dst_sb % 8 || dst_st % 8 || !aligned16(src) || !aligned16(dst)) return HDIT_EINVAL;
+  int64_t total = (int64_t)batch * tokens * (dim / 8);
+  if (total == 0) return HDIT_OK;
+  hipLaunchKernelGGL(copy_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __bf16*)src, (__bf16*)dst, total, tokens, dim / 8, src_sb, src_st, dst_sb, dst_st);
+  return hdit_host::check_launch("hdit_copy_rows");
+}

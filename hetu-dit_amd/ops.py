@@ -1,0 +1,282 @@
+"""Tensor-level entry to the C ABI: checks dtypes/devices, extracts pointers and
+strides, enqueues on PyTorch's current HIP stream.  PyTorch is only the owner
+of device memory and streams here; every computation happens in ``libhdit.so``.
+
+The same functions are registered as ``torch.ops.hdit.*`` custom ops (with
+fake/meta kernels) in ``torch_ops.py`` for callers that trace the model.
+"""
+import ctypes as C
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import EPI_BIAS, EPI_BIAS_GELU, EPI_GATE_RESIDUAL, AttnArgs, GemmProblem, QkNormJob, check
+
+bf16 = torch.bfloat16
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need(t: torch.Tensor, dtype, name: str):
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+
+
+# ---------------------------------------------------------------------------
+# grouped GEMM
+# ---------------------------------------------------------------------------
+
+def gemm_problem(
+    a: torch.Tensor,
+    w: torch.Tensor,
+    out: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    epilogue: int = EPI_BIAS,
+    resid: Optional[torch.Tensor] = None,
+    gate: Optional[torch.Tensor] = None,
+    rows_per_batch: int = 0,
+) -> GemmProblem:
+    """Describe out[m, n] = epilogue(a[m, k] @ w[n, k]^T + bias).
+
+    a, out (and resid) are 2-D views with unit inner stride (row stride free);
+    gate is an f32 [batch, n] view with unit inner stride."""
+    _need(a, bf16, "a"), _need(w, bf16, "w"), _need(out, bf16, "out")
+    m, k = a.shape
+    n, k2 = w.shape
+    if k2 != k or tuple(out.shape) != (m, n):
+        raise ValueError(f"gemm shapes do not agree: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)}")
+    if a.stride(1) != 1 or w.stride(1) != 1 or out.stride(1) != 1:
+        raise ValueError("gemm operands need a unit inner stride")
+    p = GemmProblem()
+    p.a, p.b, p.c = a.data_ptr(), w.data_ptr(), out.data_ptr()
+    p.lda, p.ldb, p.ldc = a.stride(0) if m > 1 else k, w.stride(0), out.stride(0) if m > 1 else n
+    p.m, p.n, p.k = m, n, k
+    p.epilogue = epilogue
+    if bias is not None:
+        _need(bias, bf16, "bias")
+        if bias.numel() != n or not bias.is_contiguous():
+            raise ValueError("bias must be a contiguous [n] vector")
+        p.bias = bias.data_ptr()
+    if epilogue == EPI_GATE_RESIDUAL:
+        _need(resid, bf16, "resid"), _need(gate, torch.float32, "gate")
+        if tuple(resid.shape) != (m, n) or resid.stride(1) != 1:
+            raise ValueError("resid must be [m, n] with unit inner stride")
+        if gate.dim() != 2 or gate.shape[1] != n or gate.stride(1) != 1:
+            raise ValueError("gate must be [batch, n] with unit inner stride")
+        if rows_per_batch <= 0 or m > rows_per_batch * gate.shape[0]:
+            raise ValueError("rows_per_batch does not cover m")
+        p.resid, p.gate = resid.data_ptr(), gate.data_ptr()
+        p.ldr = resid.stride(0) if m > 1 else n
+        p.rows_per_batch, p.gate_stride = rows_per_batch, gate.stride(0) if gate.shape[0] > 1 else n
+    p._keep = (a, w, out, bias, resid, gate)  # the struct only holds raw pointers
+    return p
+
+
+def gemm_launch(problems: Sequence[GemmProblem]):
+    n = len(problems)
+    arr = (GemmProblem * n)(*problems)
+    check(_lib.lib().hdit_gemm_bf16(arr, n, _stream()), "hdit_gemm_bf16")
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, gelu: bool = False,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = x @ w^T + bias (optionally GELU-tanh) on [..., k] bf16 input."""
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    if out is None:
+        out = torch.empty(*lead, w.shape[0], dtype=bf16, device=x.device)
+    gemm_launch([gemm_problem(x2, w, out.view(-1, w.shape[0]), bias, EPI_BIAS_GELU if gelu else EPI_BIAS)])
+    return out
+
+
+# ---------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------
+
+def _fill_segments(dst, tensors: Sequence[torch.Tensor], name: str) -> Tuple[int, int, int, int]:
+    """tensors: 1 or 2 views [B, S, H, d] with unit stride on d."""
+    if not 1 <= len(tensors) <= 2:
+        raise ValueError(f"{name}: one or two segments expected")
+    B, _, H, D = tensors[0].shape
+    total = 0
+    for i, t in enumerate(tensors):
+        _need(t, bf16, name)
+        if t.dim() != 4 or t.shape[0] != B or t.shape[2] != H or t.shape[3] != D:
+            raise ValueError(f"{name}: segment shapes disagree")
+        if t.stride(3) != 1:
+            raise ValueError(f"{name}: head_dim must be contiguous")
+        dst[i].ptr = t.data_ptr()
+        dst[i].stride_b, dst[i].stride_s, dst[i].stride_h = t.stride(0), t.stride(1), t.stride(2)
+        dst[i].len = t.shape[1]
+        total += t.shape[1]
+    return B, total, H, D
+
+
+def attention_args(q, k, v, o, scale: float = 0.0) -> AttnArgs:
+    a = AttnArgs()
+    B, sq, H, D = _fill_segments(a.q, q, "q")
+    Bk, skv, Hk, Dk = _fill_segments(a.k, k, "k")
+    Bv, skv2, Hv, Dv = _fill_segments(a.v, v, "v")
+    Bo, so, Ho, Do = _fill_segments(a.o, o, "o")
+    if (Bk, Hk, Dk) != (B, H, D) or (Bv, Hv, Dv) != (B, H, D) or (Bo, Ho, Do) != (B, H, D) or so != sq or skv2 != skv:
+        raise ValueError("attention operand shapes disagree")
+    a.batch, a.heads, a.head_dim, a.scale = B, H, D, scale
+    a._keep = (tuple(q), tuple(k), tuple(v), tuple(o))
+    return a
+
+
+def attention(q: Sequence[torch.Tensor], k: Sequence[torch.Tensor], v: Sequence[torch.Tensor],
+              out: Optional[Sequence[torch.Tensor]] = None, scale: float = 0.0, fp8: bool = False):
+    """Joint non-causal attention.  q/k/v are lists of one or two [B, S, H, d]
+    bf16 views (the segments of the joint sequence).  Returns the list of
+    output segments (allocated [B, S, H, d] contiguous when not given)."""
+    if out is None:
+        out = [torch.empty(t.shape, dtype=bf16, device=t.device) for t in q]
+    args = attention_args(q, k, v, out, scale)
+    lib = _lib.lib()
+    if fp8:
+        absmax = torch.empty(3, args.batch, args.heads, dtype=torch.float32, device=q[0].device)
+        check(lib.hdit_attn_absmax(C.byref(args), absmax.data_ptr(), _stream()), "hdit_attn_absmax")
+        check(lib.hdit_attn_fwd_fp8(C.byref(args), absmax.data_ptr(), _stream()), "hdit_attn_fwd_fp8")
+    else:
+        check(lib.hdit_attn_fwd_bf16(C.byref(args), _stream()), "hdit_attn_fwd_bf16")
+    return list(out)
+
+
+# ---------------------------------------------------------------------------
+# glue
+# ---------------------------------------------------------------------------
+
+def _as3d(x: torch.Tensor, name: str) -> Tuple[int, int, int, int]:
+    """[B, T, D] view whose batch stride equals T * row stride; returns (B, T, D, ld)."""
+    _need(x, bf16, name)
+    if x.dim() != 3 or x.stride(2) != 1:
+        raise ValueError(f"{name} must be [batch, tokens, dim] with unit inner stride")
+    B, T, D = x.shape
+    ld = x.stride(1) if T > 1 else D
+    if B > 1 and x.stride(0) != T * ld:
+        raise ValueError(f"{name}: batch stride must be tokens * row stride")
+    return B, T, D, ld
+
+
+def _mod(v: Optional[torch.Tensor], B: int, D: int, name: str):
+    if v is None:
+        return None, 0
+    _need(v, torch.float32, name)
+    if tuple(v.shape) != (B, D) or v.stride(1) != 1:
+        raise ValueError(f"{name} must be f32 [batch, dim] with unit inner stride")
+    return v.data_ptr(), (v.stride(0) if B > 1 else D)
+
+
+def layernorm_modulate(x, shift=None, scale=None, eps: float = 1e-6, ln_weight=None, ln_bias=None, out=None):
+    B, T, D, ldx = _as3d(x, "x")
+    if out is None:
+        out = torch.empty(B, T, D, dtype=bf16, device=x.device)
+    _, _, _, ldy = _as3d(out, "out")
+    sh, st1 = _mod(shift, B, D, "shift")
+    sc, st2 = _mod(scale, B, D, "scale")
+    if sh is not None and sc is not None and st1 != st2:
+        raise ValueError("shift and scale must share a batch stride")
+    for w in (ln_weight, ln_bias):
+        if w is not None:
+            _need(w, bf16, "ln affine")
+    check(
+        _lib.lib().hdit_layernorm_modulate(x.data_ptr(), out.data_ptr(), sh, sc, _ptr(ln_weight), _ptr(ln_bias), B, T, D,
+                                           ldx, ldy, st1 or st2, eps, _stream()),
+        "hdit_layernorm_modulate",
+    )
+    return out
+
+
+def gate_residual(x, y, gate, out=None):
+    B, T, D, ldx = _as3d(x, "x")
+    _, _, _, ldy = _as3d(y, "y")
+    if out is None:
+        out = torch.empty(B, T, D, dtype=bf16, device=x.device)
+    _, _, _, ldo = _as3d(out, "out")
+    g, gs = _mod(gate, B, D, "gate")
+    check(_lib.lib().hdit_gate_residual(x.data_ptr(), y.data_ptr(), g, out.data_ptr(), B, T, D, ldx, ldy, ldo, gs, _stream()),
+          "hdit_gate_residual")
+    return out
+
+
+def adaln_gemv(temb: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """f32 [B, n] = w @ silu(temb) + bias."""
+    _need(temb, bf16, "temb"), _need(w, bf16, "w")
+    if not (temb.is_contiguous() and w.is_contiguous()):
+        raise ValueError("adaln_gemv operands must be contiguous")
+    B, k = temb.shape
+    n = w.shape[0]
+    if bias is not None:
+        _need(bias, bf16, "bias")
+    out = torch.empty(B, n, dtype=torch.float32, device=temb.device)
+    check(_lib.lib().hdit_adaln_gemv(temb.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), B, n, k, _stream()),
+          "hdit_adaln_gemv")
+    return out
+
+
+def gelu_tanh(x: torch.Tensor, bias: Optional[torch.Tensor] = None, out=None) -> torch.Tensor:
+    _need(x, bf16, "x")
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(1) != 1:
+        raise ValueError("x needs a unit inner stride")
+    if out is None:
+        out = torch.empty(x.shape, dtype=bf16, device=x.device)
+    o2 = out.view(-1, x.shape[-1])
+    rows, dim = x2.shape
+    check(_lib.lib().hdit_gelu_tanh(x2.data_ptr(), _ptr(bias), o2.data_ptr(), rows, dim,
+                                    x2.stride(0) if rows > 1 else dim, o2.stride(0) if rows > 1 else dim, _stream()),
+          "hdit_gelu_tanh")
+    return out
+
+
+def qk_norm_rope_job(x: torch.Tensor, norm_kind: int = 0, weight=None, bias=None, cos=None, sin=None,
+                     rope_row0: int = 0) -> QkNormJob:
+    """x: [B, S, H, d] bf16 view (unit stride on d), modified in place."""
+    _need(x, bf16, "x")
+    if x.dim() != 4 or x.stride(3) != 1:
+        raise ValueError("x must be [B, S, H, d] with contiguous d")
+    j = QkNormJob()
+    j.x = x.data_ptr()
+    j.stride_b, j.stride_s, j.stride_h = x.stride(0), x.stride(1), x.stride(2)
+    j.seq = x.shape[1]
+    j.norm_kind = norm_kind
+    if weight is not None:
+        _need(weight, bf16, "weight")
+        j.weight = weight.data_ptr()
+    if bias is not None:
+        _need(bias, bf16, "bias")
+        j.bias = bias.data_ptr()
+    if cos is not None:
+        _need(cos, torch.float32, "cos"), _need(sin, torch.float32, "sin")
+        if cos.shape != sin.shape or cos.shape[1] != x.shape[3] or not (cos.is_contiguous() and sin.is_contiguous()):
+            raise ValueError("cos/sin must be contiguous f32 [rows, head_dim]")
+        j.cos_table, j.sin_table = cos.data_ptr(), sin.data_ptr()
+        j.rope_row0, j.rope_rows = rope_row0, cos.shape[0]
+    j._keep = (x, weight, bias, cos, sin)
+    return j
+
+
+def qk_norm_rope(jobs: List[QkNormJob], batch: int, heads: int, head_dim: int, eps: float = 1e-6):
+    arr = (QkNormJob * len(jobs))(*jobs)
+    check(_lib.lib().hdit_qk_norm_rope(arr, len(jobs), batch, heads, head_dim, eps, _stream()), "hdit_qk_norm_rope")
+
+
+def copy_rows(src: torch.Tensor, dst: torch.Tensor):
+    """dst[b, t, :] = src[b, t, :] for [B, T, D] bf16 views with unit inner stride."""
+    _need(src, bf16, "src"), _need(dst, bf16, "dst")
+    if src.shape != dst.shape or src.dim() != 3 or src.stride(2) != 1 or dst.stride(2) != 1:
+        raise ValueError("copy_rows needs equal-shape [B, T, D] views with unit inner stride")
+    B, T, D = src.shape
+    check(_lib.lib().hdit_copy_rows(src.data_ptr(), dst.data_ptr(), B, T, D, src.stride(0), src.stride(1), dst.stride(0),
+                                    dst.stride(1), _stream()), "hdit_copy_rows")
+    return dst

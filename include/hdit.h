@@ -1,0 +1,178 @@
+/*
+ * hdit.h -- C ABI of the MI355X (gfx950) DiT denoise-step hot path.
+ *
+ * Every entry point takes plain device pointers, sizes and strides (in
+ * elements), a HIP stream passed as void*, and returns 0 on success or a
+ * negative HDIT_E* code.  No entry point allocates, frees, synchronises or
+ * throws; work is enqueued on the given stream.  bf16 tensors are raw 16-bit
+ * storage; "f32" pointers are IEEE binary32.
+ *
+ * The reference (PKU-DAIR/Hetu-DiT) is pure Python and has no FFI of its own:
+ * each entry point below names the Python call site it replaces
+ * (paths relative to hetu_dit/model_executor/diffusion_executor/ unless
+ * stated otherwise).
+ */
+#ifndef HDIT_H
+#define HDIT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HDIT_OK 0
+#define HDIT_EINVAL (-1)      /* bad shape / stride / alignment / null pointer */
+#define HDIT_EUNSUPPORTED (-2) /* shape outside what the kernels are built for */
+#define HDIT_ELAUNCH (-3)     /* the HIP runtime refused the launch */
+
+/* Version of this ABI; bumped when a struct below changes. */
+int hdit_abi_version(void);
+/* Static string describing the last HDIT_ELAUNCH on this thread ("" if none). */
+const char* hdit_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * Grouped bf16 GEMM with fused epilogue:  C = epilogue(A . B^T + bias)
+ *
+ * A [m, k] row-major (lda), B [n, k] row-major (ldb; an nn.Linear weight),
+ * C [m, n] row-major (ldc); fp32 accumulation on MFMA.  Requirements:
+ * k % 64 == 0, n % 8 == 0, lda/ldb % 8 == 0, ldc/ldr % 4 == 0, pointers
+ * 16-byte (A, B) / 8-byte (C, resid, bias) aligned.  Up to
+ * HDIT_GEMM_MAX_PROBLEMS problems share one launch (the image and text streams
+ * of a joint block, or q|k|v|mlp of a fused projection).
+ *
+ * Replaces the nn.Linear calls at layers/attention_processor.py:688-695 (SD3
+ * q/k/v + add_q/k/v), :844-846,:867-869 (Flux), :1054-1056 (CogVideoX),
+ * :419-421,:294-295,:268 (out-projections, bias re-added at :428-447),
+ * layers/feedforward.py:74-77 (MLP + output bias), and the diffusers block's
+ * gated residual that consumes them (transformer_sd3.py:136-152).
+ * ---------------------------------------------------------------------- */
+#define HDIT_GEMM_MAX_PROBLEMS 16
+
+#define HDIT_EPI_BIAS 0          /* C = acc + bias */
+#define HDIT_EPI_BIAS_GELU 1     /* C = gelu_tanh(acc + bias) */
+#define HDIT_EPI_GATE_RESIDUAL 2 /* C = resid + gate[row / rows_per_batch] * (acc + bias) */
+
+typedef struct hdit_gemm_problem {
+  const void* a;     /* bf16 [m, k] */
+  const void* b;     /* bf16 [n, k] */
+  void* c;           /* bf16 [m, n] */
+  const void* bias;  /* bf16 [n] or NULL */
+  const void* resid; /* bf16 [m, n] (ldr), HDIT_EPI_GATE_RESIDUAL only; may alias c */
+  const float* gate; /* f32, element (batch, col) at gate[batch * gate_stride + col] */
+  int64_t lda, ldb, ldc, ldr;
+  int32_t m, n, k;
+  int32_t epilogue;
+  int32_t rows_per_batch; /* rows of A per batch element (gate lookup) */
+  int32_t gate_stride;
+} hdit_gemm_problem;
+
+int hdit_gemm_bf16(const hdit_gemm_problem* problems, int count, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Joint (image + text) flash attention, non-causal, no mask, bf16 in/out,
+ * fp32 online softmax on MFMA.
+ *
+ * Q, K, V and O are each the concatenation, along the sequence, of up to two
+ * segments that live in different buffers (segment 1 may have len 0): this is
+ * the torch.cat([image, text]) of attention_processor.py:742-744 (SD3),
+ * :894-896 (Flux, [text, image]) and the cat([text-K, cached image-K]) of
+ * :908-922 without the copy.  Element (b, s, h, e) of a segment is at
+ * ptr[b*stride_b + s*stride_s + h*stride_h + e]; head_dim is contiguous and
+ * must be 64 or 128; strides must be multiples of 8 elements and pointers
+ * 16-byte aligned.  sum(q.len) may differ from sum(k.len) (a PipeFusion query
+ * patch against the whole stale K/V buffer); k and v segment lengths must
+ * agree.  scale <= 0 selects 1/sqrt(head_dim), which is what the reference's
+ * flash_attn_func / F.scaled_dot_product_attention calls use (:752-779,
+ * :962-971, :1139-1151).
+ * ---------------------------------------------------------------------- */
+typedef struct hdit_seq_segment {
+  const void* ptr;
+  int64_t stride_b, stride_s, stride_h;
+  int32_t len;
+  int32_t pad_;
+} hdit_seq_segment;
+
+typedef struct hdit_attn_args {
+  hdit_seq_segment q[2], k[2], v[2], o[2]; /* o[i].ptr is written */
+  int32_t batch, heads, head_dim;
+  float scale;
+} hdit_attn_args;
+
+int hdit_attn_fwd_bf16(const hdit_attn_args* args, void* stream);
+
+/* Same contract; Q, K, V are quantised to fp8-e4m3 (OCP) on the fly with one
+ * absmax scale per (batch, head) taken from `absmax` (f32 [3, batch, heads]:
+ * q, k, v), P is re-quantised per tile.  `absmax` is produced by
+ * hdit_attn_absmax.  No counterpart exists in the reference (it has no fp8
+ * path); the call site is the same as hdit_attn_fwd_bf16. */
+int hdit_attn_absmax(const hdit_attn_args* args, float* absmax, void* stream);
+int hdit_attn_fwd_fp8(const hdit_attn_args* args, const float* absmax, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Bandwidth-bound glue, one coalesced pass each.
+ * ---------------------------------------------------------------------- */
+
+/* y[b,t,:] = LayerNorm(x[b,t,:]; eps, optional affine ln_weight/ln_bias (bf16))
+ *            * (1 + scale[b,:]) + shift[b,:]
+ * x, y bf16 [batch, tokens, dim] with row stride ldx / ldy and batch stride
+ * tokens*ld; shift/scale f32 with batch stride mod_stride (NULL => 0).
+ * dim % 8 == 0, dim <= 8192.  Replaces diffusers AdaLayerNormZero /
+ * AdaLayerNormZeroSingle / AdaLayerNormContinuous / CogVideoXLayerNormZero and
+ * the norm2 + modulate of the blocks called at transformer_sd3.py:136-152,
+ * transformer_flux.py:160-165,:194-198, cogvideox_transformer_3d.py:122-127. */
+int hdit_layernorm_modulate(const void* x, void* y, const float* shift, const float* scale,
+                            const void* ln_weight, const void* ln_bias, int batch, int tokens,
+                            int dim, int64_t ldx, int64_t ldy, int64_t mod_stride, float eps,
+                            void* stream);
+
+/* out = x + gate[b,:] * y   (bf16 [batch, tokens, dim], gate f32).  The gated
+ * residual of the same blocks when it is not fused into a GEMM epilogue. */
+int hdit_gate_residual(const void* x, const void* y, const float* gate, void* out, int batch,
+                       int tokens, int dim, int64_t ldx, int64_t ldy, int64_t ldo,
+                       int64_t gate_stride, void* stream);
+
+/* out[b, :] = W . silu(temb[b, :]) + bias   (W bf16 [n, k], temb bf16 [batch, k],
+ * bias bf16 [n] or NULL, out f32 [batch, n]); batch <= 8, k % 8 == 0.
+ * The `linear(silu(emb))` of every adaLN module (weight-bandwidth bound). */
+int hdit_adaln_gemv(const void* temb, const void* w, const void* bias, float* out, int batch,
+                    int n, int k, void* stream);
+
+/* y = gelu_tanh(x + bias) elementwise (bf16 [rows, dim]); bias may be NULL.
+ * diffusers GELU(approximate="tanh") inside the FeedForward wrapped at
+ * layers/feedforward.py:17-78, when not fused into the GEMM epilogue. */
+int hdit_gelu_tanh(const void* x, const void* bias, void* y, int64_t rows, int dim, int64_t ldx,
+                   int64_t ldy, void* stream);
+
+/* In-place per-head QK normalisation + rotary embedding on x[b, s, h, :]
+ * (bf16, strides as in hdit_seq_segment, head_dim 64 or 128):
+ *   norm_kind 0: none; 1: RMSNorm(eps, weight); 2: LayerNorm(eps, weight, bias)
+ *   then, for rows s in [rope_row0, rope_row0 + rope_rows):
+ *   out = x*cos[s - rope_row0] + rotate_pairs(x)*sin[s - rope_row0]  (fp32 math)
+ * cos/sin f32 [rope_rows, head_dim] (NULL => no rotation).  Up to 4 jobs per
+ * launch.  Replaces attn.norm_q/norm_k/norm_added_q/norm_added_k and
+ * apply_rotary_emb at attention_processor.py:68-120,:859-905,:1069-1082. */
+typedef struct hdit_qknorm_job {
+  void* x;
+  int64_t stride_b, stride_s, stride_h;
+  const void* weight; /* bf16 [head_dim] or NULL */
+  const void* bias;   /* bf16 [head_dim] or NULL */
+  const float* cos_table;
+  const float* sin_table;
+  int32_t seq, rope_row0, rope_rows, norm_kind;
+} hdit_qknorm_job;
+
+int hdit_qk_norm_rope(const hdit_qknorm_job* jobs, int count, int batch, int heads, int head_dim,
+                      float eps, void* stream);
+
+/* Plain strided copy of bf16 rows: dst[b, t, :dim] = src[b, t, :dim]; used to
+ * place a [batch, tokens, dim] tensor into a slice of a larger buffer (the
+ * in-place K/V patch overwrite of core/resource_manager/cache_manager.py:208-231).
+ * dim % 8 == 0. */
+int hdit_copy_rows(const void* src, void* dst, int batch, int tokens, int dim, int64_t src_sb,
+                   int64_t src_st, int64_t dst_sb, int64_t dst_st, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HDIT_H */

@@ -1,0 +1,71 @@
+"""CPU oracle for the one-GPU DiT denoise-step hot path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing under ``oracle/`` is part of the shipped
+product: it may be imported only by ``tests/``, by ``__graft_entry__.smoke()``
+and by the ``cpu_baseline`` leg of ``bench.py``, and there only as the checker
+or as the timed CPU baseline.  The product package never imports it.
+
+The oracle restates, in explicit fp32 formulas on the CPU, what the reference
+computes for the MMDiT / DiT transformer block.  The reference owns the
+attention wrapper, the attention processors, ``apply_rotary_emb``, the
+FeedForward wrapper, the block-loop callers and the KV ``CacheManager``
+(``hetu_dit/model_executor/diffusion_executor/layers/attention_processor.py``,
+``.../layers/feedforward.py``, ``hetu_dit/core/resource_manager/cache_manager.py``).
+The block arithmetic itself (adaLN-Zero, LayerNorm, gated residual, GELU-tanh
+MLP, RMSNorm, RoPE tables) lives in the third-party ``diffusers`` package
+(``setup.py:27``, ``diffusers>=0.31``, no upper pin), which is neither under
+``/root/reference`` nor installed; its published algorithm is restated here and
+anchored on the reference's call sites.
+
+Pinning status
+--------------
+The reference holds no tests, golden vectors or fixtures.  Each function is
+therefore pinned by what mathematics and PyTorch's own library routines fix
+(see ``tests/test_oracle_*.py``):
+
+* ``linear``            -- ``torch.nn.functional.linear``, identity / one-hot KATs
+* ``layer_norm``        -- ``F.layer_norm``; zero-mean / unit-variance invariant
+* ``rms_norm``          -- ``F.rms_norm``; scale invariance
+* ``gelu_tanh``         -- ``F.gelu(approximate="tanh")``; values at 0, +-1, large |x|
+* ``silu``              -- ``F.silu``
+* ``attention``         -- ``F.scaled_dot_product_attention`` (math backend), numpy
+                           brute force, rows-sum-to-one, constant-V, KV permutation
+                           invariance, query-row independence
+* ``apply_rotary_emb``  -- complex-multiplication form, norm preservation,
+                           position-0 identity, relative-position property
+* ``flux_rope_table`` / ``cogvideox_rope_table`` -- closed-form angle checks
+* stale KV buffer       -- brute-force concatenation of fresh and stale slices
+* block wiring (``sd3_joint_block``, ``flux_double_block``, ``flux_single_block``,
+  ``cogvideox_block``): the composition order, chunk orders, eps values and
+  which LayerNorm carries affine weights follow the published diffusers
+  modules (``JointTransformerBlock``, ``FluxTransformerBlock``,
+  ``FluxSingleTransformerBlock``, ``CogVideoXBlock``, ``AdaLayerNormZero``,
+  ``AdaLayerNormZeroSingle``, ``AdaLayerNormContinuous``,
+  ``CogVideoXLayerNormZero``).  diffusers cannot be imported here, so this
+  wiring is **parity unpinned** beyond the constraints the reference's call
+  sites fix (joint ordering, return order, split points, argument names) and
+  the adaLN-"Zero" identity property (zero modulation weights => block is the
+  identity on the residual stream).
+"""
+
+from .ops import (  # noqa: F401
+    silu,
+    gelu_tanh,
+    linear,
+    layer_norm,
+    rms_norm,
+    attention,
+    apply_rotary_emb,
+    flux_rope_table,
+    cogvideox_rope_table,
+    adaln_modulation,
+    modulate,
+)
+from .blocks import (  # noqa: F401
+    sd3_joint_block,
+    flux_double_block,
+    flux_single_block,
+    cogvideox_block,
+    feed_forward,
+)
+from .kv_cache import StaleKVBuffer  # noqa: F401

@@ -1,0 +1,184 @@
+"""Parity of every C-ABI kernel with the fp32 oracle on seeded inputs."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from oracle import ops as O
+from tests.util import assert_parity, bf16_round
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def g(x):
+    return x.to(torch.bfloat16).to(DEV)
+
+
+def rnd(*shape, scale=1.0, seed=None):
+    gen = torch.Generator().manual_seed(seed if seed is not None else (hash(shape) & 0xFFFF))
+    return bf16_round(torch.randn(*shape, generator=gen) * scale)
+
+
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (300, 384, 128), (666, 1536, 1536), (1, 128, 64), (1024, 512, 256)])
+def test_gemm_bias(hdit, m, n, k, cfg):
+    print(f"gemm_bias m={m} n={n} k={k} cfg={cfg}", flush=True)
+    hdit._lib.lib().hdit_gemm_force_config(cfg)
+    try:
+        a, w, b = rnd(m, k), rnd(n, k, scale=0.05), rnd(n)
+        out = hdit.ops.linear(g(a), g(w), g(b))
+        torch.cuda.synchronize()
+        assert_parity(out, O.linear(a, w, b), what="gemm bias")
+    finally:
+        hdit._lib.lib().hdit_gemm_force_config(-1)
+
+
+def test_gemm_gelu_and_gate_residual_grouped(hdit):
+    B, T1, T2, D, F = 2, 320, 77, 256, 512
+    x1, x2 = rnd(B, T1, D), rnd(B, T2, D)
+    w1, w2 = rnd(F, D, scale=0.05), rnd(F, D, scale=0.05, seed=5)
+    b1, b2 = rnd(F), rnd(F, seed=6)
+    h1 = torch.empty(B, T1, F, dtype=torch.bfloat16, device=DEV)
+    h2 = torch.empty(B, T2, F, dtype=torch.bfloat16, device=DEV)
+    ops = hdit.ops
+    ops.gemm_launch([
+        ops.gemm_problem(g(x1).view(-1, D), g(w1), h1.view(-1, F), g(b1), ops.EPI_BIAS_GELU),
+        ops.gemm_problem(g(x2).view(-1, D), g(w2), h2.view(-1, F), g(b2), ops.EPI_BIAS_GELU),
+    ])
+    torch.cuda.synchronize()
+    assert_parity(h1, O.gelu_tanh(O.linear(x1, w1, b1)), what="gelu img")
+    assert_parity(h2, O.gelu_tanh(O.linear(x2, w2, b2)), what="gelu txt")
+    # gated residual epilogue (in place on the residual stream)
+    w3, b3 = rnd(D, F, scale=0.05, seed=7), rnd(D, seed=8)
+    gate = torch.randn(B, 3 * D, generator=torch.Generator().manual_seed(9))
+    hh = bf16_round(h1.float().cpu())
+    res = g(x1).clone()
+    gate_dev = gate.to(DEV)
+    ops.gemm_launch([
+        ops.gemm_problem(h1.view(-1, F), g(w3), res.view(-1, D), g(b3), ops.EPI_GATE_RESIDUAL, resid=res.view(-1, D),
+                         gate=gate_dev[:, D:2 * D], rows_per_batch=T1)
+    ])
+    torch.cuda.synchronize()
+    want = x1 + gate[:, None, D:2 * D] * O.linear(hh, w3, b3)
+    assert_parity(res, want, what="gate residual")
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("sq,skv", [(256, 256), (77, 333), (300, 1000), (64, 64), (1, 5)])
+def test_attention_single_segment(hdit, hd, sq, skv):
+    print(f"attention hd={hd} sq={sq} skv={skv}", flush=True)
+    B, H = 2, 3
+    q, k, v = rnd(B, sq, H, hd), rnd(B, skv, H, hd, seed=1), rnd(B, skv, H, hd, seed=2)
+    (o,) = hdit.ops.attention([g(q)], [g(k)], [g(v)])
+    torch.cuda.synchronize()
+    want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
+    assert_parity(o, want, what="attention")
+
+
+def test_attention_two_segments_strided(hdit):
+    """Joint [image, text] sequence living in two buffers; K/V are the halves of
+    a packed K||V buffer (row stride 2*inner), Q patch shorter than K/V."""
+    B, H, hd, n_img, n_txt, n_q = 2, 4, 64, 520, 77, 130
+    inner = H * hd
+    q_img, q_txt = rnd(B, n_q, H, hd, seed=1), rnd(B, n_txt, H, hd, seed=2)
+    kv_img = rnd(B, n_img, 2 * inner, seed=3)
+    kv_txt = rnd(B, n_txt, 2 * inner, seed=4)
+    kvd_img, kvd_txt = g(kv_img), g(kv_txt)
+    k_img = kvd_img[:, :, :inner].unflatten(2, (H, hd))
+    v_img = kvd_img[:, :, inner:].unflatten(2, (H, hd))
+    k_txt = kvd_txt[:, :, :inner].unflatten(2, (H, hd))
+    v_txt = kvd_txt[:, :, inner:].unflatten(2, (H, hd))
+    o_img, o_txt = hdit.ops.attention([g(q_img), g(q_txt)], [k_img, k_txt], [v_img, v_txt])
+    torch.cuda.synchronize()
+    qq = torch.cat([q_img, q_txt], 1).transpose(1, 2)
+    kk = torch.cat([kv_img[..., :inner], kv_txt[..., :inner]], 1).unflatten(2, (H, hd)).transpose(1, 2)
+    vv = torch.cat([kv_img[..., inner:], kv_txt[..., inner:]], 1).unflatten(2, (H, hd)).transpose(1, 2)
+    want = O.attention(qq, kk, vv).transpose(1, 2)
+    assert_parity(o_img, want[:, :n_q], what="attention img")
+    assert_parity(o_txt, want[:, n_q:], what="attention txt")
+
+
+def test_attention_large_logits_and_scale(hdit):
+    B, H, hd, s = 1, 2, 64, 200
+    q, k, v = rnd(B, s, H, hd, scale=6.0, seed=1), rnd(B, s, H, hd, scale=6.0, seed=2), rnd(B, s, H, hd, seed=3)
+    (o,) = hdit.ops.attention([g(q)], [g(k)], [g(v)], scale=0.05)
+    torch.cuda.synchronize()
+    want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), scale=0.05).transpose(1, 2)
+    assert_parity(o, want, what="attention large logits")
+
+
+@pytest.mark.parametrize("dim", [64, 1536, 3072, 4096 + 8])
+def test_layernorm_modulate(hdit, dim):
+    B, T = 2, 37
+    x = rnd(B, T, dim, scale=2.0) + 0.5
+    x = bf16_round(x)
+    mod = torch.randn(B, 6 * dim, generator=torch.Generator().manual_seed(3))
+    md = mod.to(DEV)
+    y = hdit.ops.layernorm_modulate(g(x), md[:, :dim], md[:, dim:2 * dim], eps=1e-6)
+    torch.cuda.synchronize()
+    assert_parity(y, O.modulate(O.layer_norm(x, 1e-6), mod[:, :dim], mod[:, dim:2 * dim]), what="ln modulate")
+    # affine variant without modulation (CogVideoX norm)
+    w, b = rnd(dim, seed=4), rnd(dim, seed=5)
+    y = hdit.ops.layernorm_modulate(g(x), None, None, eps=1e-5, ln_weight=g(w), ln_bias=g(b))
+    torch.cuda.synchronize()
+    assert_parity(y, O.layer_norm(x, 1e-5, w, b), what="ln affine")
+
+
+def test_gate_residual_and_gelu(hdit):
+    B, T, D = 2, 33, 1536
+    x, y = rnd(B, T, D, seed=1), rnd(B, T, D, seed=2)
+    gate = torch.randn(B, D, generator=torch.Generator().manual_seed(3))
+    out = hdit.ops.gate_residual(g(x), g(y), gate.to(DEV))
+    torch.cuda.synchronize()
+    assert_parity(out, x + gate[:, None] * y, what="gate residual")
+    bias = rnd(D, seed=4)
+    out = hdit.ops.gelu_tanh(g(x), g(bias))
+    torch.cuda.synchronize()
+    assert_parity(out, O.gelu_tanh(x + bias), what="gelu")
+
+
+@pytest.mark.parametrize("B,n,k", [(2, 9216, 1536), (1, 18432, 512), (2, 3072, 1536), (5, 100, 64)])
+def test_adaln_gemv(hdit, B, n, k):
+    temb, w, b = rnd(B, k), rnd(n, k, scale=0.02), rnd(n, scale=0.02)
+    out = hdit.ops.adaln_gemv(g(temb), g(w), g(b))
+    torch.cuda.synchronize()
+    want = O.linear(O.silu(temb), w, b)
+    assert_parity(out, want, rel=2e-3, what="adaln gemv")
+
+
+@pytest.mark.parametrize("hd,kind", [(128, 1), (64, 2), (64, 0), (128, 0)])
+def test_qk_norm_rope(hdit, hd, kind):
+    B, S, H, n_txt = 2, 50, 3, 11
+    x = rnd(B, S, H, hd)
+    w, bias = rnd(hd, seed=1) + 1.0, rnd(hd, seed=2)
+    w = bf16_round(w)
+    ids = torch.zeros(S - n_txt, 3)
+    ids[:, 1] = torch.arange(S - n_txt) // 7
+    ids[:, 2] = torch.arange(S - n_txt) % 7
+    axes = (16, 56, 56) if hd == 128 else (16, 24, 24)
+    cos, sin = O.flux_rope_table(ids, axes)
+    xd = g(x)
+    ops = hdit.ops
+    job = ops.qk_norm_rope_job(xd, kind, g(w) if kind else None, g(bias) if kind == 2 else None, cos.to(DEV), sin.to(DEV),
+                               rope_row0=n_txt)
+    ops.qk_norm_rope([job], B, H, hd, eps=1e-6)
+    torch.cuda.synchronize()
+    xh = x.transpose(1, 2)  # [B, H, S, d]
+    if kind == 1:
+        xh = O.rms_norm(xh, 1e-6, w)
+    elif kind == 2:
+        xh = O.layer_norm(xh, 1e-6, w, bias)
+    want = torch.cat([xh[:, :, :n_txt], O.apply_rotary_emb(xh[:, :, n_txt:], cos, sin)], dim=2).transpose(1, 2)
+    assert_parity(xd, want, what="qk norm rope")
+
+
+def test_copy_rows_into_slice(hdit):
+    B, T, D = 2, 16, 128
+    src = rnd(B, T, D)
+    dst = torch.zeros(B, 64, 2 * D, dtype=torch.bfloat16, device=DEV)
+    hdit.ops.copy_rows(g(src), dst[:, 8:24, D:])
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:, 8:24, D:].float().cpu(), src)
+    assert dst[:, :8].abs().sum().item() == 0 and dst[:, :, :D].abs().sum().item() == 0
