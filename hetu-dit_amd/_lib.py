@@ -86,12 +86,12 @@ SIGNATURES = {
     "hdit_layernorm_modulate": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
-         C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_void_p],
+         C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_void_p],
     ),
     "hdit_gate_residual": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64,
-         C.c_int64, C.c_int64, C.c_void_p],
+         C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_void_p],
     ),
     "hdit_adaln_gemv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
     "hdit_gelu_tanh": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_void_p]),

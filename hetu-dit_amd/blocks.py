@@ -1,0 +1,248 @@
+"""The four transformer blocks of the denoise hot path as ``nn.Module``s that
+live in ``transformer.transformer_blocks`` / ``.single_transformer_blocks`` and
+keep the call conventions the reference's transformer wrappers use:
+
+* SD3   ``block(hidden_states=, encoder_hidden_states=, temb=) -> (enc, hid)``
+  (``models/transformers/transformer_sd3.py:136-152``)
+* Flux double, same + ``image_rotary_emb=``   (``transformer_flux.py:160-165``)
+* Flux single ``block(hidden_states=, temb=, image_rotary_emb=) -> hid`` (``:194-198``)
+* CogVideoX ``block(hidden_states=, encoder_hidden_states=, temb=, image_rotary_emb=)
+  -> (hid, enc)``                      (``cogvideox_transformer_3d.py:122-127``)
+
+Sub-module names and parameter paths are those of the diffusers blocks with
+the reference's wrappers applied (``attn.module.to_q``, ``attn.output_bias``,
+``ff.module.net.0.proj``, ``norm1.linear`` ...), which is what the reference's
+weight hot-swap addresses (``hetu_dit/utils.py:561-582``).
+
+Per block the device work is: adaLN projections (weight streaming), fused
+LayerNorm+modulate, ONE grouped GEMM per projection stage covering both
+streams with bias / GELU-tanh / gated-residual epilogues, QK-norm+RoPE in
+place, and the joint flash attention.  Inputs are never modified.
+"""
+from typing import Optional, Tuple
+
+import torch
+from torch import nn
+
+from . import ops
+from .cache_manager import get_cache_manager
+from .layers.attention_processor import _rows2d, hetuDiTAttentionWrapper
+from .layers.feedforward import hetuDiTFeedForwardWrapper
+from .layers.modules import (
+    AdaLayerNormContinuous,
+    AdaLayerNormZero,
+    AdaLayerNormZeroSingle,
+    Attention,
+    CogVideoXAttnProcessor2_0,
+    CogVideoXLayerNormZero,
+    FeedForward,
+    FluxAttnProcessor2_0,
+    JointAttnProcessor2_0,
+)
+from .registry import hetuDiTLayerWrappersRegister
+from .runtime_state import get_runtime_state
+
+
+def _wrap(layer: nn.Module) -> nn.Module:
+    """What ``_wrap_layers`` does for one sub-module
+    (``models/base_model.py:59-112``): registry lookup, construct, and register
+    the layer's KV-cache entry (``:162-178``)."""
+    wrapper = hetuDiTLayerWrappersRegister.get_wrapper(layer)(layer)
+    if isinstance(wrapper, hetuDiTAttentionWrapper):
+        get_cache_manager().register_cache_entry(wrapper.module, layer_type="attn", cache_type="naive_cache")
+    return wrapper
+
+
+def _adaln(norm: nn.Module, temb: torch.Tensor):
+    """f32 [B, chunks*D] = linear(silu(temb)); chunk views."""
+    emb = ops.adaln_gemv(temb.contiguous(), norm.linear.weight.data, norm.linear.bias.data)
+    return emb.chunk(norm.chunks, dim=1)
+
+
+def _mlp_both_streams(ff, x2, resid, gate, ff_c=None, xc2=None, resid_c=None, gate_c=None):
+    """gated-residual MLP of one or two streams: two grouped launches."""
+    p_in, h = ff.in_problem(x2)
+    probs = [p_in]
+    if ff_c is not None:
+        pc_in, hc = ff_c.in_problem(xc2)
+        probs.append(pc_in)
+    ops.gemm_launch(probs)
+    # second residual update is in place on the block's own intermediate tensor
+    probs = [ff.out_problem(h, _rows2d(resid), _rows2d(resid), gate, rows_per_batch=resid.shape[1])]
+    if ff_c is not None:
+        probs.append(ff_c.out_problem(hc, _rows2d(resid_c), _rows2d(resid_c), gate_c, rows_per_batch=resid_c.shape[1]))
+    ops.gemm_launch(probs)
+
+
+class JointTransformerBlock(nn.Module):
+    """SD3 MMDiT joint block (diffusers ``JointTransformerBlock``)."""
+
+    def __init__(self, dim: int, num_attention_heads: int, attention_head_dim: int, context_pre_only: bool = False):
+        super().__init__()
+        self.context_pre_only = context_pre_only
+        self.norm1 = AdaLayerNormZero(dim)
+        self.norm1_context = AdaLayerNormContinuous(dim, dim, eps=1e-6) if context_pre_only else AdaLayerNormZero(dim)
+        self.attn = _wrap(
+            Attention(dim, num_attention_heads, attention_head_dim, added_kv_proj_dim=dim,
+                      context_pre_only=context_pre_only, bias=True, processor=JointAttnProcessor2_0())
+        )
+        self.norm2 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+        self.ff = _wrap(FeedForward(dim))
+        if not context_pre_only:
+            self.norm2_context = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+            self.ff_context = _wrap(FeedForward(dim))
+        else:
+            self.norm2_context = None
+            self.ff_context = None
+
+    @torch.no_grad()
+    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor):
+        eps = 1e-6
+        sh_a, sc_a, g_a, sh_m, sc_m, g_m = _adaln(self.norm1, temb)
+        n = ops.layernorm_modulate(hidden_states, sh_a, sc_a, eps)
+        if self.context_pre_only:
+            c_sc, c_sh = _adaln(self.norm1_context, temb)  # AdaLayerNormContinuous: scale first
+            nc = ops.layernorm_modulate(encoder_hidden_states, c_sh, c_sc, eps)
+            hidden, _ = self.attn.forward_gated(n, nc, hidden_states, g_a)
+        else:
+            c_sh_a, c_sc_a, c_g_a, c_sh_m, c_sc_m, c_g_m = _adaln(self.norm1_context, temb)
+            nc = ops.layernorm_modulate(encoder_hidden_states, c_sh_a, c_sc_a, eps)
+            hidden, encoder = self.attn.forward_gated(n, nc, hidden_states, g_a, encoder_hidden_states, c_g_a)
+        n2 = ops.layernorm_modulate(hidden, sh_m, sc_m, eps)
+        if self.context_pre_only:
+            _mlp_both_streams(self.ff, _rows2d(n2), hidden, g_m)
+            return None, hidden
+        nc2 = ops.layernorm_modulate(encoder, c_sh_m, c_sc_m, eps)
+        _mlp_both_streams(self.ff, _rows2d(n2), hidden, g_m, self.ff_context, _rows2d(nc2), encoder, c_g_m)
+        return encoder, hidden
+
+
+class FluxTransformerBlock(nn.Module):
+    """Flux double-stream block (diffusers ``FluxTransformerBlock``)."""
+
+    def __init__(self, dim: int, num_attention_heads: int, attention_head_dim: int):
+        super().__init__()
+        self.norm1 = AdaLayerNormZero(dim)
+        self.norm1_context = AdaLayerNormZero(dim)
+        self.attn = _wrap(
+            Attention(dim, num_attention_heads, attention_head_dim, added_kv_proj_dim=dim, context_pre_only=False,
+                      bias=True, qk_norm="rms_norm", eps=1e-6, processor=FluxAttnProcessor2_0())
+        )
+        self.norm2 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+        self.ff = _wrap(FeedForward(dim))
+        self.norm2_context = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+        self.ff_context = _wrap(FeedForward(dim))
+
+    @torch.no_grad()
+    def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None):
+        eps = 1e-6
+        sh_a, sc_a, g_a, sh_m, sc_m, g_m = _adaln(self.norm1, temb)
+        c_sh_a, c_sc_a, c_g_a, c_sh_m, c_sc_m, c_g_m = _adaln(self.norm1_context, temb)
+        n = ops.layernorm_modulate(hidden_states, sh_a, sc_a, eps)
+        nc = ops.layernorm_modulate(encoder_hidden_states, c_sh_a, c_sc_a, eps)
+        hidden, encoder = self.attn.forward_gated(n, nc, hidden_states, g_a, encoder_hidden_states, c_g_a,
+                                                  image_rotary_emb=image_rotary_emb)
+        n2 = ops.layernorm_modulate(hidden, sh_m, sc_m, eps)
+        nc2 = ops.layernorm_modulate(encoder, c_sh_m, c_sc_m, eps)
+        _mlp_both_streams(self.ff, _rows2d(n2), hidden, g_m, self.ff_context, _rows2d(nc2), encoder, c_g_m)
+        return encoder, hidden
+
+
+class FluxSingleTransformerBlock(nn.Module):
+    """Flux single-stream block (diffusers ``FluxSingleTransformerBlock``): the
+    q|k|v projection and the MLP-in projection share one launch, attention
+    output and GELU(MLP) are produced side by side in one [B, S, 5D] buffer
+    (no concatenation), ``proj_out`` carries the gated residual."""
+
+    def __init__(self, dim: int, num_attention_heads: int, attention_head_dim: int, mlp_ratio: float = 4.0):
+        super().__init__()
+        self.mlp_hidden_dim = int(dim * mlp_ratio)
+        self.norm = AdaLayerNormZeroSingle(dim)
+        self.proj_mlp = nn.Linear(dim, self.mlp_hidden_dim)
+        self.act_mlp = nn.GELU(approximate="tanh")
+        self.proj_out = nn.Linear(dim + self.mlp_hidden_dim, dim)
+        self.attn = _wrap(
+            Attention(dim, num_attention_heads, attention_head_dim, bias=True, qk_norm="rms_norm", eps=1e-6,
+                      pre_only=True, processor=FluxAttnProcessor2_0())
+        )
+
+    @torch.no_grad()
+    def forward(self, hidden_states, temb, image_rotary_emb=None):
+        B, S, D = hidden_states.shape
+        sh, sc, g = _adaln(self.norm, temb)
+        n = ops.layernorm_modulate(hidden_states, sh, sc, 1e-6)
+        cat = torch.empty(B, S, D + self.mlp_hidden_dim, dtype=torch.bfloat16, device=hidden_states.device)
+        mlp_problem = ops.gemm_problem(_rows2d(n), self.proj_mlp.weight.data, cat.view(-1, cat.shape[-1])[:, D:],
+                                       self.proj_mlp.bias.data, ops.EPI_BIAS_GELU)
+        self.attn.processor(self.attn, n, encoder_hidden_states=None, image_rotary_emb=image_rotary_emb,
+                            out=cat[:, :, :D], extra_problems=[mlp_problem])
+        out = torch.empty_like(hidden_states)
+        ops.gemm_launch([
+            ops.gemm_problem(cat.view(-1, cat.shape[-1]), self.proj_out.weight.data, out.view(-1, D),
+                             self.proj_out.bias.data, ops.EPI_GATE_RESIDUAL, resid=_rows2d(hidden_states), gate=g,
+                             rows_per_batch=S)
+        ])
+        return out
+
+
+class CogVideoXBlock(nn.Module):
+    """CogVideoX block (diffusers ``CogVideoXBlock``): one weight set over the
+    joint [text, video] rows; the two streams differ only in their modulation
+    and gates.  Returns ``(hidden_states, encoder_hidden_states)``."""
+
+    def __init__(self, dim: int, num_attention_heads: int, attention_head_dim: int, time_embed_dim: int = 512):
+        super().__init__()
+        self.norm1 = CogVideoXLayerNormZero(time_embed_dim, dim, eps=1e-5)
+        self.attn1 = _wrap(
+            Attention(dim, num_attention_heads, attention_head_dim, bias=True, out_bias=True, qk_norm="layer_norm",
+                      eps=1e-6, processor=CogVideoXAttnProcessor2_0())
+        )
+        self.norm2 = CogVideoXLayerNormZero(time_embed_dim, dim, eps=1e-5)
+        self.ff = _wrap(FeedForward(dim))
+
+    def _norm_joint(self, norm, hidden, encoder, temb):
+        """Both streams' LayerNorm(affine)+modulate written into one joint
+        [B, n_txt + n_img, D] buffer in [text, video] order."""
+        sh, sc, g, e_sh, e_sc, e_g = _adaln(norm, temb)
+        B, N, D = hidden.shape
+        Nt = encoder.shape[1]
+        joint = torch.empty(B, Nt + N, D, dtype=torch.bfloat16, device=hidden.device)
+        w, b = norm.norm.weight.data, norm.norm.bias.data
+        ops.layernorm_modulate(encoder, e_sh, e_sc, norm.norm.eps, w, b, out=joint[:, :Nt])
+        ops.layernorm_modulate(hidden, sh, sc, norm.norm.eps, w, b, out=joint[:, Nt:])
+        return joint, g, e_g
+
+    @staticmethod
+    def _gated_out_problems(a_joint, weight, bias, hidden, encoder, gate, e_gate, out_h, out_e):
+        """out_stream = stream + gate_stream * (a_joint[rows of stream] @ W^T + b), per batch."""
+        B, N, D = hidden.shape
+        Nt = encoder.shape[1]
+        probs = []
+        for bi in range(B):
+            probs.append(ops.gemm_problem(a_joint[bi, :Nt], weight, out_e[bi], bias, ops.EPI_GATE_RESIDUAL,
+                                          resid=encoder[bi], gate=e_gate[bi:bi + 1], rows_per_batch=Nt))
+            probs.append(ops.gemm_problem(a_joint[bi, Nt:], weight, out_h[bi], bias, ops.EPI_GATE_RESIDUAL,
+                                          resid=hidden[bi], gate=gate[bi:bi + 1], rows_per_batch=N))
+        return probs
+
+    @torch.no_grad()
+    def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None):
+        hidden_states = hidden_states.contiguous()
+        encoder_hidden_states = encoder_hidden_states.contiguous()
+        attn = self.attn1
+        joint, g, e_g = self._norm_joint(self.norm1, hidden_states, encoder_hidden_states, temb)
+        o = attn.processor(attn, hidden_states, encoder_hidden_states, image_rotary_emb=image_rotary_emb,
+                           joint_input=joint)
+        hidden = torch.empty_like(hidden_states)
+        encoder = torch.empty_like(encoder_hidden_states)
+        ops.gemm_launch(self._gated_out_problems(
+            o, attn.module.to_out[0].weight.data, attn.output_bias.data if attn.has_output_bias else None,
+            hidden_states, encoder_hidden_states, g, e_g, hidden, encoder))
+        joint, g, e_g = self._norm_joint(self.norm2, hidden, encoder, temb)
+        p_in, h = self.ff.in_problem(joint.view(-1, joint.shape[-1]))
+        ops.gemm_launch([p_in])
+        h = h.view(joint.shape[0], joint.shape[1], -1)
+        ops.gemm_launch(self._gated_out_problems(
+            h, self.ff.module.net[2].weight.data, self.ff.output_bias.data if self.ff.has_output_bias else None,
+            hidden, encoder, g, e_g, hidden, encoder))
+        return hidden, encoder

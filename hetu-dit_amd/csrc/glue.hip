@@ -19,13 +19,15 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const __bf16* __restri
                                                           const float* __restrict__ scale,
                                                           const __bf16* __restrict__ lw,
                                                           const __bf16* __restrict__ lb, int64_t rows, int tokens,
-                                                          int dim, int64_t ldx, int64_t ldy, int64_t mod_stride,
-                                                          float eps) {
+                                                          int dim, int64_t x_sb, int64_t x_st, int64_t y_sb,
+                                                          int64_t y_st, int64_t mod_stride, float eps) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int nchunks = dim >> 3;
-  const __bf16* xr = x + row * ldx;
+  const int b = (int)(row / tokens);
+  const int64_t t = row - (int64_t)b * tokens;
+  const __bf16* xr = x + b * x_sb + t * x_st;
   i32x4 raw[NCH];
 #pragma unroll
   for (int i = 0; i < NCH; i++) {
@@ -58,10 +60,9 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const __bf16* __restri
     }
   }
   const float rstd = rsqrtf(wave_sum(q) * inv_d + eps);
-  const int b = (int)(row / tokens);
   const float* sh = shift ? shift + (int64_t)b * mod_stride : nullptr;
   const float* sc = scale ? scale + (int64_t)b * mod_stride : nullptr;
-  __bf16* yr = y + row * ldy;
+  __bf16* yr = y + b * y_sb + t * y_st;
 #pragma unroll
   for (int i = 0; i < NCH; i++) {
     int c = lane + i * 64;
@@ -108,16 +109,17 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const __bf16* __restri
 __global__ void __launch_bounds__(256) gate_residual_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ y,
                                                             const float* __restrict__ gate, __bf16* __restrict__ out,
                                                             int64_t total_chunks, int tokens, int chunks_per_row,
-                                                            int64_t ldx, int64_t ldy, int64_t ldo,
-                                                            int64_t gate_stride) {
+                                                            int64_t x_sb, int64_t x_st, int64_t y_sb, int64_t y_st,
+                                                            int64_t o_sb, int64_t o_st, int64_t gate_stride) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total_chunks) return;
   int64_t row = i / chunks_per_row;
   int c = (int)(i - row * chunks_per_row);
   int b = (int)(row / tokens);
+  int64_t t = row - (int64_t)b * tokens;
   float fx[8], fy[8];
-  unpack8(__builtin_nontemporal_load((const i32x4*)(x + row * ldx + c * 8)), fx);
-  unpack8(__builtin_nontemporal_load((const i32x4*)(y + row * ldy + c * 8)), fy);
+  unpack8(__builtin_nontemporal_load((const i32x4*)(x + b * x_sb + t * x_st + c * 8)), fx);
+  unpack8(__builtin_nontemporal_load((const i32x4*)(y + b * y_sb + t * y_st + c * 8)), fy);
   const float* g = gate + (int64_t)b * gate_stride + c * 8;
   f32x4 g0 = *(const f32x4*)g, g1 = *(const f32x4*)(g + 4);
 #pragma unroll
@@ -125,7 +127,7 @@ __global__ void __launch_bounds__(256) gate_residual_kernel(const __bf16* __rest
     fx[e] += g0[e] * fy[e];
     fx[e + 4] += g1[e] * fy[e + 4];
   }
-  __builtin_nontemporal_store(pack8(fx), (i32x4*)(out + row * ldo + c * 8));
+  __builtin_nontemporal_store(pack8(fx), (i32x4*)(out + b * o_sb + t * o_st + c * 8));
 }
 
 // ---------------------------------------------------------------------------
@@ -295,9 +297,10 @@ inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
 extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate(const void* x, void* y, const float* shift, const float* scale,
                                        const void* ln_weight, const void* ln_bias, int batch, int tokens, int dim,
-                                       int64_t ldx, int64_t ldy, int64_t mod_stride, float eps, void* stream) {
+                                       int64_t x_sb, int64_t x_st, int64_t y_sb, int64_t y_st, int64_t mod_stride,
+                                       float eps, void* stream) {
   if (!x || !y || batch < 0 || tokens < 0 || dim <= 0) return HDIT_EINVAL;
-  if (dim % 8 || ldx % 8 || ldy % 8 || mod_stride % 4) return HDIT_EINVAL;
+  if (dim % 8 || x_sb % 8 || x_st % 8 || y_sb % 8 || y_st % 8 || mod_stride % 4) return HDIT_EINVAL;
   if (dim > 8192) return HDIT_EUNSUPPORTED;
   if (!aligned16(x) || !aligned16(y) || !aligned16(shift) || !aligned16(scale) || !aligned16(ln_weight) ||
       !aligned16(ln_bias))
@@ -309,8 +312,8 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate(co
   int nch = (dim / 8 + 63) / 64;
 #define LN_LAUNCH(N)                                                                                             \
   hipLaunchKernelGGL(ln_modulate_kernel<N>, grid, block, 0, s, (const __bf16*)x, (__bf16*)y, shift, scale,      \
-                     (const __bf16*)ln_weight, (const __bf16*)ln_bias, rows, tokens, dim, ldx, ldy, mod_stride, \
-                     eps)
+                     (const __bf16*)ln_weight, (const __bf16*)ln_bias, rows, tokens, dim, x_sb, x_st, y_sb,     \
+                     y_st, mod_stride, eps)
   if (nch <= 1) LN_LAUNCH(1);
   else if (nch <= 2) LN_LAUNCH(2);
   else if (nch <= 3) LN_LAUNCH(3);
@@ -324,16 +327,17 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate(co
 }
 
 extern "C" __attribute__((visibility("default"))) int hdit_gate_residual(const void* x, const void* y, const float* gate, void* out, int batch, int tokens,
-                                  int dim, int64_t ldx, int64_t ldy, int64_t ldo, int64_t gate_stride,
-                                  void* stream) {
+                                  int dim, int64_t x_sb, int64_t x_st, int64_t y_sb, int64_t y_st, int64_t o_sb,
+                                  int64_t o_st, int64_t gate_stride, void* stream) {
   if (!x || !y || !gate || !out || batch < 0 || tokens < 0 || dim <= 0) return HDIT_EINVAL;
-  if (dim % 8 || ldx % 8 || ldy % 8 || ldo % 8 || gate_stride % 4) return HDIT_EINVAL;
+  if (dim % 8 || x_sb % 8 || x_st % 8 || y_sb % 8 || y_st % 8 || o_sb % 8 || o_st % 8 || gate_stride % 4)
+    return HDIT_EINVAL;
   if (!aligned16(x) || !aligned16(y) || !aligned16(out) || !aligned16(gate)) return HDIT_EINVAL;
   int64_t total = (int64_t)batch * tokens * (dim / 8);
   if (total == 0) return HDIT_OK;
   hipLaunchKernelGGL(gate_residual_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const __bf16*)x, (const __bf16*)y, gate, (__bf16*)out, total, tokens, dim / 8, ldx, ldy, ldo,
-                     gate_stride);
+                     (const __bf16*)x, (const __bf16*)y, gate, (__bf16*)out, total, tokens, dim / 8, x_sb, x_st, y_sb,
+                     y_st, o_sb, o_st, gate_stride);
   return hdit_host::check_launch("hdit_gate_residual");
 }
 

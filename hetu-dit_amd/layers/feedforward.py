@@ -1,0 +1,63 @@
+"""FeedForward wrapper with the interface of the reference's
+``layers/feedforward.py:17-78``: wraps ``net = [GELU(proj), Dropout, Linear]``,
+slices ``net[0].proj`` rows / ``net[2]`` columns by tensor-parallel rank, moves
+``net[2].bias`` to ``self.output_bias`` (added after the reduce).  ``forward``
+is two GEMM launches: bias + GELU-tanh fused into the first epilogue, the
+output bias (and optionally the block's gated residual) into the second."""
+import torch
+from torch import nn
+
+from .. import ops
+from ..parallel_state import get_tensor_model_parallel_rank, get_tensor_model_parallel_world_size, get_tp_group
+from ..registry import hetuDiTLayerWrappersRegister
+from .base_layer import hetuDiTDiffusionLayerBaseWrapper
+from .modules import GELU, FeedForward
+
+
+@hetuDiTLayerWrappersRegister.register(FeedForward)
+class hetuDiTFeedForwardWrapper(hetuDiTDiffusionLayerBaseWrapper):
+    def __init__(self, feedforward: FeedForward):
+        super().__init__(module=feedforward)
+        tp_degree = get_tensor_model_parallel_world_size()
+        tp_rank = get_tensor_model_parallel_rank()
+        act = self.module.net[0]
+        if isinstance(act, GELU):
+            act.proj.weight.data = act.proj.weight.data.chunk(tp_degree, dim=0)[tp_rank]
+            if act.proj.bias is not None:
+                act.proj.bias.data = act.proj.bias.data.chunk(tp_degree, dim=0)[tp_rank]
+        else:
+            raise TypeError(f"activation_fn {type(act)} not supported")
+        if getattr(act, "approximate", "tanh") != "tanh":
+            raise TypeError("only GELU(approximate='tanh') is built")
+        self.module.net[2].weight.data = self.module.net[2].weight.chunk(tp_degree, dim=1)[tp_rank]
+        self.has_output_bias = False
+        if self.module.net[2].bias is not None:
+            self.register_parameter("output_bias", nn.Parameter(self.module.net[2].bias.data.clone(), requires_grad=False))
+            self.module.net[2].bias = None
+            self.has_output_bias = True
+
+    # -- problems, so that both streams of a joint block share launches ---------
+    def in_problem(self, x2: torch.Tensor):
+        """x2 [rows, D] -> (problem, h [rows, F]) with bias + GELU-tanh epilogue."""
+        proj = self.module.net[0].proj
+        h = torch.empty(x2.shape[0], proj.weight.shape[0], dtype=torch.bfloat16, device=x2.device)
+        bias = proj.bias.data if proj.bias is not None else None
+        return ops.gemm_problem(x2, proj.weight.data, h, bias, ops.EPI_BIAS_GELU), h
+
+    def out_problem(self, h: torch.Tensor, out2: torch.Tensor, resid2=None, gate=None, rows_per_batch: int = 0):
+        w = self.module.net[2].weight.data
+        bias = self.output_bias.data if self.has_output_bias else None
+        if resid2 is None:
+            return ops.gemm_problem(h, w, out2, bias)
+        return ops.gemm_problem(h, w, out2, bias, ops.EPI_GATE_RESIDUAL, resid=resid2, gate=gate,
+                                rows_per_batch=rows_per_batch)
+
+    def forward(self, hidden_states: torch.Tensor, *args, **kwargs) -> torch.Tensor:
+        x = hidden_states if hidden_states.is_contiguous() else hidden_states.contiguous()
+        x2 = x.view(-1, x.shape[-1])
+        p1, h = self.in_problem(x2)
+        ops.gemm_launch([p1])
+        out = torch.empty(*x.shape[:-1], self.module.net[2].weight.shape[0], dtype=torch.bfloat16, device=x.device)
+        ops.gemm_launch([self.out_problem(h, out.view(-1, out.shape[-1]))])
+        get_tp_group().all_reduce(out)
+        return out

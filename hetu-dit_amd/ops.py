@@ -156,16 +156,15 @@ def attention(q: Sequence[torch.Tensor], k: Sequence[torch.Tensor], v: Sequence[
 # glue
 # ---------------------------------------------------------------------------
 
-def _as3d(x: torch.Tensor, name: str) -> Tuple[int, int, int, int]:
-    """[B, T, D] view whose batch stride equals T * row stride; returns (B, T, D, ld)."""
+def _as3d(x: torch.Tensor, name: str) -> Tuple[int, int, int, int, int]:
+    """[B, T, D] view with unit inner stride; returns (B, T, D, batch stride, token stride)."""
     _need(x, bf16, name)
     if x.dim() != 3 or x.stride(2) != 1:
         raise ValueError(f"{name} must be [batch, tokens, dim] with unit inner stride")
     B, T, D = x.shape
-    ld = x.stride(1) if T > 1 else D
-    if B > 1 and x.stride(0) != T * ld:
-        raise ValueError(f"{name}: batch stride must be tokens * row stride")
-    return B, T, D, ld
+    st = x.stride(1) if T > 1 else D
+    sb = x.stride(0) if B > 1 else T * st
+    return B, T, D, sb, st
 
 
 def _mod(v: Optional[torch.Tensor], B: int, D: int, name: str):
@@ -178,10 +177,12 @@ def _mod(v: Optional[torch.Tensor], B: int, D: int, name: str):
 
 
 def layernorm_modulate(x, shift=None, scale=None, eps: float = 1e-6, ln_weight=None, ln_bias=None, out=None):
-    B, T, D, ldx = _as3d(x, "x")
+    B, T, D, xsb, xst = _as3d(x, "x")
     if out is None:
         out = torch.empty(B, T, D, dtype=bf16, device=x.device)
-    _, _, _, ldy = _as3d(out, "out")
+    Bo, To, Do, ysb, yst = _as3d(out, "out")
+    if (Bo, To, Do) != (B, T, D):
+        raise ValueError("out shape differs from x")
     sh, st1 = _mod(shift, B, D, "shift")
     sc, st2 = _mod(scale, B, D, "scale")
     if sh is not None and sc is not None and st1 != st2:
@@ -191,20 +192,23 @@ def layernorm_modulate(x, shift=None, scale=None, eps: float = 1e-6, ln_weight=N
             _need(w, bf16, "ln affine")
     check(
         _lib.lib().hdit_layernorm_modulate(x.data_ptr(), out.data_ptr(), sh, sc, _ptr(ln_weight), _ptr(ln_bias), B, T, D,
-                                           ldx, ldy, st1 or st2, eps, _stream()),
+                                           xsb, xst, ysb, yst, st1 or st2, eps, _stream()),
         "hdit_layernorm_modulate",
     )
     return out
 
 
 def gate_residual(x, y, gate, out=None):
-    B, T, D, ldx = _as3d(x, "x")
-    _, _, _, ldy = _as3d(y, "y")
+    B, T, D, xsb, xst = _as3d(x, "x")
+    By, Ty, Dy, ysb, yst = _as3d(y, "y")
     if out is None:
         out = torch.empty(B, T, D, dtype=bf16, device=x.device)
-    _, _, _, ldo = _as3d(out, "out")
+    Bo, To, Do, osb, ost = _as3d(out, "out")
+    if (By, Ty, Dy) != (B, T, D) or (Bo, To, Do) != (B, T, D):
+        raise ValueError("gate_residual operand shapes differ")
     g, gs = _mod(gate, B, D, "gate")
-    check(_lib.lib().hdit_gate_residual(x.data_ptr(), y.data_ptr(), g, out.data_ptr(), B, T, D, ldx, ldy, ldo, gs, _stream()),
+    check(_lib.lib().hdit_gate_residual(x.data_ptr(), y.data_ptr(), g, out.data_ptr(), B, T, D, xsb, xst, ysb, yst, osb, ost,
+                                        gs, _stream()),
           "hdit_gate_residual")
     return out
 

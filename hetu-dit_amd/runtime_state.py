@@ -1,0 +1,86 @@
+"""Patch state the hot path consults: the fields of the reference's
+``DiTRuntimeState`` (``hetu_dit/core/distributed/runtime_state.py:97-111``)
+that attention processors, the KV cache and the transformer block loop read,
+with the same names, plus the patch-metadata arithmetic of
+``_calc_patches_metadata`` (``:333-446``) for one sequence-parallel rank."""
+from typing import List, Optional
+
+
+class DiTRuntimeState:
+    def __init__(self):
+        self.patch_mode: bool = False
+        self.pipeline_patch_idx: int = 0
+        self.num_pipeline_patch: int = 1
+        self.pp_patches_height: List[int] = []
+        self.pp_patches_start_idx_local: List[int] = [0]
+        self.pp_patches_token_start_idx_local: List[int] = [0]
+        self.pp_patches_token_num: List[int] = []
+        self.max_condition_sequence_length: int = 0
+        # forced False by the reference (runtime_state.py:188,:225)
+        self.split_text_embed_in_sp: bool = False
+
+    # -- runtime_state.py:254-264 -------------------------------------------
+    def set_patched_mode(self, patch_mode: bool):
+        self.patch_mode = patch_mode
+        self.pipeline_patch_idx = 0
+
+    def next_patch(self):
+        if self.patch_mode:
+            self.pipeline_patch_idx += 1
+            if self.pipeline_patch_idx == self.num_pipeline_patch:
+                self.pipeline_patch_idx = 0
+        else:
+            self.pipeline_patch_idx = 0
+
+    # -- runtime_state.py:333-446 at sequence-parallel degree 1 ---------------
+    def set_patches(self, latents_height: int, latents_width: int, patch_size: int, num_pipeline_patch: int):
+        """Split the latent rows into pipeline patches the way the reference
+        does: equal heights rounded up to a multiple of ``patch_size``, the
+        last patch takes the remainder; token ranges follow from the width."""
+        want = num_pipeline_patch
+        h = (latents_height + want - 1) // want
+        h = (h + patch_size - 1) // patch_size * patch_size
+        n = (latents_height + h - 1) // h
+        heights = [h] * (n - 1)
+        last = latents_height - h * (n - 1)
+        if last % patch_size != 0:
+            raise ValueError(
+                f"The height of the last pipeline patch is {last}, which is not a multiple of patch_size {patch_size}"
+            )
+        heights.append(last)
+        starts = [0]
+        for x in heights:
+            starts.append(starts[-1] + x)
+        per_row = latents_width // patch_size
+        tok = [per_row * (s // patch_size) for s in starts]
+        self.num_pipeline_patch = n
+        self.pp_patches_height = heights
+        self.pp_patches_start_idx_local = starts
+        self.pp_patches_token_start_idx_local = tok
+        self.pp_patches_token_num = [tok[i + 1] - tok[i] for i in range(n)]
+        self.pipeline_patch_idx = 0
+
+    def set_token_patches(self, token_starts: List[int]):
+        """Set the token ranges directly (a shard benchmark has no latent grid)."""
+        self.num_pipeline_patch = len(token_starts) - 1
+        self.pp_patches_token_start_idx_local = list(token_starts)
+        self.pp_patches_token_num = [token_starts[i + 1] - token_starts[i] for i in range(self.num_pipeline_patch)]
+        self.pipeline_patch_idx = 0
+
+
+_RUNTIME: Optional[DiTRuntimeState] = DiTRuntimeState()
+
+
+def get_runtime_state() -> DiTRuntimeState:
+    assert _RUNTIME is not None, "Runtime state has not been initialized."
+    return _RUNTIME
+
+
+def runtime_state_is_initialized() -> bool:
+    return _RUNTIME is not None
+
+
+def reset_runtime_state() -> DiTRuntimeState:
+    global _RUNTIME
+    _RUNTIME = DiTRuntimeState()
+    return _RUNTIME

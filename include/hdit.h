@@ -115,22 +115,23 @@ int hdit_attn_fwd_fp8(const hdit_attn_args* args, const float* absmax, void* str
 
 /* y[b,t,:] = LayerNorm(x[b,t,:]; eps, optional affine ln_weight/ln_bias (bf16))
  *            * (1 + scale[b,:]) + shift[b,:]
- * x, y bf16 [batch, tokens, dim] with row stride ldx / ldy and batch stride
- * tokens*ld; shift/scale f32 with batch stride mod_stride (NULL => 0).
+ * x, y bf16 [batch, tokens, dim]: element (b, t, e) at ptr[b*_sb + t*_st + e]
+ * (so a stream can be read from / written into a slice of a joint buffer);
+ * shift/scale f32 with batch stride mod_stride (NULL => 0).
  * dim % 8 == 0, dim <= 8192.  Replaces diffusers AdaLayerNormZero /
  * AdaLayerNormZeroSingle / AdaLayerNormContinuous / CogVideoXLayerNormZero and
  * the norm2 + modulate of the blocks called at transformer_sd3.py:136-152,
  * transformer_flux.py:160-165,:194-198, cogvideox_transformer_3d.py:122-127. */
 int hdit_layernorm_modulate(const void* x, void* y, const float* shift, const float* scale,
                             const void* ln_weight, const void* ln_bias, int batch, int tokens,
-                            int dim, int64_t ldx, int64_t ldy, int64_t mod_stride, float eps,
-                            void* stream);
+                            int dim, int64_t x_sb, int64_t x_st, int64_t y_sb, int64_t y_st,
+                            int64_t mod_stride, float eps, void* stream);
 
 /* out = x + gate[b,:] * y   (bf16 [batch, tokens, dim], gate f32).  The gated
  * residual of the same blocks when it is not fused into a GEMM epilogue. */
 int hdit_gate_residual(const void* x, const void* y, const float* gate, void* out, int batch,
-                       int tokens, int dim, int64_t ldx, int64_t ldy, int64_t ldo,
-                       int64_t gate_stride, void* stream);
+                       int tokens, int dim, int64_t x_sb, int64_t x_st, int64_t y_sb, int64_t y_st,
+                       int64_t o_sb, int64_t o_st, int64_t gate_stride, void* stream);
 
 /* out[b, :] = W . silu(temb[b, :]) + bias   (W bf16 [n, k], temb bf16 [batch, k],
  * bias bf16 [n] or NULL, out f32 [batch, n]); batch <= 8, k % 8 == 0.

@@ -191,7 +191,10 @@ def flux_attention(
         return o
     o_txt, o_img = o[:, :n_txt], o[:, n_txt:]
     o_img = _lin(p, prefix + ".to_out.0", o_img)
-    o_txt = _lin(p, prefix + ".to_add_out", o_txt)
+    # The wrapper moves to_add_out.bias into `encoder_output_bias`
+    # (attention_processor.py:176-192) and its Flux branch never adds it back
+    # (:284-305): the reference computes the text out-projection WITHOUT bias.
+    o_txt = linear(o_txt, p[prefix + ".to_add_out.weight"], None)
     return o_img, o_txt
 
 

@@ -27,3 +27,20 @@ def bf16_round(x: torch.Tensor) -> torch.Tensor:
     """fp32 values that are exactly representable in bf16 (so the oracle and
     the kernels consume identical inputs)."""
     return x.to(torch.bfloat16).float()
+
+
+def oracle_params(block) -> dict:
+    """fp32 parameter dict in the unwrapped (diffusers) naming the oracle
+    uses, from a product block whose layers carry the reference's wrappers:
+    drop the ``.module`` hop and put the re-homed output biases back under the
+    Linear they came from."""
+    out = {}
+    for name, p in block.named_parameters():
+        key = name.replace(".module.", ".")
+        if key.endswith(".encoder_output_bias"):
+            key = key[: -len("encoder_output_bias")] + "to_add_out.bias"
+        elif key.endswith(".output_bias"):
+            base = key[: -len(".output_bias")]
+            key = base + (".net.2.bias" if base.startswith("ff") else ".to_out.0.bias")
+        out[key] = p.detach().float().cpu()
+    return out
