@@ -1,0 +1,209 @@
+"""Benchmark of the one-GPU DiT denoise-step hot path.
+
+``python bench.py [--gpus 1] [--steps K] [--warmup W]`` times K passes of the
+24-block SD3-shape MMDiT stack (BASELINE.json configs[1]: bf16, batch 2 = CFG
+pair, 4096 image + 333 text tokens, hidden 1536, 24 x 64 heads, last block
+context_pre_only) on synthetic inputs already resident in HBM, and prints one
+JSON line.  ``roofline`` describes the dominant kernel (the grouped MFMA GEMM):
+algorithmic flops per launch / average launch time, measured with HIP events
+on the launch stream in a separate instrumented pass.  ``cpu_baseline`` is the
+fp32 oracle of configs[0] (one SD3 joint block, batch 1, 1024 + 333 tokens)
+timed on this host's cores and extrapolated to 24 blocks.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_HBM_GBS = 8000.0
+
+
+def build_stack(cfg, device, seed=0):
+    import torch
+
+    from hetu_dit_amd import transformer
+
+    with torch.device(device):
+        stack = transformer.SD3TransformerBlocks(cfg["layers"], cfg["dim"], cfg["heads"], cfg["head_dim"])
+    gen = torch.Generator(device=device).manual_seed(seed)
+    for _, p in sorted(stack.named_parameters(), key=lambda kv: kv[0]):
+        p.data = (torch.randn(p.shape, generator=gen, device=device) * 0.02).to(torch.bfloat16)
+        p.requires_grad_(False)
+    return stack
+
+
+def algorithmic_flops(cfg):
+    B, Ni, Nt, D = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"]
+    S = Ni + Nt
+    gemm = 24.0 * S * D * D * B * cfg["layers"] - 18.0 * Nt * D * D * B  # last block: text stream stops after q|k|v
+    attn = 4.0 * S * S * D * B * cfg["layers"]
+    return gemm, attn
+
+
+def cpu_baseline(runs=3):
+    """fp32 oracle of configs[0] on the host cores (a reported baseline, not a target)."""
+    import torch
+
+    import oracle
+    from hetu_dit_amd import blocks, synthetic
+    from tests.util import oracle_params
+
+    cfg = synthetic.CONFIGS["sd3_512"]
+    torch.set_num_threads(os.cpu_count() or 1)
+    blk = blocks.JointTransformerBlock(cfg["dim"], cfg["heads"], cfg["head_dim"])
+    synthetic.init_module_(blk, 100)
+    params = oracle_params(blk)
+    x = synthetic.randn_bf16((cfg["batch"], cfg["n_img"], cfg["dim"]), 101).float()
+    e = synthetic.randn_bf16((cfg["batch"], cfg["n_txt"], cfg["dim"]), 102).float()
+    t = synthetic.randn_bf16((cfg["batch"], cfg["dim"]), 103).float()
+    oracle.sd3_joint_block(params, x, e, t, cfg["heads"])  # warm-up
+    times = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        oracle.sd3_joint_block(params, x, e, t, cfg["heads"])
+        times.append((time.perf_counter() - t0) * 1e3)
+    ms_block = statistics.median(times)
+    return {
+        "value": round(ms_block * 24, 2),
+        "unit": "ms",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"fp32 oracle, configs[0] SD3 joint block (B1, 1024+333 tokens, D1536): median of {runs} runs = "
+                  f"{ms_block:.1f} ms/block, value = 24 x block (extrapolated step, no CFG pair); os.cpu_count()="
+                  f"{os.cpu_count()}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the one-GPU hot path only: run with --gpus 1 "
+              "(every box of this build has one GPU; how the path shards is described in DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import hetu_dit_amd  # noqa: F401  (raises if libhdit.so is missing)
+    from hetu_dit_amd import ops, synthetic
+    from hetu_dit_amd.runtime_state import reset_runtime_state
+
+    hetu_dit_amd._lib.lib()
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    cfg = synthetic.CONFIGS["sd3_1024"]
+    reset_runtime_state()
+    stack = build_stack(cfg, dev)
+    B, Ni, Nt, D = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"]
+    gen = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(B, Ni, D, generator=gen, device=dev).to(torch.bfloat16)
+    e = torch.randn(B, Nt, D, generator=gen, device=dev).to(torch.bfloat16)
+    t = torch.randn(B, D, generator=gen, device=dev).to(torch.bfloat16)
+
+    def step():
+        return stack(x, e, t)
+
+    for _ in range(max(args.warmup, 1)):
+        out = step()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+
+    use_graph = not args.no_graph
+    if use_graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            g_out = step()
+        graph.replay()
+        torch.cuda.synchronize()
+        # a replay must reproduce the eager result bit for bit (same kernels, same inputs)
+        if not torch.equal(g_out, out):
+            use_graph = False
+        run = graph.replay if use_graph else step
+    else:
+        run = step
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # instrumented eager pass: HIP events around every launch on the launch stream
+    timer = ops.KernelTimer()
+    ops.set_timer(timer)
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    ops.set_timer(None)
+    summ = timer.summary()
+
+    def per_class(kind):
+        n, ms, work = summ.get(kind, (0, 0.0, 0.0))
+        return n, ms, work
+
+    n_g, ms_g, fl_g = per_class("gemm")
+    n_a, ms_a, fl_a = per_class("attn_bf16")
+    gemm_tflops = fl_g / ms_g / 1e9 if ms_g else 0.0
+    attn_tflops = fl_a / ms_a / 1e9 if ms_a else 0.0
+    glue = {}
+    for kind in ("ln_modulate", "adaln_gemv", "gate_residual", "qk_norm_rope"):
+        n, ms, nbytes = per_class(kind)
+        if n:
+            glue[kind] = {"launches_per_step": n // 3, "avg_us": round(ms / n * 1e3, 2),
+                          "achieved_GBps": round(nbytes / ms / 1e6, 1), "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    gemm_fl, attn_fl = algorithmic_flops(cfg)
+    result = {
+        "metric": "ms per DiT denoise step (1 GPU)",
+        "value": round(ms_step, 3),
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 3),
+        "ms_per_block": round(ms_step / cfg["layers"], 4),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic (seeded N(0,1) activations, N(0,0.02) random-init weights, resident in HBM)",
+        "config": {"workload": "configs[1]: SD3-shape denoise step, 24 joint blocks, B2 (CFG pair), 4096 image + 333 text "
+                               "tokens, D1536, 24x64 heads, last block context_pre_only",
+                   "launch": "hip-graph replay" if use_graph else "eager"},
+        "step_tflops": round((gemm_fl + attn_fl) / ms_step / 1e9, 1),
+        "roofline": {
+            "kernel": "gemm_kernel (grouped bf16 MFMA GEMM, all projection/MLP launches of the step)",
+            "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+            "launches_per_step": n_g // 3, "avg_launch_us": round(ms_g / max(n_g, 1) * 1e3, 2),
+            "flops_per_launch": round(fl_g / max(n_g, 1), 1),
+        },
+        "roofline_attention": {
+            "kernel": "attn_fwd_kernel<64> (joint flash attention)", "bound": "mfma", "achieved": round(attn_tflops, 1),
+            "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
+            "launches_per_step": n_a // 3, "avg_launch_us": round(ms_a / max(n_a, 1) * 1e3, 2),
+            "flops_per_launch": round(fl_a / max(n_a, 1), 1),
+        },
+        "roofline_glue": glue,
+        "reference_prior": {"ms_per_step": 242.7, "note": "hetu_dit/model_profiler.py:116-121, SD3 1024^2 1 GPU, "
+                                                            "hardware unlabelled (README testbed NVIDIA L20); not the same hardware"},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

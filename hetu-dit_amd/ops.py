@@ -20,6 +20,45 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+class KernelTimer:
+    """Optional per-launch HIP-event timing on the launch stream.  When a timer
+    is installed (``set_timer``) every C-ABI launch is bracketed by a pair of
+    events on PyTorch's current stream -- the stream the kernel runs on -- and
+    logged as (kernel class, algorithmic work, events).  ``work`` is flops for
+    the MFMA kernels and bytes for the bandwidth-bound ones."""
+
+    def __init__(self):
+        self.records = []
+
+    def summary(self):
+        """class -> (launches, total ms, total work)"""
+        out = {}
+        for kind, work, e0, e1 in self.records:
+            n, ms, w = out.get(kind, (0, 0.0, 0.0))
+            out[kind] = (n + 1, ms + e0.elapsed_time(e1), w + work)
+        return out
+
+
+_TIMER: Optional[KernelTimer] = None
+
+
+def set_timer(timer: Optional[KernelTimer]):
+    global _TIMER
+    _TIMER = timer
+
+
+def _run(kind: str, work: float, call):
+    t = _TIMER
+    if t is None:
+        return call()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    rc = call()
+    e1.record()
+    t.records.append((kind, work, e0, e1))
+    return rc
+
+
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
@@ -84,7 +123,8 @@ def gemm_problem(
 def gemm_launch(problems: Sequence[GemmProblem]):
     n = len(problems)
     arr = (GemmProblem * n)(*problems)
-    check(_lib.lib().hdit_gemm_bf16(arr, n, _stream()), "hdit_gemm_bf16")
+    flops = sum(2.0 * p.m * p.n * p.k for p in problems) if _TIMER is not None else 0.0
+    check(_run("gemm", flops, lambda: _lib.lib().hdit_gemm_bf16(arr, n, _stream())), "hdit_gemm_bf16")
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, gelu: bool = False,
@@ -143,12 +183,17 @@ def attention(q: Sequence[torch.Tensor], k: Sequence[torch.Tensor], v: Sequence[
         out = [torch.empty(t.shape, dtype=bf16, device=t.device) for t in q]
     args = attention_args(q, k, v, out, scale)
     lib = _lib.lib()
+    sq, skv = sum(t.shape[1] for t in q), sum(t.shape[1] for t in k)
+    flops = 4.0 * args.batch * args.heads * sq * skv * args.head_dim
     if fp8:
         absmax = torch.empty(3, args.batch, args.heads, dtype=torch.float32, device=q[0].device)
-        check(lib.hdit_attn_absmax(C.byref(args), absmax.data_ptr(), _stream()), "hdit_attn_absmax")
-        check(lib.hdit_attn_fwd_fp8(C.byref(args), absmax.data_ptr(), _stream()), "hdit_attn_fwd_fp8")
+        nbytes = 2.0 * args.batch * args.heads * args.head_dim * (sq + 2 * skv)
+        check(_run("attn_absmax", nbytes, lambda: lib.hdit_attn_absmax(C.byref(args), absmax.data_ptr(), _stream())),
+              "hdit_attn_absmax")
+        check(_run("attn_fp8", flops, lambda: lib.hdit_attn_fwd_fp8(C.byref(args), absmax.data_ptr(), _stream())),
+              "hdit_attn_fwd_fp8")
     else:
-        check(lib.hdit_attn_fwd_bf16(C.byref(args), _stream()), "hdit_attn_fwd_bf16")
+        check(_run("attn_bf16", flops, lambda: lib.hdit_attn_fwd_bf16(C.byref(args), _stream())), "hdit_attn_fwd_bf16")
     return list(out)
 
 
@@ -191,8 +236,10 @@ def layernorm_modulate(x, shift=None, scale=None, eps: float = 1e-6, ln_weight=N
         if w is not None:
             _need(w, bf16, "ln affine")
     check(
-        _lib.lib().hdit_layernorm_modulate(x.data_ptr(), out.data_ptr(), sh, sc, _ptr(ln_weight), _ptr(ln_bias), B, T, D,
-                                           xsb, xst, ysb, yst, st1 or st2, eps, _stream()),
+        _run("ln_modulate", 4.0 * B * T * D,
+             lambda: _lib.lib().hdit_layernorm_modulate(x.data_ptr(), out.data_ptr(), sh, sc, _ptr(ln_weight),
+                                                        _ptr(ln_bias), B, T, D, xsb, xst, ysb, yst, st1 or st2, eps,
+                                                        _stream())),
         "hdit_layernorm_modulate",
     )
     return out
@@ -207,8 +254,9 @@ def gate_residual(x, y, gate, out=None):
     if (By, Ty, Dy) != (B, T, D) or (Bo, To, Do) != (B, T, D):
         raise ValueError("gate_residual operand shapes differ")
     g, gs = _mod(gate, B, D, "gate")
-    check(_lib.lib().hdit_gate_residual(x.data_ptr(), y.data_ptr(), g, out.data_ptr(), B, T, D, xsb, xst, ysb, yst, osb, ost,
-                                        gs, _stream()),
+    check(_run("gate_residual", 6.0 * B * T * D,
+               lambda: _lib.lib().hdit_gate_residual(x.data_ptr(), y.data_ptr(), g, out.data_ptr(), B, T, D, xsb, xst, ysb,
+                                                     yst, osb, ost, gs, _stream())),
           "hdit_gate_residual")
     return out
 
@@ -223,7 +271,9 @@ def adaln_gemv(temb: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
     if bias is not None:
         _need(bias, bf16, "bias")
     out = torch.empty(B, n, dtype=torch.float32, device=temb.device)
-    check(_lib.lib().hdit_adaln_gemv(temb.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), B, n, k, _stream()),
+    check(_run("adaln_gemv", 2.0 * n * k,
+               lambda: _lib.lib().hdit_adaln_gemv(temb.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), B, n, k,
+                                                  _stream())),
           "hdit_adaln_gemv")
     return out
 
@@ -272,7 +322,10 @@ def qk_norm_rope_job(x: torch.Tensor, norm_kind: int = 0, weight=None, bias=None
 
 def qk_norm_rope(jobs: List[QkNormJob], batch: int, heads: int, head_dim: int, eps: float = 1e-6):
     arr = (QkNormJob * len(jobs))(*jobs)
-    check(_lib.lib().hdit_qk_norm_rope(arr, len(jobs), batch, heads, head_dim, eps, _stream()), "hdit_qk_norm_rope")
+    nbytes = sum(4.0 * batch * j.seq * heads * head_dim for j in jobs)
+    check(_run("qk_norm_rope", nbytes,
+               lambda: _lib.lib().hdit_qk_norm_rope(arr, len(jobs), batch, heads, head_dim, eps, _stream())),
+          "hdit_qk_norm_rope")
 
 
 def copy_rows(src: torch.Tensor, dst: torch.Tensor):
