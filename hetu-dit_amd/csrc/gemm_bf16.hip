@@ -1,22 +1,36 @@
 // Grouped bf16 GEMM for gfx950:  C[m, n] = epilogue(A[m, k] . B[n, k]^T + bias)
 //
-// Persistent kernel: one 512-thread workgroup per CU walks a static list of
-// 256x256 (or smaller) output tiles.  Both operands are k-contiguous, so A and
-// B tiles are staged the same way: `global_load_lds_dwordx4` copies 64-wide k
-// slabs straight from global memory into LDS (no VGPR staging, no ds_write),
-// two LDS stages, one barrier per slab.  A wave-wide direct load writes 1 KiB
-// of LDS in lane order, i.e. 8 rows x 128 bytes; the XOR swizzle that keeps
-// the later ds_read_b128 fragment reads conflict-free is applied on the global
-// side (lane l fetches 16-byte chunk (l%8)^(l/8) of row l/8), which stays
-// inside one 128-byte line, so the global access remains fully coalesced.
-// The first slab of the NEXT tile is requested before the epilogue of the
-// current one, so tile prologues are hidden behind stores.
+// Persistent kernel, one 256-thread workgroup (2x2 waves) per CU, walking a
+// static list of output tiles of (64*TM) x (64*TN) elements; a wave owns a
+// (32*TM) x (32*TN) sub-tile in accumulators (v_mfma_f32_32x32x16_bf16).
 //
-// MFMA mapping: v_mfma_f32_32x32x16_bf16 with the weight fragment as "A" (rows
-// = n) and the activation fragment as "B" (columns = m): a lane's accumulator
-// holds one output row m and runs of 4 consecutive n.  Lanes l and l^32 swap
-// halves (v_permlane32_swap) so that each lane stores 16 contiguous bytes; the
-// epilogue fuses bias, GELU-tanh or the gated residual.
+// Staging.  Both operands are k-contiguous, so A and B tiles are staged the
+// same way: `global_load_lds_dwordx4` copies 64-wide k slabs straight from
+// global memory into LDS (no VGPR staging, no ds_write).  A wave-wide direct
+// load writes 1 KiB of LDS in lane order = 8 rows x 128 bytes.  The XOR swizzle
+// that keeps the ds_read_b128 fragment reads conflict-free is applied on the
+// global side: the lane that fills 16-byte slot p of row r fetches chunk
+// p ^ ((r>>1)&7) of that row, which stays inside one 128-byte line, so the
+// global access remains fully coalesced.  Swizzling by (r>>1)&7 makes the 16
+// rows one ds_read_b128 pass touches land on 16 distinct 16-byte slots of the
+// 256-byte LDS bank window (measured 202 B/clk/CU, against 117 B/clk for r&7).
+//
+// Pipeline.  The k slabs of all tiles of a workgroup form one flat stream with
+// two LDS stages.  While slab g is multiplied, slab g+1 is in flight; in the
+// last k-step of slab g every wave waits for its own copies, the workgroup
+// barrier makes slab g+1 visible and proves stage(g) free, the first
+// fragments of slab g+1 are read and the copy of slab g+2 is issued -- all
+// under the remaining MFMAs of slab g.  Fragments are double-buffered in
+// registers one k-step ahead.  Tile boundaries are invisible to the stream, so
+// a tile's first slabs arrive during the previous tile's last slab and
+// epilogue.
+//
+// Epilogue.  A lane's accumulator holds one output row m and runs of 4
+// consecutive n; lanes l and l^32 swap halves (v_permlane32_swap) to own 8
+// consecutive n.  bias / GELU-tanh / gate are applied there, the bf16 result is
+// staged through a wave-private 8 KiB LDS window and written back with 16
+// lanes covering 256 contiguous bytes of a row (the residual is read in that
+// same coalesced layout and added in fp32 before the final rounding).
 //
 // One launch covers up to HDIT_GEMM_MAX_PROBLEMS problems.  Tiles are dealt to
 // workgroups so that the workgroups of one XCD (workgroup id mod 8; each XCD
@@ -29,6 +43,9 @@ constexpr int BK = 64;          // k elements per LDS stage
 constexpr int ROW_BYTES = 128;  // BK * sizeof(bf16)
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 8;
+constexpr int NW = 4;
+constexpr int NT = 256;
+constexpr int EPI_WAVE_BYTES = 8192;  // 32 rows x 128 columns of bf16
 
 struct GemmTable {
   int count;
@@ -36,19 +53,18 @@ struct GemmTable {
   hdit_gemm_problem p[HDIT_GEMM_MAX_PROBLEMS];
 };
 
-template <int BM_, int BN_, int WGM_, int WGN_>
+template <int TM_, int TN_>
 struct Cfg {
-  static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
-  static constexpr int NW = WGM * WGN;
-  static constexpr int NT = NW * 64;
-  static constexpr int WM = BM / WGM, WN = BN / WGN;
-  static constexpr int TM = WM / 32, TN = WN / 32;
-  static constexpr int A_LOADS = BM / 8 / NW;  // direct-to-LDS wave loads per wave per stage (8 rows each)
+  static constexpr int TM = TM_, TN = TN_;
+  static constexpr int BM = 64 * TM, BN = 64 * TN;
+  static constexpr int WM = 32 * TM, WN = 32 * TN;
+  static constexpr int A_LOADS = BM / 8 / NW;  // direct-to-LDS wave loads per wave per slab (8 rows each)
   static constexpr int B_LOADS = BN / 8 / NW;
   static constexpr int A_BYTES = BM * ROW_BYTES;
   static constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
-  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/waves mismatch");
+  static constexpr int EPI_OFF = 2 * STAGE_BYTES;
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES + NW * EPI_WAVE_BYTES;
+  static_assert(TN <= 4, "epilogue staging window is 128 columns wide");
 };
 
 struct TileCoord {
@@ -78,109 +94,160 @@ __device__ __forceinline__ void lds_dma16(const void* gptr, unsigned char* lds_d
                                    (void __attribute__((address_space(3)))*)lds_dst_uniform, 16, 0, 0);
 }
 
+#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
 template <class C>
-__global__ void __launch_bounds__(C::NT) gemm_kernel(const GemmTable tab, int total_tiles, int tiles_per_xcd,
-                                                      int wgs_per_xcd) {
+__global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total_tiles, int tiles_per_xcd,
+                                                  int wgs_per_xcd) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  constexpr int TM = C::TM, TN = C::TN;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, lh = lane >> 5;
-  const int wm0 = (wave / C::WGN) * C::WM;
-  const int wn0 = (wave % C::WGN) * C::WN;
+  const int wm0 = (wave >> 1) * C::WM;
+  const int wn0 = (wave & 1) * C::WN;
 
   // tiles of this workgroup: XCD x owns logical tiles [x*tiles_per_xcd, (x+1)*tiles_per_xcd),
   // dealt round-robin to that XCD's workgroups
   const int xcd = blockIdx.x % NUM_XCD;
-  const int wg_in_xcd = blockIdx.x / NUM_XCD;
   const int xcd_begin = xcd * tiles_per_xcd;
   const int xcd_end = min(xcd_begin + tiles_per_xcd, total_tiles);
+  int lid = xcd_begin + blockIdx.x / NUM_XCD;
+  if (lid >= xcd_end) return;
 
-  // lane-constant parts of the direct-to-LDS copy: row-in-group l/8, swizzled chunk
+  // ---- producer: the slab stream, two slabs ahead of the MFMAs ---------------
+  // Lane-constant parts of a direct-to-LDS copy: row-in-group l/8; the chunk a lane fetches is
+  // (l%8) ^ ((row>>1)&7) with row = 8*grp + l/8 and grp = wave + 4*i, whose parity is that of `wave`.
   const int ld_row = lane >> 3;
-  const int ld_chunk = (lane & 7) ^ ld_row;
-
-  auto issue_stage = [&](const TileCoord& tc, int kt, int stage) {
+  const int ld_chunk = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+  int p_lid = lid;
+  bool p_valid = true;
+  int p_kt = 0, p_KT = 0;
+  const unsigned char* p_abase = nullptr;
+  const unsigned char* p_bbase = nullptr;
+  unsigned p_aoff[C::A_LOADS], p_boff[C::B_LOADS];
+  auto p_setup = [&]() {
+    const TileCoord tc = locate<C>(tab, p_lid);
     const hdit_gemm_problem& pr = tab.p[tc.pi];
-    const __bf16* A = (const __bf16*)pr.a;
-    const __bf16* B = (const __bf16*)pr.b;
-    unsigned char* base = lds + stage * C::STAGE_BYTES;
+    p_abase = (const unsigned char*)pr.a;
+    p_bbase = (const unsigned char*)pr.b;
+    p_KT = pr.k / BK;
+    p_kt = 0;
 #pragma unroll
     for (int i = 0; i < C::A_LOADS; i++) {
-      const int grp = wave + i * C::NW;  // 8-row group inside the tile
-      const int gr = min(tc.m0 + grp * 8 + ld_row, pr.m - 1);
-      lds_dma16(A + (int64_t)gr * pr.lda + kt * BK + ld_chunk * 8, base + grp * 1024);
+      const int gr = min(tc.m0 + (wave + i * NW) * 8 + ld_row, pr.m - 1);
+      p_aoff[i] = (unsigned)(((int64_t)gr * pr.lda + ld_chunk * 8) * 2);
     }
 #pragma unroll
     for (int i = 0; i < C::B_LOADS; i++) {
-      const int grp = wave + i * C::NW;
-      const int gr = min(tc.n0 + grp * 8 + ld_row, pr.n - 1);
-      lds_dma16(B + (int64_t)gr * pr.ldb + kt * BK + ld_chunk * 8, base + C::A_BYTES + grp * 1024);
+      const int gr = min(tc.n0 + (wave + i * NW) * 8 + ld_row, pr.n - 1);
+      p_boff[i] = (unsigned)(((int64_t)gr * pr.ldb + ld_chunk * 8) * 2);
+    }
+  };
+  auto p_issue = [&](int stage) {
+    if (!p_valid) return;
+    unsigned char* base = lds + stage * C::STAGE_BYTES + wave * 1024;
+    const unsigned char* ak = p_abase + (size_t)p_kt * ROW_BYTES;
+    const unsigned char* bk = p_bbase + (size_t)p_kt * ROW_BYTES;
+#pragma unroll
+    for (int i = 0; i < C::A_LOADS; i++) lds_dma16(ak + p_aoff[i], base + i * NW * 1024);
+#pragma unroll
+    for (int i = 0; i < C::B_LOADS; i++) lds_dma16(bk + p_boff[i], base + C::A_BYTES + i * NW * 1024);
+    if (++p_kt == p_KT) {
+      p_lid += wgs_per_xcd;
+      p_valid = p_lid < xcd_end;
+      if (p_valid) p_setup();
     }
   };
 
-  // fragment read offsets: row r, logical chunk c -> r*128 + ((c ^ (r&7)) << 4); r&7 == l32&7 for every fragment
-  const int swz = l32 & 7;
+  // ---- consumer ------------------------------------------------------------
+  // fragment read offsets: row r, logical chunk c -> r*128 + ((c ^ ((r>>1)&7)) << 4); fragment rows are
+  // l32 plus a multiple of 32, so (r>>1)&7 == (l32>>1)&7
+  const int swz = (l32 >> 1) & 7;
   int a_off[4], b_off[4];  // per k-step (chunk = 2*ks + lh)
 #pragma unroll
   for (int ks = 0; ks < 4; ks++) {
     a_off[ks] = (wm0 + l32) * ROW_BYTES + (((ks * 2 + lh) ^ swz) << 4);
     b_off[ks] = C::A_BYTES + (wn0 + l32) * ROW_BYTES + (((ks * 2 + lh) ^ swz) << 4);
   }
+  bf16x8 fa[2][TM], fb[2][TN];
+  auto read_frags = [&](const unsigned char* sbase, int ks, int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa[buf][i] = *(const bf16x8*)(sbase + a_off[ks] + i * 32 * ROW_BYTES);
+#pragma unroll
+    for (int j = 0; j < TN; j++) fb[buf][j] = *(const bf16x8*)(sbase + b_off[ks] + j * 32 * ROW_BYTES);
+  };
 
-  int lid = xcd_begin + wg_in_xcd;
-  if (lid >= xcd_end) return;
-  TileCoord tc = locate<C>(tab, lid);
-  int stage = 0;
-  issue_stage(tc, 0, stage);
+  p_setup();
+  p_issue(0);
+  p_issue(1);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
+  int stage = 0;
+  read_frags(lds, 0, 0);
+
+  // wave-private epilogue staging window
+  unsigned char* epi = lds + C::EPI_OFF + wave * EPI_WAVE_BYTES;
 
   while (true) {
+    const TileCoord tc = locate<C>(tab, lid);
     const hdit_gemm_problem& pr = tab.p[tc.pi];
     const int KT = pr.k / BK;
-    const int next_lid = lid + wgs_per_xcd;
-    const bool has_next = next_lid < xcd_end;
-    TileCoord ntc = tc;
-    if (has_next) ntc = locate<C>(tab, next_lid);
 
-    f32x16 acc[C::TM][C::TN];
+    f32x16 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < C::TM; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int j = 0; j < C::TN; j++)
+      for (int j = 0; j < TN; j++)
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
     for (int kt = 0; kt < KT; kt++) {
-      // request the next slab (or the next tile's first slab) into the other stage
-      if (kt + 1 < KT) issue_stage(tc, kt + 1, stage ^ 1);
-      else if (has_next) issue_stage(ntc, 0, stage ^ 1);
-
       const unsigned char* sbase = lds + stage * C::STAGE_BYTES;
-      bf16x8 fa[2][C::TM], fb[2][C::TN];
 #pragma unroll
-      for (int i = 0; i < C::TM; i++) fa[0][i] = *(const bf16x8*)(sbase + a_off[0] + i * 32 * ROW_BYTES);
+      for (int ks = 0; ks < 3; ks++) {
+        const int cur = ks & 1;
+        read_frags(sbase, ks + 1, cur ^ 1);
 #pragma unroll
-      for (int j = 0; j < C::TN; j++) fb[0][j] = *(const bf16x8*)(sbase + b_off[0] + j * 32 * ROW_BYTES);
+        for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) {
-        const int cur = ks & 1, nxt = cur ^ 1;
-        if (ks + 1 < 4) {
-#pragma unroll
-          for (int i = 0; i < C::TM; i++) fa[nxt][i] = *(const bf16x8*)(sbase + a_off[ks + 1] + i * 32 * ROW_BYTES);
-#pragma unroll
-          for (int j = 0; j < C::TN; j++) fb[nxt][j] = *(const bf16x8*)(sbase + b_off[ks + 1] + j * 32 * ROW_BYTES);
-        }
-#pragma unroll
-        for (int i = 0; i < C::TM; i++)
-#pragma unroll
-          for (int j = 0; j < C::TN; j++)
+          for (int j = 0; j < TN; j++)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+        // issue order inside this k-step: one fragment read per MFMA until the next step's fragments are
+        // requested, then the remaining MFMAs (the reads get a full k-step to land)
+        // (an MFMA goes first, so that the wait for THIS step's fragments is placed while no younger
+        // read is outstanding and costs nothing)
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        constexpr int PAIRS = (TM + TN < TM * TN - 1) ? TM + TN : TM * TN - 1;
+#pragma unroll
+        for (int t = 0; t < PAIRS; t++) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        }
+        if (TM + TN - PAIRS > 0) __builtin_amdgcn_sched_group_barrier(0x100, TM + TN - PAIRS, 0);
+        if (TM * TN - 1 - PAIRS > 0) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1 - PAIRS, 0);
+        SCHED_FENCE();
       }
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's direct-to-LDS copies have landed
+      // last k-step (fragment buffer 1): first half of the MFMAs, then turn the stages over
+#pragma unroll
+      for (int i = 0; i < TM / 2; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+      SCHED_FENCE();
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my copies landed, my reads of this stage are done
       __syncthreads();
       stage ^= 1;
+      read_frags(lds + stage * C::STAGE_BYTES, 0, 0);
+      p_issue(stage ^ 1);
+      SCHED_FENCE();
+#pragma unroll
+      for (int i = TM / 2; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+      SCHED_FENCE();
     }
 
     // ---- epilogue ---------------------------------------------------------
@@ -188,20 +255,22 @@ __global__ void __launch_bounds__(C::NT) gemm_kernel(const GemmTable tab, int to
     const __bf16* __restrict__ bias = (const __bf16*)pr.bias;
     const __bf16* __restrict__ resid = (const __bf16*)pr.resid;
     const float* __restrict__ gate = pr.gate;
-    const int epi = pr.epilogue;
+    const int epi_mode = pr.epilogue;
     const int M = pr.m, N = pr.n;
     const int64_t ldc = pr.ldc, ldr = pr.ldr;
+    const int ncol0 = tc.n0 + wn0;
 #pragma unroll
-    for (int i = 0; i < C::TM; i++) {
-      const int m = tc.m0 + wm0 + i * 32 + l32;
+    for (int i = 0; i < TM; i++) {
+      const int mrow0 = tc.m0 + wm0 + i * 32;
+      const int m = mrow0 + l32;
       const float* grow = nullptr;
-      if (epi == HDIT_EPI_GATE_RESIDUAL) grow = gate + (int64_t)(min(m, M - 1) / pr.rows_per_batch) * pr.gate_stride;
+      if (epi_mode == HDIT_EPI_GATE_RESIDUAL) grow = gate + (int64_t)(min(m, M - 1) / pr.rows_per_batch) * pr.gate_stride;
 #pragma unroll
-      for (int j = 0; j < C::TN; j++) {
+      for (int j = 0; j < TN; j++) {
 #pragma unroll
         for (int gp = 0; gp < 2; gp++) {
-          // accumulator groups g = 2gp (even) and 2gp+1 (odd): columns 8g + 4*lh + e.  After the swap
-          // lanes < 32 hold the 8 columns of the even group, lanes >= 32 those of the odd group.
+          // accumulator groups g = 2gp (even) and 2gp+1 (odd) hold columns 8g + 4*lh + e.  After the swap
+          // lanes < 32 own the 8 columns of the even group, lanes >= 32 those of the odd group.
           float v[8];
 #pragma unroll
           for (int e = 0; e < 4; e++) {
@@ -210,35 +279,52 @@ __global__ void __launch_bounds__(C::NT) gemm_kernel(const GemmTable tab, int to
             v[e] = __int_as_float(sw[0]);
             v[4 + e] = __int_as_float(sw[1]);
           }
-          const int n = tc.n0 + wn0 + j * 32 + (2 * gp + lh) * 8;
-          if (m >= M || n >= N) continue;
+          const int chunk = j * 4 + 2 * gp + lh;  // 16-byte chunk inside the wave's 256-byte row
+          const int n = min(ncol0 + chunk * 8, N - 8);
           if (bias) {
             float bf[8];
             hdit::unpack8(*(const i32x4*)(bias + n), bf);
 #pragma unroll
             for (int e = 0; e < 8; e++) v[e] += bf[e];
           }
-          if (epi == HDIT_EPI_BIAS_GELU) {
+          if (epi_mode == HDIT_EPI_BIAS_GELU) {
 #pragma unroll
             for (int e = 0; e < 8; e++) v[e] = hdit::gelu_tanh_f(v[e]);
-          } else if (epi == HDIT_EPI_GATE_RESIDUAL) {
-            float rf[8];
-            hdit::unpack8(*(const i32x4*)(resid + (int64_t)m * ldr + n), rf);
+          } else if (epi_mode == HDIT_EPI_GATE_RESIDUAL) {
             f32x4 g0 = *(const f32x4*)(grow + n), g1 = *(const f32x4*)(grow + n + 4);
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-              v[e] = rf[e] + g0[e] * v[e];
-              v[4 + e] = rf[4 + e] + g1[e] * v[4 + e];
+              v[e] *= g0[e];
+              v[4 + e] *= g1[e];
             }
           }
-          *(i32x4*)(Cp + (int64_t)m * ldc + n) = hdit::pack8(v);
+          *(i32x4*)(epi + l32 * 256 + ((chunk ^ (l32 & 15)) << 4)) = hdit::pack8(v);
+        }
+      }
+      // coalesced write-back of this 32 x (32*TN) block: 16 lanes cover one row
+      const int rchunk = lane & 15;
+#pragma unroll
+      for (int it = 0; it < 8; it++) {
+        const int r = it * 4 + (lane >> 4);
+        const int mm = mrow0 + r;
+        const int nn = ncol0 + rchunk * 8;
+        i32x4 val = *(const i32x4*)(epi + r * 256 + ((rchunk ^ (r & 15)) << 4));
+        if (rchunk < 4 * TN && mm < M && nn < N) {
+          if (epi_mode == HDIT_EPI_GATE_RESIDUAL) {
+            float u[8], rf[8];
+            hdit::unpack8(val, u);
+            hdit::unpack8(*(const i32x4*)(resid + (int64_t)mm * ldr + nn), rf);
+#pragma unroll
+            for (int e = 0; e < 8; e++) u[e] += rf[e];
+            val = hdit::pack8(u);
+          }
+          *(i32x4*)(Cp + (int64_t)mm * ldc + nn) = val;
         }
       }
     }
 
-    if (!has_next) break;
-    lid = next_lid;
-    tc = ntc;
+    lid += wgs_per_xcd;
+    if (lid >= xcd_end) break;
   }
 }
 
@@ -259,15 +345,23 @@ int launch(const GemmTable& tab, int total_tiles, hipStream_t stream) {
     }
     attr_set = true;
   }
-  const int per_cu = (2 * C::LDS_BYTES <= 160 * 1024 && C::NT <= 256) ? 2 : 1;
+  const int per_cu = (2 * C::LDS_BYTES <= 160 * 1024) ? 2 : 1;
   int max_wgs = (num_cus * per_cu) / NUM_XCD * NUM_XCD;
   if (max_wgs < NUM_XCD) max_wgs = NUM_XCD;
   const int tiles_per_xcd = (total_tiles + NUM_XCD - 1) / NUM_XCD;
   int wgs_per_xcd = max_wgs / NUM_XCD;
   if (wgs_per_xcd > tiles_per_xcd) wgs_per_xcd = tiles_per_xcd;
-  hipLaunchKernelGGL(gemm_kernel<C>, dim3(wgs_per_xcd * NUM_XCD), dim3(C::NT), C::LDS_BYTES, stream, tab, total_tiles,
+  hipLaunchKernelGGL(gemm_kernel<C>, dim3(wgs_per_xcd * NUM_XCD), dim3(NT), C::LDS_BYTES, stream, tab, total_tiles,
                      tiles_per_xcd, wgs_per_xcd);
   return hdit_host::check_launch("hdit_gemm_bf16");
+}
+
+template <class C>
+int count_tiles(const hdit_gemm_problem* problems, int count) {
+  int total = 0;
+  for (int i = 0; i < count; i++)
+    total += ((problems[i].m + C::BM - 1) / C::BM) * ((problems[i].n + C::BN - 1) / C::BN);
+  return total;
 }
 
 template <class C>
@@ -285,11 +379,21 @@ int build_and_launch(const hdit_gemm_problem* problems, int count, hipStream_t s
   return launch<C>(tab, total, stream);
 }
 
-using Cfg256x256 = Cfg<256, 256, 2, 4>;
-using Cfg256x128 = Cfg<256, 128, 4, 2>;
-using Cfg128x128 = Cfg<128, 128, 2, 2>;
+using Cfg256x256 = Cfg<4, 4>;
+using Cfg256x192 = Cfg<4, 3>;
+using Cfg128x256 = Cfg<2, 4>;
+using Cfg128x128 = Cfg<2, 2>;
 
 int g_force_cfg = -1;
+
+// Relative cost of a launch with a given tile shape on 256 CUs: rounds of tiles times the time of one tile
+// (proportional to its area; smaller tiles pay more per flop for fragment traffic and epilogue).
+template <class C>
+double launch_cost(const hdit_gemm_problem* problems, int count, double per_flop_penalty, int slots) {
+  const int tiles = count_tiles<C>(problems, count);
+  const int rounds = (tiles + slots - 1) / slots;
+  return (double)rounds * C::BM * C::BN * per_flop_penalty;
+}
 
 }  // namespace
 
@@ -299,7 +403,6 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
   if (!problems || count < 0 || count > HDIT_GEMM_MAX_PROBLEMS) return HDIT_EINVAL;
   hdit_gemm_problem live[HDIT_GEMM_MAX_PROBLEMS];
   int nlive = 0;
-  int64_t tiles256 = 0, tiles_mid = 0;
   for (int i = 0; i < count; i++) {
     const hdit_gemm_problem& p = problems[i];
     if (p.m < 0 || p.n <= 0 || p.k <= 0) return HDIT_EINVAL;
@@ -308,28 +411,33 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
     if (p.k % BK != 0 || p.n % 8 != 0) return HDIT_EUNSUPPORTED;
     if (p.lda % 8 || p.ldb % 8 || p.ldc % 8) return HDIT_EINVAL;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uintptr_t)p.c | (uintptr_t)p.bias) & 15) return HDIT_EINVAL;
+    // the direct-to-LDS copies address rows with 32-bit byte offsets from the operand base
+    if ((int64_t)p.m * p.lda * 2 >= (1ll << 32) || (int64_t)p.n * p.ldb * 2 >= (1ll << 32)) return HDIT_EUNSUPPORTED;
     if (p.epilogue < HDIT_EPI_BIAS || p.epilogue > HDIT_EPI_GATE_RESIDUAL) return HDIT_EINVAL;
     if (p.epilogue == HDIT_EPI_GATE_RESIDUAL) {
       if (!p.resid || !p.gate || p.rows_per_batch <= 0 || p.ldr % 8) return HDIT_EINVAL;
       if (((uintptr_t)p.resid & 15) || ((uintptr_t)p.gate & 15) || p.gate_stride % 4) return HDIT_EINVAL;
     }
-    tiles256 += (int64_t)((p.m + 255) / 256) * ((p.n + 255) / 256);
-    tiles_mid += (int64_t)((p.m + 255) / 256) * ((p.n + 127) / 128);
     live[nlive++] = p;
   }
   if (nlive == 0) return HDIT_OK;
   hipStream_t s = (hipStream_t)stream;
   int cfg = g_force_cfg;
   if (cfg < 0) {
-    // Prefer the largest tile that still gives every CU (256 of them) work for
-    // about two rounds; small launches fall back to smaller tiles.
-    if (tiles256 >= 2 * 256) cfg = 0;
-    else if (tiles_mid >= 256) cfg = 1;
-    else cfg = 2;
+    const double c0 = launch_cost<Cfg256x256>(live, nlive, 1.00, 256);
+    const double c1 = launch_cost<Cfg256x192>(live, nlive, 1.04, 256);
+    const double c2 = launch_cost<Cfg128x256>(live, nlive, 1.10, 256);
+    const double c3 = launch_cost<Cfg128x128>(live, nlive, 1.30, 256);
+    cfg = 0;
+    double best = c0;
+    if (c1 < best) best = c1, cfg = 1;
+    if (c2 < best) best = c2, cfg = 2;
+    if (c3 < best) best = c3, cfg = 3;
   }
   switch (cfg) {
     case 0: return build_and_launch<Cfg256x256>(live, nlive, s);
-    case 1: return build_and_launch<Cfg256x128>(live, nlive, s);
+    case 1: return build_and_launch<Cfg256x192>(live, nlive, s);
+    case 2: return build_and_launch<Cfg128x256>(live, nlive, s);
     default: return build_and_launch<Cfg128x128>(live, nlive, s);
   }
 }
