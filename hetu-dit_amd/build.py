@@ -14,6 +14,7 @@ HIPCC_FLAGS = [
     "-std=c++17",
     "-fPIC",
     "-fvisibility=hidden",
+    "-fno-honor-nans",  # no kernel relies on NaN propagation; lets fmax chains become v_max3 without canonicalisation
     # packed-fp32 VALU forms are kept out of every kernel
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]

@@ -19,6 +19,8 @@
 // Q, K, V, O are each up to two sequence segments in different buffers, so the
 // joint [image, text] / [text, image] sequences and the "fresh text + stale
 // image buffer" K/V of a PipeFusion patch need no concatenation copy.
+#include <type_traits>
+
 #include "hdit_common.h"
 
 namespace {
@@ -49,13 +51,21 @@ struct AttnParams {
 
 template <int HD>
 struct Lds {
-  static constexpr int K_ROW = HD * 2 + 16;  // bytes; +16 keeps 8 consecutive rows on distinct banks
-  static constexpr int V_ROW = HD * 2 + 32;  // +32: the 4 key rows of one transpose read hit distinct banks
+  // Row strides chosen for the 64-bank (256-byte) LDS window: a ds_read_b128 pass covers 16 consecutive K
+  // rows, which must land on 16 distinct 16-byte slots (stride = 16 mod 256 works); a transpose-read pass
+  // covers 4 consecutive V rows x 64 bytes, which must land on 4 distinct 64-byte slots (stride = 64 mod 256).
+  static constexpr int K_ROW = HD * 2 + 16;
+  static constexpr int V_ROW = HD * 2 + 64;
   static constexpr int K_BYTES = BKV * K_ROW;
   static constexpr int V_BYTES = BKV * V_ROW;
   static constexpr int STAGE = K_BYTES + V_BYTES;
   static constexpr int TOTAL = 2 * STAGE;
 };
+
+// The running row maximum is only raised when some row's maximum grew by more than this many powers of
+// two; until then exp2(s - m) may reach 2^8, harmless for the bf16 P operand and the fp32 row sums, and the
+// accumulator rescale (the most expensive VALU block after the exponentials) is skipped for most tiles.
+constexpr float RESCALE_THRESHOLD = 8.0f;
 
 template <int HD>
 __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const AttnParams P, int q_tiles) {
@@ -83,15 +93,50 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     for (int ks = 0; ks < KS; ks++) qf[qb][ks] = *(const bf16x8*)(rp + ks * 16 + lh * 8);
   }
 
-  // ---- K/V tile staging
+  // ---- K/V tile staging: global -> registers -> LDS.  A tile that lies inside one segment is addressed as
+  // (wave-uniform base) + (loop-invariant per-thread offset); the tile that straddles the segment boundary
+  // and the last, clamped tile take the per-row path.
   i32x4 kreg[NCH], vreg[NCH];
-  auto load_tile = [&](int t) {
+  unsigned koff[2][NCH], voff[2][NCH];
 #pragma unroll
-    for (int i = 0; i < NCH; i++) {
-      int c = tid + i * 256, row = c / CPR, cc = c % CPR;
-      int r = min(t * BKV + row, P.skv - 1);
-      kreg[i] = *(const i32x4*)(row_ptr(P.k, b, h, r) + cc * 8);
-      vreg[i] = *(const i32x4*)(row_ptr(P.v, b, h, r) + cc * 8);
+  for (int i = 0; i < NCH; i++) {
+    const int c = tid + i * 256, row = c / CPR, cc = c % CPR;
+    koff[0][i] = (unsigned)((row * P.k.ss0 + cc * 8) * 2);
+    koff[1][i] = (unsigned)((row * P.k.ss1 + cc * 8) * 2);
+    voff[0][i] = (unsigned)((row * P.v.ss0 + cc * 8) * 2);
+    voff[1][i] = (unsigned)((row * P.v.ss1 + cc * 8) * 2);
+  }
+  const unsigned char* kb0 = (const unsigned char*)(P.k.p0 + b * P.k.sb0 + h * P.k.sh0);
+  const unsigned char* kb1 = (const unsigned char*)(P.k.p1 + b * P.k.sb1 + h * P.k.sh1);
+  const unsigned char* vb0 = (const unsigned char*)(P.v.p0 + b * P.v.sb0 + h * P.v.sh0);
+  const unsigned char* vb1 = (const unsigned char*)(P.v.p1 + b * P.v.sb1 + h * P.v.sh1);
+  const int len0 = P.k.len0;
+  auto load_tile = [&](int t) {
+    const int r0 = t * BKV;
+    if (r0 + BKV <= len0) {
+      const unsigned char* kb = kb0 + (int64_t)r0 * P.k.ss0 * 2;
+      const unsigned char* vb = vb0 + (int64_t)r0 * P.v.ss0 * 2;
+#pragma unroll
+      for (int i = 0; i < NCH; i++) {
+        kreg[i] = *(const i32x4*)(kb + koff[0][i]);
+        vreg[i] = *(const i32x4*)(vb + voff[0][i]);
+      }
+    } else if (r0 >= len0 && r0 + BKV <= P.skv) {
+      const unsigned char* kb = kb1 + (int64_t)(r0 - len0) * P.k.ss1 * 2;
+      const unsigned char* vb = vb1 + (int64_t)(r0 - len0) * P.v.ss1 * 2;
+#pragma unroll
+      for (int i = 0; i < NCH; i++) {
+        kreg[i] = *(const i32x4*)(kb + koff[1][i]);
+        vreg[i] = *(const i32x4*)(vb + voff[1][i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NCH; i++) {
+        int c = tid + i * 256, row = c / CPR, cc = c % CPR;
+        int r = min(r0 + row, P.skv - 1);
+        kreg[i] = *(const i32x4*)(row_ptr(P.k, b, h, r) + cc * 8);
+        vreg[i] = *(const i32x4*)(row_ptr(P.v, b, h, r) + cc * 8);
+      }
     }
   };
   auto store_tile = [&](int stage) {
@@ -117,39 +162,27 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   // lane-constant part of the V^T transpose-read address:
   // 16-lane group G = lane/16, x = lane%16: key row 4*(G/2) + x/4, column 16*(G%2) + 4*(x%4)
   const int vt_off = (4 * (lane >> 5) + ((lane & 15) >> 2)) * L::V_ROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  const int k_off = l32 * L::K_ROW + lh * 16;
+  const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
-  const int NT = (P.skv + BKV - 1) / BKV;
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-  if (NT > 1) load_tile(1);
-
-  for (int t = 0; t < NT; t++) {
-    const unsigned char* sk = lds + (t & 1) * L::STAGE;
+  // one K/V tile: scores, online softmax, PV.  MASK: keys >= valid do not exist (last tile only).
+  auto tile_compute = [&](const unsigned char* sk, auto mask_tag, int valid) {
+    constexpr bool MASK = decltype(mask_tag)::value;
     const unsigned char* sv = sk + L::K_BYTES;
-
-    // ---- S^T[kb][qb] = K_tile . Q^T
+    // ---- S^T[kb][qb] = K_tile . Q^T (first k-step starts from a zero accumulator operand)
     f32x16 sacc[2][2];
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-      for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) sacc[kb][qb][v] = 0.f;
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
-        bf16x8 kf = *(const bf16x8*)(sk + (kb * 32 + l32) * L::K_ROW + (ks * 2 + lh) * 16);
+        bf16x8 kf = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + ks * 32);
 #pragma unroll
         for (int qb = 0; qb < 2; qb++)
-          sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], sacc[kb][qb], 0, 0, 0);
+          sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], ks == 0 ? zero16 : sacc[kb][qb], 0, 0, 0);
       }
     }
-
-    // ---- mask keys past the end (last tile only)
-    if (t == NT - 1 && (P.skv % BKV) != 0) {
-      const int valid = P.skv - t * BKV;
+    if (MASK) {
 #pragma unroll
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
@@ -162,42 +195,55 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
         }
     }
 
-    // ---- online softmax (log2 domain); P^T rounded to bf16 in place
-    bf16x8 pf[2][4];  // [qb][u], u = 2*kb + half: 16 keys per PV k-step
+    // ---- online softmax in the log2 domain.  A lane owns one query column per qb and 32 of its 64 keys;
+    // the other 32 live in lane^32.
+    bf16x8 pf[2][4];  // [qb][u], u = 2*kb + half: the 16 keys of PV k-step u
+    float mcand[2];
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
-      float mx = sacc[0][qb][0];
+      float mx = fmaxf(sacc[0][qb][0], sacc[1][qb][0]);
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) mx = fmaxf(mx, sacc[kb][qb][v]);
+      for (int v = 1; v < 16; v++) mx = fmaxf(mx, fmaxf(sacc[0][qb][v], sacc[1][qb][v]));
       auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(mx), __float_as_int(mx), false, false);
       mx = fmaxf(__int_as_float(sw[0]), __int_as_float(sw[1]));
-      const float m_new = fmaxf(m_run[qb], mx * P.scale_log2);
-      const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
-      m_run[qb] = m_new;
-      float rs = 0.f;
+      mcand[qb] = fmaxf(m_run[qb], mx * P.scale_log2);
+    }
+    // raise the running maxima (and rescale) only if some row outgrew the threshold: wave-uniform branch
+    const bool grow = (mcand[0] - m_run[0] > RESCALE_THRESHOLD) || (mcand[1] - m_run[1] > RESCALE_THRESHOLD);
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - mcand[qb]);
+        m_run[qb] = mcand[qb];
+        l_run[qb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) oacc[db][qb][v] *= alpha;
+      }
+    }
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      const float m = m_run[qb];
+      float rs = l_run[qb];
 #pragma unroll
       for (int kb = 0; kb < 2; kb++) {
-        float p[16];
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          p[v] = __builtin_amdgcn_exp2f(sacc[kb][qb][v] * P.scale_log2 - m_new);
-          rs += p[v];
-        }
 #pragma unroll
         for (int hh = 0; hh < 2; hh++) {
           i32x4 pk;
 #pragma unroll
-          for (int e = 0; e < 4; e++) pk[e] = (int)hdit::pack2(p[hh * 8 + 2 * e], p[hh * 8 + 2 * e + 1]);
+          for (int e = 0; e < 4; e++) {
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][qb][hh * 8 + 2 * e], P.scale_log2, -m));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][qb][hh * 8 + 2 * e + 1], P.scale_log2, -m));
+            const uint32_t pp = hdit::pack2(p0, p1);
+            pk[e] = (int)pp;
+            // row sum of exactly the bf16 values that enter the PV product
+            rs = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pp), ones2, rs, false);
+          }
           pf[qb][kb * 2 + hh] = __builtin_bit_cast(bf16x8, pk);
         }
       }
-      l_run[qb] = l_run[qb] * alpha + rs;
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) oacc[db][qb][v] *= alpha;
+      l_run[qb] = rs;
     }
 
     // ---- O^T[db][qb] += V^T . P^T
@@ -217,10 +263,25 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
           oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qb][u], oacc[db][qb], 0, 0, 0);
       }
     }
+  };
 
-    if (t + 1 < NT) store_tile((t + 1) & 1);
+  const int NT = (P.skv + BKV - 1) / BKV;
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  if (NT > 1) load_tile(1);
+
+  for (int t = 0; t < NT - 1; t++) {
+    tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
+    store_tile((t + 1) & 1);
     __syncthreads();
     if (t + 2 < NT) load_tile(t + 2);
+  }
+  {
+    const int t = NT - 1;
+    const int valid = P.skv - t * BKV;
+    if (valid < BKV) tile_compute(lds + (t & 1) * L::STAGE, std::true_type{}, valid);
+    else tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
   }
 
   // ---- normalise and write O[q][d]: lane owns q = qb*32 + l32, d = 32*db + 8*(v/4) + 4*lh + v%4

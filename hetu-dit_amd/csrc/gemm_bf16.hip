@@ -5,25 +5,26 @@
 // (32*TM) x (32*TN) sub-tile in accumulators (v_mfma_f32_32x32x16_bf16).
 //
 // Staging.  Both operands are k-contiguous, so A and B tiles are staged the
-// same way: `global_load_lds_dwordx4` copies 64-wide k slabs straight from
+// same way: `global_load_lds_dwordx4` copies 32-wide k slabs straight from
 // global memory into LDS (no VGPR staging, no ds_write).  A wave-wide direct
-// load writes 1 KiB of LDS in lane order = 8 rows x 128 bytes.  The XOR swizzle
+// load writes 1 KiB of LDS in lane order = 16 rows x 64 bytes.  The XOR swizzle
 // that keeps the ds_read_b128 fragment reads conflict-free is applied on the
 // global side: the lane that fills 16-byte slot p of row r fetches chunk
-// p ^ ((r>>1)&7) of that row, which stays inside one 128-byte line, so the
-// global access remains fully coalesced.  Swizzling by (r>>1)&7 makes the 16
-// rows one ds_read_b128 pass touches land on 16 distinct 16-byte slots of the
-// 256-byte LDS bank window (measured 202 B/clk/CU, against 117 B/clk for r&7).
+// p ^ ((r>>2)&3) of that row's 64-byte slab, so the global access stays
+// coalesced, and the 16 rows one ds_read_b128 pass touches land on 16 distinct
+// 16-byte slots of the 256-byte LDS bank window (a linear pattern measured
+// 202 B/clk/CU, a 2-way conflicting one 117 B/clk).
 //
-// Pipeline.  The k slabs of all tiles of a workgroup form one flat stream with
-// two LDS stages.  While slab g is multiplied, slab g+1 is in flight; in the
-// last k-step of slab g every wave waits for its own copies, the workgroup
-// barrier makes slab g+1 visible and proves stage(g) free, the first
-// fragments of slab g+1 are read and the copy of slab g+2 is issued -- all
-// under the remaining MFMAs of slab g.  Fragments are double-buffered in
-// registers one k-step ahead.  Tile boundaries are invisible to the stream, so
-// a tile's first slabs arrive during the previous tile's last slab and
-// epilogue.
+// Pipeline.  The k slabs of all tiles of a workgroup form one flat stream over
+// four LDS stages.  While slab h is multiplied, slabs h+1 and h+2 have landed
+// or are landing and the copies of slab h+3 are issued a few at a time between
+// the MFMAs (a burst of copies starves the fragment reads).  In the last
+// k-step of slab h every wave waits for its own copies of slab h+1, the
+// workgroup barrier makes that slab visible and proves stage(h) free, and the
+// first fragments of slab h+1 are read under the remaining MFMAs of slab h.
+// Fragments are double-buffered in registers one k-step ahead.  Tile
+// boundaries are invisible to the stream, so a tile's first slabs arrive
+// during the previous tile's last slabs and epilogue.
 //
 // Epilogue.  A lane's accumulator holds one output row m and runs of 4
 // consecutive n; lanes l and l^32 swap halves (v_permlane32_swap) to own 8
@@ -39,8 +40,9 @@
 
 namespace {
 
-constexpr int BK = 64;          // k elements per LDS stage
-constexpr int ROW_BYTES = 128;  // BK * sizeof(bf16)
+constexpr int BK = 32;         // k elements per LDS stage
+constexpr int ROW_BYTES = 64;  // BK * sizeof(bf16)
+constexpr int STAGES = 4;
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 8;
 constexpr int NW = 4;
@@ -58,12 +60,14 @@ struct Cfg {
   static constexpr int TM = TM_, TN = TN_;
   static constexpr int BM = 64 * TM, BN = 64 * TN;
   static constexpr int WM = 32 * TM, WN = 32 * TN;
-  static constexpr int A_LOADS = BM / 8 / NW;  // direct-to-LDS wave loads per wave per slab (8 rows each)
-  static constexpr int B_LOADS = BN / 8 / NW;
+  static constexpr int A_LOADS = BM / 16 / NW;  // direct-to-LDS wave loads per wave per slab (16 rows each)
+  static constexpr int B_LOADS = BN / 16 / NW;
+  static constexpr int LOADS = A_LOADS + B_LOADS;
   static constexpr int A_BYTES = BM * ROW_BYTES;
   static constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
-  static constexpr int EPI_OFF = 2 * STAGE_BYTES;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES + NW * EPI_WAVE_BYTES;
+  static constexpr int EPI_OFF = STAGES * STAGE_BYTES;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + NW * EPI_WAVE_BYTES;
+  static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile/waves mismatch");
   static_assert(TN <= 4, "epilogue staging window is 128 columns wide");
 };
 
@@ -89,9 +93,20 @@ __device__ __forceinline__ TileCoord locate(const GemmTable& tab, int lid) {
   return tc;
 }
 
-__device__ __forceinline__ void lds_dma16(const void* gptr, unsigned char* lds_dst_uniform) {
-  __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)gptr,
-                                   (void __attribute__((address_space(3)))*)lds_dst_uniform, 16, 0, 0);
+// One wave-wide direct-to-LDS copy: lane l's 16 bytes at base + voff land at LDS byte address
+// lds_addr + 16*l.  Written as inline assembly on purpose: the compiler's wait-count insertion treats a
+// `__builtin_amdgcn_global_load_lds` as a pending write to all of LDS and forces vmcnt(0) before the next
+// ds_read, which would drain the whole copy pipeline at every slab; here the copies are only ever
+// waited for with the explicit s_waitcnt before the workgroup barrier.
+__device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr_uniform), "v"(voff), "s"(base_uniform)
+               : "m0");
+}
+
+__device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
+  return (unsigned)(uintptr_t)((const __attribute__((address_space(3))) unsigned char*)p);
 }
 
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
@@ -116,17 +131,17 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
   int lid = xcd_begin + blockIdx.x / NUM_XCD;
   if (lid >= xcd_end) return;
 
-  // ---- producer: the slab stream, two slabs ahead of the MFMAs ---------------
-  // Lane-constant parts of a direct-to-LDS copy: row-in-group l/8; the chunk a lane fetches is
-  // (l%8) ^ ((row>>1)&7) with row = 8*grp + l/8 and grp = wave + 4*i, whose parity is that of `wave`.
-  const int ld_row = lane >> 3;
-  const int ld_chunk = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+  // ---- producer: the slab stream, three slabs ahead of the MFMAs -------------
+  // Lane-constant parts of a direct-to-LDS copy: row-in-group l/4; the chunk a lane fetches is
+  // (l%4) ^ ((row>>2)&3) with row = 16*grp + l/4, i.e. (l%4) ^ ((l>>4)&3).
+  const int ld_row = lane >> 2;
+  const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);
   int p_lid = lid;
   bool p_valid = true;
   int p_kt = 0, p_KT = 0;
   const unsigned char* p_abase = nullptr;
   const unsigned char* p_bbase = nullptr;
-  unsigned p_aoff[C::A_LOADS], p_boff[C::B_LOADS];
+  unsigned p_off[C::LOADS];
   auto p_setup = [&]() {
     const TileCoord tc = locate<C>(tab, p_lid);
     const hdit_gemm_problem& pr = tab.p[tc.pi];
@@ -136,38 +151,46 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
     p_kt = 0;
 #pragma unroll
     for (int i = 0; i < C::A_LOADS; i++) {
-      const int gr = min(tc.m0 + (wave + i * NW) * 8 + ld_row, pr.m - 1);
-      p_aoff[i] = (unsigned)(((int64_t)gr * pr.lda + ld_chunk * 8) * 2);
+      const int gr = min(tc.m0 + (wave + i * NW) * 16 + ld_row, pr.m - 1);
+      p_off[i] = (unsigned)(((int64_t)gr * pr.lda + ld_chunk * 8) * 2);
     }
 #pragma unroll
     for (int i = 0; i < C::B_LOADS; i++) {
-      const int gr = min(tc.n0 + (wave + i * NW) * 8 + ld_row, pr.n - 1);
-      p_boff[i] = (unsigned)(((int64_t)gr * pr.ldb + ld_chunk * 8) * 2);
+      const int gr = min(tc.n0 + (wave + i * NW) * 16 + ld_row, pr.n - 1);
+      p_off[C::A_LOADS + i] = (unsigned)(((int64_t)gr * pr.ldb + ld_chunk * 8) * 2);
     }
   };
-  auto p_issue = [&](int stage) {
+  // copies [first, last) of the current producer slab into `stage`.  Unconditional (no branch may split
+  // the MFMA stream it is interleaved with): once the stream is exhausted the last slab is simply copied
+  // again into a stage nobody will read.
+  const unsigned lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds)) + wave * 1024;
+  auto p_issue_one = [&](int stage, int i) {
+    const unsigned dst = lds0 + stage * C::STAGE_BYTES;
+    if (i < C::A_LOADS) lds_dma16(p_abase + (size_t)p_kt * ROW_BYTES, p_off[i], dst + i * NW * 1024);
+    else lds_dma16(p_bbase + (size_t)p_kt * ROW_BYTES, p_off[i], dst + C::A_BYTES + (i - C::A_LOADS) * NW * 1024);
+  };
+  auto p_issue = [&](int stage, int first, int last) {
+#pragma unroll
+    for (int i = 0; i < C::LOADS; i++)
+      if (i >= first && i < last) p_issue_one(stage, i);
+  };
+  auto p_advance = [&]() {
     if (!p_valid) return;
-    unsigned char* base = lds + stage * C::STAGE_BYTES + wave * 1024;
-    const unsigned char* ak = p_abase + (size_t)p_kt * ROW_BYTES;
-    const unsigned char* bk = p_bbase + (size_t)p_kt * ROW_BYTES;
-#pragma unroll
-    for (int i = 0; i < C::A_LOADS; i++) lds_dma16(ak + p_aoff[i], base + i * NW * 1024);
-#pragma unroll
-    for (int i = 0; i < C::B_LOADS; i++) lds_dma16(bk + p_boff[i], base + C::A_BYTES + i * NW * 1024);
     if (++p_kt == p_KT) {
       p_lid += wgs_per_xcd;
       p_valid = p_lid < xcd_end;
       if (p_valid) p_setup();
+      else p_kt = p_KT - 1;
     }
   };
 
   // ---- consumer ------------------------------------------------------------
-  // fragment read offsets: row r, logical chunk c -> r*128 + ((c ^ ((r>>1)&7)) << 4); fragment rows are
-  // l32 plus a multiple of 32, so (r>>1)&7 == (l32>>1)&7
-  const int swz = (l32 >> 1) & 7;
-  int a_off[4], b_off[4];  // per k-step (chunk = 2*ks + lh)
+  // fragment read offsets: row r, logical chunk c -> r*64 + ((c ^ ((r>>2)&3)) << 4); fragment rows are
+  // l32 plus a multiple of 32, so (r>>2)&3 == (l32>>2)&3
+  const int swz = (l32 >> 2) & 3;
+  int a_off[2], b_off[2];  // per k-step (chunk = 2*ks + lh)
 #pragma unroll
-  for (int ks = 0; ks < 4; ks++) {
+  for (int ks = 0; ks < 2; ks++) {
     a_off[ks] = (wm0 + l32) * ROW_BYTES + (((ks * 2 + lh) ^ swz) << 4);
     b_off[ks] = C::A_BYTES + (wn0 + l32) * ROW_BYTES + (((ks * 2 + lh) ^ swz) << 4);
   }
@@ -180,8 +203,11 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
   };
 
   p_setup();
-  p_issue(0);
-  p_issue(1);
+#pragma unroll 1
+  for (int st = 0; st < STAGES - 1; st++) {
+    p_issue(st, 0, C::LOADS);
+    p_advance();
+  }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
   int stage = 0;
@@ -189,6 +215,9 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
 
   // wave-private epilogue staging window
   unsigned char* epi = lds + C::EPI_OFF + wave * EPI_WAVE_BYTES;
+  constexpr int NMMA = TM * TN;
+  constexpr int L0 = (C::LOADS + 1) / 2;  // copies issued in k-step 0, the rest in k-step 1
+  constexpr int NR = (TM + TN < NMMA - 1) ? TM + TN : NMMA - 1;  // MFMAs that are followed by a fragment read
 
   while (true) {
     const TileCoord tc = locate<C>(tab, lid);
@@ -205,42 +234,50 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
 
     for (int kt = 0; kt < KT; kt++) {
       const unsigned char* sbase = lds + stage * C::STAGE_BYTES;
+      const int pstage = (stage + STAGES - 1) & (STAGES - 1);  // freed by the previous slab's barrier
+      // ---- k-step 0: request the fragments of k-step 1 one per MFMA (an MFMA goes first, so that its
+      // wait for this step's fragments is placed while no younger read is outstanding and costs nothing),
+      // then one copy of slab h+3 per MFMA, then the remaining MFMAs
+      read_frags(sbase, 1, 1);
 #pragma unroll
-      for (int ks = 0; ks < 3; ks++) {
-        const int cur = ks & 1;
-        read_frags(sbase, ks + 1, cur ^ 1);
+      for (int t = 0; t < NMMA; t++) {
+        acc[t / TN][t % TN] =
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][t % TN], fa[0][t / TN], acc[t / TN][t % TN], 0, 0, 0);
+        if (t == NR) {  // all fragment reads are placed: pin the order so far
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 #pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-          for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
-        // issue order inside this k-step: one fragment read per MFMA until the next step's fragments are
-        // requested, then the remaining MFMAs (the reads get a full k-step to land)
-        // (an MFMA goes first, so that the wait for THIS step's fragments is placed while no younger
-        // read is outstanding and costs nothing)
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        constexpr int PAIRS = (TM + TN < TM * TN - 1) ? TM + TN : TM * TN - 1;
-#pragma unroll
-        for (int t = 0; t < PAIRS; t++) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+          for (int u = 0; u < TM + TN; u++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                // DS read
+            if (u < NR) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+          }
+          SCHED_FENCE();
         }
-        if (TM + TN - PAIRS > 0) __builtin_amdgcn_sched_group_barrier(0x100, TM + TN - PAIRS, 0);
-        if (TM * TN - 1 - PAIRS > 0) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1 - PAIRS, 0);
-        SCHED_FENCE();
+        if (t > NR && t - NR - 1 < L0) {
+          p_issue_one(pstage, t - NR - 1);
+          SCHED_FENCE();
+        }
       }
-      // last k-step (fragment buffer 1): first half of the MFMAs, then turn the stages over
-#pragma unroll
-      for (int i = 0; i < TM / 2; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+      if (NMMA - 1 - NR < L0) p_issue(pstage, NMMA - 1 - NR, L0);  // tiles with fewer MFMAs than slots
       SCHED_FENCE();
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my copies landed, my reads of this stage are done
+      // ---- k-step 1, first part: the remaining copies, one per MFMA
+#pragma unroll
+      for (int t = 0; t < NMMA / 2; t++) {
+        acc[t / TN][t % TN] =
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][t % TN], fa[1][t / TN], acc[t / TN][t % TN], 0, 0, 0);
+        if (t < C::LOADS - L0) {
+          p_issue_one(pstage, L0 + t);
+          SCHED_FENCE();
+        }
+      }
+      if (NMMA / 2 < C::LOADS - L0) p_issue(pstage, L0 + NMMA / 2, C::LOADS);
+      SCHED_FENCE();
+      p_advance();
+      // ---- turn the stages over: slab h+1 must have landed (h+2, h+3 may still be in flight; stores
+      // of an epilogue that are younger than those copies only make the wait conservative)
+      __builtin_amdgcn_s_waitcnt(0x0070 | ((2 * C::LOADS) & 15) | (((2 * C::LOADS) >> 4) << 14));
       __syncthreads();
-      stage ^= 1;
+      stage = (stage + 1) & (STAGES - 1);
       read_frags(lds + stage * C::STAGE_BYTES, 0, 0);
-      p_issue(stage ^ 1);
       SCHED_FENCE();
 #pragma unroll
       for (int i = TM / 2; i < TM; i++)
@@ -425,8 +462,8 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
   int cfg = g_force_cfg;
   if (cfg < 0) {
     const double c0 = launch_cost<Cfg256x256>(live, nlive, 1.00, 256);
-    const double c1 = launch_cost<Cfg256x192>(live, nlive, 1.04, 256);
-    const double c2 = launch_cost<Cfg128x256>(live, nlive, 1.10, 256);
+    const double c1 = launch_cost<Cfg256x192>(live, nlive, 1.05, 256);
+    const double c2 = launch_cost<Cfg128x256>(live, nlive, 1.08, 256);
     const double c3 = launch_cost<Cfg128x128>(live, nlive, 1.30, 256);
     cfg = 0;
     double best = c0;

@@ -51,14 +51,18 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 __device__ __forceinline__ float gelu_tanh_f(float x) {
-  // 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3); 1 + tanh(u) = 2 - 2/(1 + e^{2u})
-  const float c = 0.7978845608028654f;
-  float u = c * (x + 0.044715f * x * x * x);
-  float e = __expf(2.0f * u);
-  return x * (1.0f - 1.0f / (1.0f + e));
+  // 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3), equals x * sigmoid(2u) = x / (1 + 2^(-2u log2 e)).
+  // Written on v_exp_f32 / v_rcp_f32 directly: five full-rate VALU ops and two transcendentals per value.
+  const float k = 2.0f * 0.7978845608028654f * 1.4426950408889634f;  // 2 sqrt(2/pi) log2(e)
+  const float t = x * x;
+  const float p = __builtin_fmaf(t, 0.044715f * k, k);
+  const float e = __builtin_amdgcn_exp2f(-(x * p));
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
-__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
 
 }  // namespace hdit
 
