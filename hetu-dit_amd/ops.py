@@ -190,7 +190,9 @@ def attention(q: Sequence[torch.Tensor], k: Sequence[torch.Tensor], v: Sequence[
         nbytes = 2.0 * args.batch * args.heads * args.head_dim * (sq + 2 * skv)
         check(_run("attn_absmax", nbytes, lambda: lib.hdit_attn_absmax(C.byref(args), absmax.data_ptr(), _stream())),
               "hdit_attn_absmax")
-        check(_run("attn_fp8", flops, lambda: lib.hdit_attn_fwd_fp8(C.byref(args), absmax.data_ptr(), _stream())),
+        ws = torch.empty(lib.hdit_attn_fp8_workspace_bytes(C.byref(args)), dtype=torch.uint8, device=q[0].device)
+        check(_run("attn_fp8", flops,
+                   lambda: lib.hdit_attn_fwd_fp8(C.byref(args), absmax.data_ptr(), ws.data_ptr(), _stream())),
               "hdit_attn_fwd_fp8")
     else:
         check(_run("attn_bf16", flops, lambda: lib.hdit_attn_fwd_bf16(C.byref(args), _stream())), "hdit_attn_fwd_bf16")

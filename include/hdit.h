@@ -101,13 +101,16 @@ typedef struct hdit_attn_args {
 
 int hdit_attn_fwd_bf16(const hdit_attn_args* args, void* stream);
 
-/* Same contract; Q, K, V are quantised to fp8-e4m3 (OCP) on the fly with one
+/* Same contract on the fp8-e4m3 (OCP) MFMA path: Q, K, V are quantised with one
  * absmax scale per (batch, head) taken from `absmax` (f32 [3, batch, heads]:
- * q, k, v), P is re-quantised per tile.  `absmax` is produced by
- * hdit_attn_absmax.  No counterpart exists in the reference (it has no fp8
- * path); the call site is the same as hdit_attn_fwd_bf16. */
+ * q, k, v; written by hdit_attn_absmax), P is re-quantised per tile.  K and V
+ * are quantised once into `workspace` (hdit_attn_fp8_workspace_bytes(args)
+ * bytes, 16-byte aligned, caller-owned).  No counterpart exists in the
+ * reference (it has no fp8 path); the call site is that of
+ * hdit_attn_fwd_bf16. */
 int hdit_attn_absmax(const hdit_attn_args* args, float* absmax, void* stream);
-int hdit_attn_fwd_fp8(const hdit_attn_args* args, const float* absmax, void* stream);
+int64_t hdit_attn_fp8_workspace_bytes(const hdit_attn_args* args);
+int hdit_attn_fwd_fp8(const hdit_attn_args* args, const float* absmax, void* workspace, void* stream);
 
 /* ------------------------------------------------------------------------
  * Bandwidth-bound glue, one coalesced pass each.

@@ -187,3 +187,32 @@ def test_sd3_pipefusion_patches_stale_kv(hdit):
         assert_parity(got, want, what=f"patch {p}")
         rs.next_patch()
     assert rs.pipeline_patch_idx == 0
+
+
+@pytest.mark.parametrize("family", ["sd3", "cogvideox"])
+def test_block_with_fp8_attention(hdit, family):
+    """The fp8-e4m3 attention path inside a block, against the fp32 oracle at the tolerance BASELINE.json
+    states for it: relative L2 <= 3e-2 on the block outputs."""
+    from hetu_dit_amd import blocks, synthetic
+
+    if family == "sd3":
+        B, N, Nt, D, H = 2, 320, 77, 256, 4
+        blk, params = make(hdit, blocks.JointTransformerBlock, 51, D, H, 64)
+        blk.attn.fp8_attention = True
+        x, e, t = synthetic.randn_bf16((B, N, D), 52), synthetic.randn_bf16((B, Nt, D), 53), synthetic.randn_bf16((B, D), 54)
+        enc, hid = blk(hidden_states=x.to(DEV), encoder_hidden_states=e.to(DEV), temb=t.to(DEV))
+        torch.cuda.synchronize()
+        o_enc, o_hid = oracle.sd3_joint_block(params, x.float(), e.float(), t.float(), H)
+    else:
+        B, Nt, grid, D, H, hd = 1, 26, (3, 6, 8), 256, 4, 64
+        N = grid[0] * grid[1] * grid[2]
+        cos, sin = synthetic.rope_table(synthetic.cogvideox_positions(*grid), (16, 24, 24))
+        blk, params = make(hdit, blocks.CogVideoXBlock, 55, D, H, hd, time_embed_dim=64)
+        blk.attn1.fp8_attention = True
+        x, e, t = synthetic.randn_bf16((B, N, D), 56), synthetic.randn_bf16((B, Nt, D), 57), synthetic.randn_bf16((B, 64), 58)
+        hid, enc = blk(hidden_states=x.to(DEV), encoder_hidden_states=e.to(DEV), temb=t.to(DEV),
+                       image_rotary_emb=(cos.to(DEV), sin.to(DEV)))
+        torch.cuda.synchronize()
+        o_hid, o_enc = oracle.cogvideox_block(params, x.float(), e.float(), t.float(), (cos, sin), H)
+    assert_parity(hid, o_hid, rel=3e-2, cos=0.999, what=f"{family} fp8 hidden")
+    assert_parity(enc, o_enc, rel=3e-2, cos=0.999, what=f"{family} fp8 encoder")
