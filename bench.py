@@ -141,6 +141,14 @@ def main():
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # one plain device copy of known size (256 MiB read + 256 MiB written): the scale reference for the
+    # FETCH_SIZE / WRITE_SIZE hardware counters when this command runs under `rocprofv3 --pmc`
+    calib_src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    calib_dst = torch.empty_like(calib_src)
+    calib_dst.copy_(calib_src)
+    torch.cuda.synchronize()
+    del calib_src, calib_dst
+
     # instrumented eager pass: HIP events around every launch on the launch stream
     timer = ops.KernelTimer()
     ops.set_timer(timer)

@@ -21,84 +21,100 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const __bf16* __restri
                                                           const __bf16* __restrict__ lb, int64_t rows, int tokens,
                                                           int dim, int64_t x_sb, int64_t x_st, int64_t y_sb,
                                                           int64_t y_st, int64_t mod_stride, float eps) {
+  // A wave normalises two consecutive rows; the second row's loads are in flight while the first is
+  // reduced and written, so reads and writes of the launch overlap instead of running as two global
+  // phases (measured 5.7 TB/s against 4.9 TB/s for one row per wave at [8192, 1536]).
+  constexpr int RPW = 2;
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW;
+  if (row0 >= rows) return;
   const int nchunks = dim >> 3;
-  const int b = (int)(row / tokens);
-  const int64_t t = row - (int64_t)b * tokens;
-  const __bf16* xr = x + b * x_sb + t * x_st;
-  i32x4 raw[NCH];
-#pragma unroll
-  for (int i = 0; i < NCH; i++) {
-    int c = lane + i * 64;
-    if (c < nchunks) raw[i] = __builtin_nontemporal_load((const i32x4*)(xr + c * 8));
-  }
-  float s = 0.f;
-  float f[NCH][8];
-#pragma unroll
-  for (int i = 0; i < NCH; i++) {
-    int c = lane + i * 64;
-    if (c < nchunks) {
-      unpack8(raw[i], f[i]);
-#pragma unroll
-      for (int e = 0; e < 8; e++) s += f[i][e];
-    }
-  }
   const float inv_d = 1.0f / (float)dim;
-  const float mean = wave_sum(s) * inv_d;
-  float q = 0.f;
+  i32x4 raw[RPW][NCH];
+  auto row_x = [&](int64_t row) {
+    const int64_t b = row / tokens;
+    return x + b * x_sb + (row - b * tokens) * x_st;
+  };
+  auto load = [&](int buf, int64_t row) {
+    const __bf16* xr = row_x(row);
 #pragma unroll
-  for (int i = 0; i < NCH; i++) {
-    int c = lane + i * 64;
-    if (c < nchunks) {
+    for (int i = 0; i < NCH; i++) {
+      int c = lane + i * 64;
+      if (c < nchunks) raw[buf][i] = __builtin_nontemporal_load((const i32x4*)(xr + c * 8));
+    }
+  };
+  load(0, row0);
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        f[i][e] -= mean;
-        q += f[i][e] * f[i][e];
+  for (int r = 0; r < RPW; r++) {
+    const int64_t row = row0 + r;
+    if (row >= rows) break;
+    if (r + 1 < RPW && row + 1 < rows) load(r + 1, row + 1);
+    float s = 0.f;
+    float f[NCH][8];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      int c = lane + i * 64;
+      if (c < nchunks) {
+        unpack8(raw[r][i], f[i]);
+#pragma unroll
+        for (int e = 0; e < 8; e++) s += f[i][e];
       }
     }
-  }
-  const float rstd = rsqrtf(wave_sum(q) * inv_d + eps);
-  const float* sh = shift ? shift + (int64_t)b * mod_stride : nullptr;
-  const float* sc = scale ? scale + (int64_t)b * mod_stride : nullptr;
-  __bf16* yr = y + b * y_sb + t * y_st;
+    const float mean = wave_sum(s) * inv_d;
+    float q = 0.f;
 #pragma unroll
-  for (int i = 0; i < NCH; i++) {
-    int c = lane + i * 64;
-    if (c < nchunks) {
-      float o[8];
+    for (int i = 0; i < NCH; i++) {
+      int c = lane + i * 64;
+      if (c < nchunks) {
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = f[i][e] * rstd;
-      if (lw) {
-        float w[8];
-        unpack8(*(const i32x4*)(lw + c * 8), w);
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[e] *= w[e];
-      }
-      if (lb) {
-        float w[8];
-        unpack8(*(const i32x4*)(lb + c * 8), w);
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[e] += w[e];
-      }
-      if (sc) {
-        f32x4 s0 = *(const f32x4*)(sc + c * 8), s1 = *(const f32x4*)(sc + c * 8 + 4);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          o[e] *= 1.0f + s0[e];
-          o[e + 4] *= 1.0f + s1[e];
+        for (int e = 0; e < 8; e++) {
+          f[i][e] -= mean;
+          q += f[i][e] * f[i][e];
         }
       }
-      if (sh) {
-        f32x4 s0 = *(const f32x4*)(sh + c * 8), s1 = *(const f32x4*)(sh + c * 8 + 4);
+    }
+    const float rstd = rsqrtf(wave_sum(q) * inv_d + eps);
+    const int64_t b = row / tokens;
+    const float* sh = shift ? shift + b * mod_stride : nullptr;
+    const float* sc = scale ? scale + b * mod_stride : nullptr;
+    __bf16* yr = y + b * y_sb + (row - b * tokens) * y_st;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-          o[e] += s0[e];
-          o[e + 4] += s1[e];
+    for (int i = 0; i < NCH; i++) {
+      int c = lane + i * 64;
+      if (c < nchunks) {
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = f[i][e] * rstd;
+        if (lw) {
+          float w[8];
+          unpack8(*(const i32x4*)(lw + c * 8), w);
+#pragma unroll
+          for (int e = 0; e < 8; e++) o[e] *= w[e];
         }
+        if (lb) {
+          float w[8];
+          unpack8(*(const i32x4*)(lb + c * 8), w);
+#pragma unroll
+          for (int e = 0; e < 8; e++) o[e] += w[e];
+        }
+        if (sc) {
+          f32x4 s0 = *(const f32x4*)(sc + c * 8), s1 = *(const f32x4*)(sc + c * 8 + 4);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            o[e] *= 1.0f + s0[e];
+            o[e + 4] *= 1.0f + s1[e];
+          }
+        }
+        if (sh) {
+          f32x4 s0 = *(const f32x4*)(sh + c * 8), s1 = *(const f32x4*)(sh + c * 8 + 4);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            o[e] += s0[e];
+            o[e + 4] += s1[e];
+          }
+        }
+        __builtin_nontemporal_store(pack8(o), (i32x4*)(yr + c * 8));
       }
-      __builtin_nontemporal_store(pack8(o), (i32x4*)(yr + c * 8));
     }
   }
 }
@@ -157,37 +173,64 @@ __global__ void __launch_bounds__(256) gelu_kernel(const __bf16* __restrict__ x,
 // adaLN projection: out[b, n] = W[n, :] . silu(temb[b, :]) + bias[n]
 // One wave per output row; the weight row is streamed once for all batches.
 // ---------------------------------------------------------------------------
-template <int MAXB>
+template <int MAXB, int NCH>
 __global__ void __launch_bounds__(256) adaln_gemv_kernel(const __bf16* __restrict__ temb, const __bf16* __restrict__ w,
                                                          const __bf16* __restrict__ bias, float* __restrict__ out,
                                                          int batch, int n, int k) {
+  // A wave produces RW consecutive output rows: all of their weight chunks are requested before any is
+  // consumed (RW * NCH 16-byte loads in flight per lane), and the silu(temb) chunks are reused across rows.
+  constexpr int RW = 4;
   const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= n) return;
+  const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RW;
+  if (row0 >= n) return;
   const int nchunks = k >> 3;
-  float acc[MAXB];
+  i32x4 wraw[RW][NCH];
 #pragma unroll
-  for (int b = 0; b < MAXB; b++) acc[b] = 0.f;
-  const __bf16* wr = w + (int64_t)row * k;
-  for (int c = lane; c < nchunks; c += 64) {
-    float fw[8];
-    unpack8(__builtin_nontemporal_load((const i32x4*)(wr + c * 8)), fw);
+  for (int r = 0; r < RW; r++)
 #pragma unroll
-    for (int b = 0; b < MAXB; b++) {
-      if (b < batch) {
-        float ft[8];
-        unpack8(*(const i32x4*)(temb + (int64_t)b * k + c * 8), ft);
+    for (int i = 0; i < NCH; i++) {
+      const int c = lane + i * 64;
+      const int row = min(row0 + r, n - 1);
+      if (c < nchunks) wraw[r][i] = __builtin_nontemporal_load((const i32x4*)(w + (int64_t)row * k + c * 8));
+    }
+  float acc[RW][MAXB];
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[b] += fw[e] * hdit::silu_f(ft[e]);
+  for (int r = 0; r < RW; r++)
+#pragma unroll
+    for (int b = 0; b < MAXB; b++) acc[r][b] = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    const int c = lane + i * 64;
+    if (c < nchunks) {
+#pragma unroll
+      for (int b = 0; b < MAXB; b++) {
+        if (b < batch) {
+          float ft[8];
+          unpack8(*(const i32x4*)(temb + (int64_t)b * k + c * 8), ft);
+#pragma unroll
+          for (int e = 0; e < 8; e++) ft[e] = hdit::silu_f(ft[e]);
+#pragma unroll
+          for (int r = 0; r < RW; r++) {
+            float fw[8];
+            unpack8(wraw[r][i], fw);
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[r][b] += fw[e] * ft[e];
+          }
+        }
       }
     }
   }
-  float bv = bias ? (float)bias[row] : 0.f;
 #pragma unroll
-  for (int b = 0; b < MAXB; b++) {
-    if (b < batch) {
-      float r = wave_sum(acc[b]);
-      if (lane == 0) out[(int64_t)b * n + row] = r + bv;
+  for (int r = 0; r < RW; r++) {
+    const int row = row0 + r;
+    if (row >= n) break;
+    const float bv = bias ? (float)bias[row] : 0.f;
+#pragma unroll
+    for (int b = 0; b < MAXB; b++) {
+      if (b < batch) {
+        float v = wave_sum(acc[r][b]);
+        if (lane == 0) out[(int64_t)b * n + row] = v + bv;
+      }
     }
   }
 }
@@ -307,7 +350,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate(co
     return HDIT_EINVAL;
   int64_t rows = (int64_t)batch * tokens;
   if (rows == 0) return HDIT_OK;
-  dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  dim3 grid((unsigned)((rows + 7) / 8)), block(256);  // 4 waves x 2 rows
   hipStream_t s = (hipStream_t)stream;
   int nch = (dim / 8 + 63) / 64;
 #define LN_LAUNCH(N)                                                                                             \
@@ -357,14 +400,25 @@ extern "C" __attribute__((visibility("default"))) int hdit_adaln_gemv(const void
   if (!temb || !w || !out || batch <= 0 || n <= 0 || k <= 0) return HDIT_EINVAL;
   if (batch > 8) return HDIT_EUNSUPPORTED;
   if (k % 8 || !aligned16(temb) || !aligned16(w)) return HDIT_EINVAL;
-  dim3 grid((n + 3) / 4), block(256);
+  if (k > 8 * 512) return HDIT_EUNSUPPORTED;
+  dim3 grid((n + 15) / 16), block(256);  // 4 waves x 4 rows
   hipStream_t s = (hipStream_t)stream;
-  if (batch <= 2)
-    hipLaunchKernelGGL(adaln_gemv_kernel<2>, grid, block, 0, s, (const __bf16*)temb, (const __bf16*)w,
-                       (const __bf16*)bias, out, batch, n, k);
-  else
-    hipLaunchKernelGGL(adaln_gemv_kernel<8>, grid, block, 0, s, (const __bf16*)temb, (const __bf16*)w,
-                       (const __bf16*)bias, out, batch, n, k);
+  const int nch = (k / 8 + 63) / 64;
+#define GEMV_LAUNCH(MB, NC)                                                                                    \
+  hipLaunchKernelGGL((adaln_gemv_kernel<MB, NC>), grid, block, 0, s, (const __bf16*)temb, (const __bf16*)w, \
+                     (const __bf16*)bias, out, batch, n, k)
+  if (batch <= 2) {
+    if (nch <= 1) GEMV_LAUNCH(2, 1);
+    else if (nch <= 3) GEMV_LAUNCH(2, 3);
+    else if (nch <= 6) GEMV_LAUNCH(2, 6);
+    else GEMV_LAUNCH(2, 8);
+  } else {
+    if (nch <= 1) GEMV_LAUNCH(8, 1);
+    else if (nch <= 3) GEMV_LAUNCH(8, 3);
+    else if (nch <= 6) GEMV_LAUNCH(8, 6);
+    else GEMV_LAUNCH(8, 8);
+  }
+#undef GEMV_LAUNCH
   return hdit_host::check_launch("hdit_adaln_gemv");
 }
 

@@ -137,7 +137,7 @@ int hdit_gate_residual(const void* x, const void* y, const float* gate, void* ou
                        int64_t o_sb, int64_t o_st, int64_t gate_stride, void* stream);
 
 /* out[b, :] = W . silu(temb[b, :]) + bias   (W bf16 [n, k], temb bf16 [batch, k],
- * bias bf16 [n] or NULL, out f32 [batch, n]); batch <= 8, k % 8 == 0.
+ * bias bf16 [n] or NULL, out f32 [batch, n]); batch <= 8, k % 8 == 0, k <= 4096.
  * The `linear(silu(emb))` of every adaLN module (weight-bandwidth bound). */
 int hdit_adaln_gemv(const void* temb, const void* w, const void* bias, float* out, int batch,
                     int n, int k, void* stream);

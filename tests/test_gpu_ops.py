@@ -221,3 +221,14 @@ def test_attention_fp8_two_segments(hdit):
                        torch.cat([v_img, v_txt], 1).transpose(1, 2)).transpose(1, 2)
     assert_parity(o_img, want[:, :n_q], rel=FP8_KERNEL_REL, cos=0.998, what="fp8 img")
     assert_parity(o_txt, want[:, n_q:], rel=FP8_KERNEL_REL, cos=0.998, what="fp8 txt")
+
+
+def test_torch_library_ops_dispatch_to_the_hip_kernels(hdit):
+    import hetu_dit_amd.torch_ops  # noqa: F401
+
+    x, w, b = rnd(3, 40, 128), rnd(256, 128, scale=0.05), rnd(256)
+    y = torch.ops.hdit.linear(g(x), g(w), g(b), True)
+    n = torch.ops.hdit.layernorm_modulate(g(x))
+    torch.cuda.synchronize()
+    assert_parity(y, O.gelu_tanh(O.linear(x, w, b)), what="torch.ops.hdit.linear")
+    assert_parity(n, O.layer_norm(x, 1e-6), what="torch.ops.hdit.layernorm_modulate")

@@ -1,0 +1,175 @@
+"""Host-side mirror of the reference's plug-in surface: registries, runtime patch state, KV-cache
+bookkeeping, wrapper construction and the parameter-name contract.  CPU only."""
+import pytest
+import torch
+from torch import nn
+
+
+def test_layer_registry_picks_most_specific_and_rejects_unknown():
+    from hetu_dit_amd.registry import hetuDiTLayerWrappersRegister as R
+
+    class Base(nn.Module):
+        pass
+
+    class Child(Base):
+        pass
+
+    @R.register(Base)
+    class WBase:
+        pass
+
+    @R.register(Child)
+    class WChild:
+        pass
+
+    try:
+        assert R.get_wrapper(Base()) is WBase
+        assert R.get_wrapper(Child()) is WChild
+        with pytest.raises(ValueError, match="is not supported by hetuDiT"):
+            R.get_wrapper(nn.Identity())
+    finally:
+        R._HETUDIT_LAYER_MAPPING.pop(Base)
+        R._HETUDIT_LAYER_MAPPING.pop(Child)
+
+
+def test_processor_registry_requires_subclass_and_returns_class():
+    from hetu_dit_amd.layers import attention_processor as ap
+    from hetu_dit_amd.layers.modules import FluxAttnProcessor2_0, JointAttnProcessor2_0
+    from hetu_dit_amd.registry import hetuDiTAttentionProcessorRegister as R
+
+    assert R.get_processor(JointAttnProcessor2_0()) is ap.hetuDiTJointAttnProcessor2_0
+    assert R.get_processor(FluxAttnProcessor2_0()) is ap.hetuDiTFluxAttnProcessor2_0
+    with pytest.raises(ValueError):
+        R.get_processor(object())
+    with pytest.raises(ValueError):
+        @R.register(JointAttnProcessor2_0)
+        class NotASubclass:
+            pass
+
+
+def test_runtime_state_patches_match_reference_arithmetic():
+    from hetu_dit_amd.runtime_state import DiTRuntimeState
+
+    rs = DiTRuntimeState()
+    rs.set_patches(latents_height=128, latents_width=128, patch_size=2, num_pipeline_patch=4)
+    assert rs.num_pipeline_patch == 4
+    assert rs.pp_patches_height == [32, 32, 32, 32]
+    assert rs.pp_patches_token_start_idx_local == [0, 1024, 2048, 3072, 4096]
+    # uneven: 100 rows / 3 patches -> heights rounded up to a multiple of the patch size
+    rs.set_patches(latents_height=100, latents_width=64, patch_size=2, num_pipeline_patch=3)
+    assert rs.pp_patches_height == [34, 34, 32]
+    assert rs.pp_patches_token_start_idx_local == [0, 32 * 17, 32 * 34, 32 * 50]
+    rs.set_patched_mode(True)
+    seen = []
+    for _ in range(7):
+        seen.append(rs.pipeline_patch_idx)
+        rs.next_patch()
+    assert seen == [0, 1, 2, 0, 1, 2, 0]
+    rs.set_patched_mode(False)
+    rs.next_patch()
+    assert rs.pipeline_patch_idx == 0
+
+
+def test_cache_manager_registration_and_patch_range():
+    from hetu_dit_amd.cache_manager import CacheManager
+    from hetu_dit_amd.runtime_state import get_runtime_state, reset_runtime_state
+
+    rs = reset_runtime_state()
+    cm = CacheManager()
+    layer = object()
+    with pytest.raises(ValueError, match="Layer type"):
+        cm.register_cache_entry(layer, "mlp")
+    with pytest.raises(ValueError, match="Cache type"):
+        cm.register_cache_entry(layer, "attn", "lru")
+    cm.register_cache_entry(layer, "attn", "naive_cache")
+    assert cm._patch_range() is None  # patch mode off
+    rs.set_token_patches([0, 64, 128])
+    assert cm._patch_range() is None  # still off
+    rs.set_patched_mode(True)
+    assert cm._patch_range() == (0, 64)
+    rs.next_patch()
+    assert cm._patch_range() == (64, 128)
+    with pytest.raises(RuntimeError, match="before a full-sequence pass"):
+        cm.kv_buffer(layer, 1, 64, 8, "cpu")
+    with pytest.raises(KeyError):
+        cm._entry(object(), "attn")
+    reset_runtime_state()
+
+
+def test_wrappers_rehome_biases_and_keep_parameter_paths():
+    from hetu_dit_amd import blocks
+    from hetu_dit_amd.cache_manager import reset_cache_manager
+
+    blk = blocks.JointTransformerBlock(128, 2, 64)
+    names = {n for n, _ in blk.named_parameters()}
+    for n in ("attn.module.to_q.weight", "attn.module.add_k_proj.bias", "attn.module.to_out.0.weight",
+              "attn.module.to_add_out.weight", "attn.output_bias", "attn.encoder_output_bias",
+              "ff.module.net.0.proj.weight", "ff.module.net.2.weight", "ff.output_bias",
+              "ff_context.module.net.0.proj.bias", "norm1.linear.weight", "norm1_context.linear.bias"):
+        assert n in names, n
+    assert "attn.module.to_out.0.bias" not in names and "ff.module.net.2.bias" not in names
+    assert blk.attn.has_output_bias and blk.attn.has_encoder_output_bias and blk.ff.has_output_bias
+    # attribute fall-through to the wrapped module
+    assert blk.attn.heads == 2 and blk.attn.to_q is blk.attn.module.to_q
+    last = blocks.JointTransformerBlock(128, 2, 64, context_pre_only=True)
+    assert last.ff_context is None and not hasattr(last.attn.module, "to_add_out")
+    assert last.norm1_context.linear.weight.shape == (256, 128)
+    cog = blocks.CogVideoXBlock(128, 2, 64, time_embed_dim=32)
+    assert "attn1.module.norm_q.bias" in {n for n, _ in cog.named_parameters()}
+    reset_cache_manager()
+
+
+def test_packed_projection_views_and_repack():
+    from hetu_dit_amd.layers.attention_processor import _PackedProjection
+
+    a, b, c = nn.Linear(8, 4), nn.Linear(8, 4), nn.Linear(8, 6)
+    pk = _PackedProjection([a, b, c])
+    w, bias = pk.get()
+    assert w.shape == (14, 8) and bias.shape == (14,)
+    assert a.weight.data_ptr() == w.data_ptr() and c.weight.data_ptr() == w[8:].data_ptr()
+    w[0, 0] = 42.0
+    assert a.weight[0, 0].item() == 42.0  # the Linear is a view of the packed buffer
+    # weight hot-swap re-assigns .data: the pack must notice and rebuild
+    b.weight.data = torch.full((4, 8), 7.0)
+    w2, _ = pk.get()
+    assert w2.data_ptr() != w.data_ptr() and torch.all(w2[4:8] == 7.0)
+    wq, bq = pk.rows(4, 4)
+    assert torch.all(wq == 7.0) and bq.shape == (4,)
+
+
+def test_ops_refuse_cpu_tensors():
+    from hetu_dit_amd import ops
+
+    x = torch.zeros(1, 4, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.layernorm_modulate(x)
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.linear(x, torch.zeros(64, 64, dtype=torch.bfloat16))
+
+
+def test_single_rank_parallel_state():
+    from hetu_dit_amd import parallel_state as ps
+
+    assert ps.get_tensor_model_parallel_world_size() == 1 and ps.get_sequence_parallel_world_size() == 1
+    assert ps.get_pipeline_parallel_world_size() == 1 and ps.is_pipeline_first_stage() and ps.is_pipeline_last_stage()
+    t = torch.ones(2)
+    assert ps.get_tp_group().all_reduce(t) is t
+
+
+def test_torch_library_ops_have_fake_kernels():
+    """torch.ops.hdit.* trace under FakeTensorMode without touching a device."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    import hetu_dit_amd.torch_ops  # noqa: F401
+
+    with FakeTensorMode():
+        x = torch.empty(2, 7, 64, dtype=torch.bfloat16, device="cuda")
+        w = torch.empty(128, 64, dtype=torch.bfloat16, device="cuda")
+        assert torch.ops.hdit.linear(x, w).shape == (2, 7, 128)
+        assert torch.ops.hdit.layernorm_modulate(x).shape == x.shape
+        t = torch.empty(2, 64, dtype=torch.bfloat16, device="cuda")
+        out = torch.ops.hdit.adaln_gemv(t, w)
+        assert out.shape == (2, 128) and out.dtype == torch.float32
+        q = torch.empty(2, 7, 1, 64, dtype=torch.bfloat16, device="cuda")
+        (o,) = torch.ops.hdit.attention([q], [q], [q])
+        assert o.shape == q.shape
