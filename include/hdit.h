@@ -36,8 +36,8 @@ const char* hdit_last_error(void);
  *
  * A [m, k] row-major (lda), B [n, k] row-major (ldb; an nn.Linear weight),
  * C [m, n] row-major (ldc); fp32 accumulation on MFMA.  Requirements:
- * k % 64 == 0, n % 8 == 0, lda/ldb % 8 == 0, ldc/ldr % 4 == 0, pointers
- * 16-byte (A, B) / 8-byte (C, resid, bias) aligned.  Up to
+ * k % 32 == 0, n % 8 == 0, lda/ldb/ldc/ldr % 8 == 0, every pointer 16-byte
+ * aligned, m * lda and n * ldb below 2^31 elements.  Up to
  * HDIT_GEMM_MAX_PROBLEMS problems share one launch (the image and text streams
  * of a joint block, or q|k|v|mlp of a fused projection).
  *
