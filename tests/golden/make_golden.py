@@ -37,6 +37,7 @@ CASES = {
 
 
 def build(name):
+    reset_cache_manager()  # drop entries of earlier blocks; the new block registers its own below
     c = CASES[name]
     blk = getattr(blocks, c["cls"])(*c["args"], **c["kw"])
     synthetic.init_module_(blk, c["seed"])
@@ -76,7 +77,6 @@ def build(name):
         t = synthetic.randn_bf16((c["B"], c["kw"]["time_embed_dim"]), s + 3).float()
         hid, enc = oracle.cogvideox_block(params, x, e, t, (cos, sin), H)
         out.update(cos=cos, sin=sin, hidden_states=x, encoder_hidden_states=e, temb=t, out_hidden=hid, out_encoder=enc)
-    reset_cache_manager()
     return blk, params, {k: (v.numpy() if isinstance(v, torch.Tensor) else v) for k, v in out.items()}
 
 
