@@ -36,6 +36,8 @@
 // One launch covers up to HDIT_GEMM_MAX_PROBLEMS problems.  Tiles are dealt to
 // workgroups so that the workgroups of one XCD (workgroup id mod 8; each XCD
 // has a private L2) own a contiguous, 8-tile-row-grouped range.
+#include <type_traits>
+
 #include "hdit_common.h"
 
 namespace {
@@ -66,7 +68,8 @@ struct Cfg {
   static constexpr int A_BYTES = BM * ROW_BYTES;
   static constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
   static constexpr int EPI_OFF = STAGES * STAGE_BYTES;
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + NW * EPI_WAVE_BYTES;
+  static constexpr int BIAS_OFF = EPI_OFF + NW * EPI_WAVE_BYTES;  // one 1 KiB bias slot per wave
+  static constexpr int LDS_BYTES = BIAS_OFF + NW * 1024;
   static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile/waves mismatch");
   static_assert(TN <= 4, "epilogue staging window is 128 columns wide");
 };
@@ -202,6 +205,19 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
     for (int j = 0; j < TN; j++) fb[buf][j] = *(const bf16x8*)(sbase + b_off[ks] + j * 32 * ROW_BYTES);
   };
 
+  // Bias of a tile: every wave copies the 32*TN bias values of its own columns (8 per lane, lanes past the
+  // end clamped) into a private LDS slot when it starts the tile; the copy is older than the tile's slab
+  // copies, so the slab waits cover it.  A problem without bias copies from its B operand and ignores it,
+  // which keeps the number of outstanding copies per tile fixed.
+  const unsigned char* bias_slot = lds + C::BIAS_OFF + wave * 1024;
+  const unsigned bias_lds = __builtin_amdgcn_readfirstlane(lds_address(lds)) + C::BIAS_OFF + wave * 1024;
+  auto issue_bias = [&](const TileCoord& tc) {
+    const hdit_gemm_problem& pr = tab.p[tc.pi];
+    const unsigned char* src = pr.bias ? (const unsigned char*)pr.bias : (const unsigned char*)pr.b;
+    lds_dma16(src, (unsigned)(min(tc.n0 + wn0 + lane * 8, pr.n - 8) * 2), bias_lds);
+  };
+  issue_bias(locate<C>(tab, lid));
+
   p_setup();
 #pragma unroll 1
   for (int st = 0; st < STAGES - 1; st++) {
@@ -216,13 +232,18 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
   // wave-private epilogue staging window
   unsigned char* epi = lds + C::EPI_OFF + wave * EPI_WAVE_BYTES;
   constexpr int NMMA = TM * TN;
-  constexpr int L0 = (C::LOADS + 1) / 2;  // copies issued in k-step 0, the rest in k-step 1
-  constexpr int NR = (TM + TN < NMMA - 1) ? TM + TN : NMMA - 1;  // MFMAs that are followed by a fragment read
+  constexpr int NRD = TM + TN;            // fragment reads per k-step
+  constexpr int RD_MFMA = (NRD + 1) / 2;  // MFMAs that are followed by two fragment reads
+  constexpr int L0 = (C::LOADS + 1) / 2;  // copies issued under k-step 0, the rest under k-step 1
+  static_assert(RD_MFMA <= NMMA, "not enough MFMAs to place the fragment reads");
 
+  bool first_tile = true;
   while (true) {
     const TileCoord tc = locate<C>(tab, lid);
     const hdit_gemm_problem& pr = tab.p[tc.pi];
     const int KT = pr.k / BK;
+    if (!first_tile) issue_bias(tc);
+    first_tile = false;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -232,133 +253,156 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-    for (int kt = 0; kt < KT; kt++) {
-      const unsigned char* sbase = lds + stage * C::STAGE_BYTES;
-      const int pstage = (stage + STAGES - 1) & (STAGES - 1);  // freed by the previous slab's barrier
-      // ---- k-step 0: request the fragments of k-step 1 one per MFMA (an MFMA goes first, so that its
-      // wait for this step's fragments is placed while no younger read is outstanding and costs nothing),
-      // then one copy of slab h+3 per MFMA, then the remaining MFMAs
-      read_frags(sbase, 1, 1);
+    // One k-step: the MFMAs on fragment buffer `buf`.  Under them, pinned in this order: two reads per MFMA
+    // of the fragments the next k-step needs (an MFMA goes first, so that its wait for its own fragments
+    // is placed while no younger read is outstanding), then one copy of slab h+3 per MFMA, then the
+    // remaining MFMAs, which give the last read time to return.
+    auto k_step = [&](int buf, const unsigned char* rd_base, int rd_ks, int pstage, int cp_first, int cp_last) {
+      read_frags(rd_base, rd_ks, buf ^ 1);
 #pragma unroll
       for (int t = 0; t < NMMA; t++) {
         acc[t / TN][t % TN] =
-            __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][t % TN], fa[0][t / TN], acc[t / TN][t % TN], 0, 0, 0);
-        if (t == NR) {  // all fragment reads are placed: pin the order so far
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][t % TN], fa[buf][t / TN], acc[t / TN][t % TN], 0, 0, 0);
+        if (t == RD_MFMA - 1) {
 #pragma unroll
-          for (int u = 0; u < TM + TN; u++) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                // DS read
-            if (u < NR) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+          for (int u = 0; u < RD_MFMA; u++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                              // MFMA
+            if (2 * u + 2 <= NRD) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // DS reads
+            else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           }
           SCHED_FENCE();
         }
-        if (t > NR && t - NR - 1 < L0) {
-          p_issue_one(pstage, t - NR - 1);
+        if (t >= RD_MFMA && cp_first + (t - RD_MFMA) < cp_last) {
+          p_issue_one(pstage, cp_first + (t - RD_MFMA));
           SCHED_FENCE();
         }
       }
-      if (NMMA - 1 - NR < L0) p_issue(pstage, NMMA - 1 - NR, L0);  // tiles with fewer MFMAs than slots
+      if (cp_first + (NMMA - RD_MFMA) < cp_last) p_issue(pstage, cp_first + (NMMA - RD_MFMA), cp_last);
       SCHED_FENCE();
-      // ---- k-step 1, first part: the remaining copies, one per MFMA
-#pragma unroll
-      for (int t = 0; t < NMMA / 2; t++) {
-        acc[t / TN][t % TN] =
-            __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][t % TN], fa[1][t / TN], acc[t / TN][t % TN], 0, 0, 0);
-        if (t < C::LOADS - L0) {
-          p_issue_one(pstage, L0 + t);
-          SCHED_FENCE();
-        }
-      }
-      if (NMMA / 2 < C::LOADS - L0) p_issue(pstage, L0 + NMMA / 2, C::LOADS);
-      SCHED_FENCE();
-      p_advance();
-      // ---- turn the stages over: slab h+1 must have landed (h+2, h+3 may still be in flight; stores
-      // of an epilogue that are younger than those copies only make the wait conservative)
-      __builtin_amdgcn_s_waitcnt(0x0070 | ((2 * C::LOADS) & 15) | (((2 * C::LOADS) >> 4) << 14));
+    };
+
+    for (int kt = 0; kt < KT; kt++) {
+      const int pstage = (stage + STAGES - 1) & (STAGES - 1);  // freed by the previous slab's barrier
+      k_step(0, lds + stage * C::STAGE_BYTES, 1, pstage, 0, L0);
+      // ---- turn the stages over: every wave's copies of slab h+1 must have landed (slab h+2 and the L0
+      // copies of slab h+3 may still be in flight; stores of an epilogue that are younger than those
+      // copies only make the wait conservative), and the fragments read above must be in registers
+      __builtin_amdgcn_s_waitcnt(0x0070 | ((C::LOADS + L0) & 15) | (((C::LOADS + L0) >> 4) << 14));
       __syncthreads();
       stage = (stage + 1) & (STAGES - 1);
-      read_frags(lds + stage * C::STAGE_BYTES, 0, 0);
-      SCHED_FENCE();
-#pragma unroll
-      for (int i = TM / 2; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
-      SCHED_FENCE();
+      k_step(1, lds + stage * C::STAGE_BYTES, 0, pstage, L0, C::LOADS);
+      p_advance();
     }
 
     // ---- epilogue ---------------------------------------------------------
-    __bf16* __restrict__ Cp = (__bf16*)pr.c;
-    const __bf16* __restrict__ bias = (const __bf16*)pr.bias;
-    const __bf16* __restrict__ resid = (const __bf16*)pr.resid;
-    const float* __restrict__ gate = pr.gate;
-    const int epi_mode = pr.epilogue;
-    const int M = pr.m, N = pr.n;
-    const int64_t ldc = pr.ldc, ldr = pr.ldr;
-    const int ncol0 = tc.n0 + wn0;
+    if (KT < 3) __builtin_amdgcn_s_waitcnt(0x0f70);  // the bias copy is only known to have landed after three slab waits
+    auto epilogue = [&](auto mode_tag) {
+      constexpr int MODE = decltype(mode_tag)::value;
+      constexpr bool GATED = MODE == HDIT_EPI_GATE_RESIDUAL;
+      __bf16* __restrict__ Cp = (__bf16*)pr.c;
+      const __bf16* __restrict__ resid = (const __bf16*)pr.resid;
+      const float* __restrict__ gate = pr.gate;
+      const int M = pr.m, N = pr.n;
+      const int64_t ldc = pr.ldc, ldr = pr.ldr;
+      const int ncol0 = tc.n0 + wn0;
+
+      // this wave's bias columns, 8 per 16-byte chunk, from the slot its own copy filled at the start of the
+      // tile (zeros when the problem has no bias)
+      const int bias_mask = pr.bias ? -1 : 0;
+      i32x4 bia[TN * 2];
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-      const int mrow0 = tc.m0 + wm0 + i * 32;
-      const int m = mrow0 + l32;
-      const float* grow = nullptr;
-      if (epi_mode == HDIT_EPI_GATE_RESIDUAL) grow = gate + (int64_t)(min(m, M - 1) / pr.rows_per_batch) * pr.gate_stride;
+      for (int c = 0; c < TN * 2; c++) bia[c] = *(const i32x4*)(bias_slot + ((c * 2 + lh) << 4)) & bias_mask;
+
+      // Write-back layout: 16 lanes cover one 256-byte row segment, a wave covers 4 rows per pass, 8 passes
+      // per 32-row block.  The residual rows and the gate columns of a block are requested one block ahead,
+      // before the stores of the block in front of them: vector memory operations retire in order, so a load
+      // placed behind stores would wait for the stores' round trip.
+      const int rchunk = lane & 15;
+      const int wr_n = ncol0 + rchunk * 8;
+      const int wr_nc = min(wr_n, N - 8);
+      i32x4 rres[8];
+      f32x4 gte0, gte1;
+      bool straddle = false;
+      auto prefetch = [&](int i) {
+        const int mrow0 = tc.m0 + wm0 + i * 32;
 #pragma unroll
-      for (int j = 0; j < TN; j++) {
+        for (int it = 0; it < 8; it++) {
+          const int mm = min(mrow0 + it * 4 + (lane >> 4), M - 1);
+          rres[it] = *(const i32x4*)(resid + (int64_t)mm * ldr + wr_nc);
+        }
+        const int b_lo = min(mrow0, M - 1) / pr.rows_per_batch;
+        straddle = min(mrow0 + 31, M - 1) >= (b_lo + 1) * pr.rows_per_batch;
+        const float* g = gate + (int64_t)b_lo * pr.gate_stride + wr_nc;
+        gte0 = *(const f32x4*)g;
+        gte1 = *(const f32x4*)(g + 4);
+      };
+      if (GATED) prefetch(0);
+
 #pragma unroll
-        for (int gp = 0; gp < 2; gp++) {
-          // accumulator groups g = 2gp (even) and 2gp+1 (odd) hold columns 8g + 4*lh + e.  After the swap
-          // lanes < 32 own the 8 columns of the even group, lanes >= 32 those of the odd group.
-          float v[8];
+      for (int i = 0; i < TM; i++) {
+        const int mrow0 = tc.m0 + wm0 + i * 32;
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
-            auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(acc[i][j][(2 * gp) * 4 + e]),
-                                                       __float_as_int(acc[i][j][(2 * gp + 1) * 4 + e]), false, false);
-            v[e] = __int_as_float(sw[0]);
-            v[4 + e] = __int_as_float(sw[1]);
-          }
-          const int chunk = j * 4 + 2 * gp + lh;  // 16-byte chunk inside the wave's 256-byte row
-          const int n = min(ncol0 + chunk * 8, N - 8);
-          if (bias) {
-            float bf[8];
-            hdit::unpack8(*(const i32x4*)(bias + n), bf);
+        for (int j = 0; j < TN; j++) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) v[e] += bf[e];
-          }
-          if (epi_mode == HDIT_EPI_BIAS_GELU) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = hdit::gelu_tanh_f(v[e]);
-          } else if (epi_mode == HDIT_EPI_GATE_RESIDUAL) {
-            f32x4 g0 = *(const f32x4*)(grow + n), g1 = *(const f32x4*)(grow + n + 4);
+          for (int gp = 0; gp < 2; gp++) {
+            // accumulator groups g = 2gp (even) and 2gp+1 (odd) hold columns 8g + 4*lh + e.  After the swap
+            // lanes < 32 own the 8 columns of the even group, lanes >= 32 those of the odd group.
+            float v[8], bf[8];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-              v[e] *= g0[e];
-              v[4 + e] *= g1[e];
+              auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(acc[i][j][(2 * gp) * 4 + e]),
+                                                         __float_as_int(acc[i][j][(2 * gp + 1) * 4 + e]), false, false);
+              v[e] = __int_as_float(sw[0]);
+              v[4 + e] = __int_as_float(sw[1]);
             }
-          }
-          *(i32x4*)(epi + l32 * 256 + ((chunk ^ (l32 & 15)) << 4)) = hdit::pack8(v);
-        }
-      }
-      // coalesced write-back of this 32 x (32*TN) block: 16 lanes cover one row
-      const int rchunk = lane & 15;
+            const int chunk = j * 4 + 2 * gp + lh;  // 16-byte chunk inside the wave's 256-byte row
+            hdit::unpack8(bia[j * 2 + gp], bf);
 #pragma unroll
-      for (int it = 0; it < 8; it++) {
-        const int r = it * 4 + (lane >> 4);
-        const int mm = mrow0 + r;
-        const int nn = ncol0 + rchunk * 8;
-        i32x4 val = *(const i32x4*)(epi + r * 256 + ((rchunk ^ (r & 15)) << 4));
-        if (rchunk < 4 * TN && mm < M && nn < N) {
-          if (epi_mode == HDIT_EPI_GATE_RESIDUAL) {
+            for (int e = 0; e < 8; e++) v[e] += bf[e];
+            if (MODE == HDIT_EPI_BIAS_GELU) {
+#pragma unroll
+              for (int e = 0; e < 8; e++) v[e] = hdit::gelu_tanh_f(v[e]);
+            }
+            *(i32x4*)(epi + l32 * 256 + ((chunk ^ (l32 & 15)) << 4)) = hdit::pack8(v);
+          }
+        }
+        // coalesced write-back of this 32 x (32*TN) block
+        i32x4 outv[8];
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+          const int r = it * 4 + (lane >> 4);
+          i32x4 val = *(const i32x4*)(epi + r * 256 + ((rchunk ^ (r & 15)) << 4));
+          if (GATED) {
+            f32x4 g0 = gte0, g1 = gte1;
+            if (straddle) {  // rows of this block belong to different batch elements: fetch the gate per row
+              const int mm = min(mrow0 + r, M - 1);
+              const float* g = gate + (int64_t)(mm / pr.rows_per_batch) * pr.gate_stride + wr_nc;
+              g0 = *(const f32x4*)g;
+              g1 = *(const f32x4*)(g + 4);
+            }
             float u[8], rf[8];
             hdit::unpack8(val, u);
-            hdit::unpack8(*(const i32x4*)(resid + (int64_t)mm * ldr + nn), rf);
+            hdit::unpack8(rres[it], rf);
 #pragma unroll
-            for (int e = 0; e < 8; e++) u[e] += rf[e];
+            for (int e = 0; e < 4; e++) {
+              u[e] = __builtin_fmaf(g0[e], u[e], rf[e]);
+              u[4 + e] = __builtin_fmaf(g1[e], u[4 + e], rf[4 + e]);
+            }
             val = hdit::pack8(u);
           }
-          *(i32x4*)(Cp + (int64_t)mm * ldc + nn) = val;
+          outv[it] = val;
+        }
+        if (GATED && i + 1 < TM) prefetch(i + 1);
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+          const int mm = mrow0 + it * 4 + (lane >> 4);
+          if (rchunk < 4 * TN && mm < M && wr_n < N) *(i32x4*)(Cp + (int64_t)mm * ldc + wr_n) = outv[it];
         }
       }
-    }
+    };
+    if (pr.epilogue == HDIT_EPI_BIAS) epilogue(std::integral_constant<int, HDIT_EPI_BIAS>{});
+    else if (pr.epilogue == HDIT_EPI_BIAS_GELU) epilogue(std::integral_constant<int, HDIT_EPI_BIAS_GELU>{});
+    else epilogue(std::integral_constant<int, HDIT_EPI_GATE_RESIDUAL>{});
 
     lid += wgs_per_xcd;
     if (lid >= xcd_end) break;
@@ -416,7 +460,6 @@ int build_and_launch(const hdit_gemm_problem* problems, int count, hipStream_t s
   return launch<C>(tab, total, stream);
 }
 
-using Cfg256x256 = Cfg<4, 4>;
 using Cfg256x192 = Cfg<4, 3>;
 using Cfg128x256 = Cfg<2, 4>;
 using Cfg128x128 = Cfg<2, 2>;
@@ -461,20 +504,17 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
   hipStream_t s = (hipStream_t)stream;
   int cfg = g_force_cfg;
   if (cfg < 0) {
-    const double c0 = launch_cost<Cfg256x256>(live, nlive, 1.00, 256);
-    const double c1 = launch_cost<Cfg256x192>(live, nlive, 1.05, 256);
-    const double c2 = launch_cost<Cfg128x256>(live, nlive, 1.08, 256);
-    const double c3 = launch_cost<Cfg128x128>(live, nlive, 1.30, 256);
+    const double c0 = launch_cost<Cfg256x192>(live, nlive, 1.00, 256);
+    const double c1 = launch_cost<Cfg128x256>(live, nlive, 1.03, 256);
+    const double c2 = launch_cost<Cfg128x128>(live, nlive, 1.24, 256);
     cfg = 0;
     double best = c0;
     if (c1 < best) best = c1, cfg = 1;
     if (c2 < best) best = c2, cfg = 2;
-    if (c3 < best) best = c3, cfg = 3;
   }
   switch (cfg) {
-    case 0: return build_and_launch<Cfg256x256>(live, nlive, s);
-    case 1: return build_and_launch<Cfg256x192>(live, nlive, s);
-    case 2: return build_and_launch<Cfg128x256>(live, nlive, s);
+    case 0: return build_and_launch<Cfg256x192>(live, nlive, s);
+    case 1: return build_and_launch<Cfg128x256>(live, nlive, s);
     default: return build_and_launch<Cfg128x128>(live, nlive, s);
   }
 }
