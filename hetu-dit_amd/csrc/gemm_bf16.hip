@@ -5,33 +5,32 @@
 // (32*TM) x (32*TN) sub-tile in accumulators (v_mfma_f32_32x32x16_bf16).
 //
 // Staging.  Both operands are k-contiguous, so A and B tiles are staged the
-// same way: `global_load_lds_dwordx4` copies 32-wide k slabs straight from
-// global memory into LDS (no VGPR staging, no ds_write).  A wave-wide direct
-// load writes 1 KiB of LDS in lane order = 16 rows x 64 bytes.  The XOR swizzle
-// that keeps the ds_read_b128 fragment reads conflict-free is applied on the
-// global side: the lane that fills 16-byte slot p of row r fetches chunk
-// p ^ ((r>>2)&3) of that row's 64-byte slab, so the global access stays
-// coalesced, and the 16 rows one ds_read_b128 pass touches land on 16 distinct
-// 16-byte slots of the 256-byte LDS bank window (a linear pattern measured
-// 202 B/clk/CU, a 2-way conflicting one 117 B/clk).
+// same way, in slabs of 64 k (128 bytes per row).  A wave-wide global load
+// fetches 8 rows x 128 bytes, eight lanes per row: every request covers whole
+// 128-byte cache lines (64-byte row pieces were measured at half the L2->CU
+// rate, 29 B/clk/CU against 58).  The data waits in registers for one slab time
+// and is then written to LDS with ds_write_b128 into rows of 128 bytes whose
+// 16-byte chunks are XOR-swizzled with (row>>1)&7: the 16 lanes of a
+// ds_read_b128 pass (16 rows, one chunk) and of a ds_write_b128 pass (2 rows,
+// 8 chunks) then land on 16 distinct 16-byte slots of the 256-byte bank window.
 //
 // Pipeline.  The k slabs of all tiles of a workgroup form one flat stream over
-// four LDS stages.  While slab h is multiplied, slabs h+1 and h+2 have landed
-// or are landing and the copies of slab h+3 are issued a few at a time between
-// the MFMAs (a burst of copies starves the fragment reads).  In the last
-// k-step of slab h every wave waits for its own copies of slab h+1, the
-// workgroup barrier makes that slab visible and proves stage(h) free, and the
-// first fragments of slab h+1 are read under the remaining MFMAs of slab h.
-// Fragments are double-buffered in registers one k-step ahead.  Tile
+// two LDS stages.  While slab h is multiplied out of stage h&1, the registers
+// holding slab h+1 are written to the other stage and immediately refilled
+// with the global loads of slab h+2, one write+load pair every few MFMAs (the
+// loads have a whole slab time to arrive).  Fragments are double-buffered in
+// registers one k-step ahead; the workgroup barrier sits before the last
+// k-step of a slab, whose fragments are already in registers, so that the
+// first fragments of slab h+1 are read under that k-step's MFMAs.  Tile
 // boundaries are invisible to the stream, so a tile's first slabs arrive
-// during the previous tile's last slabs and epilogue.
+// during the previous tile's last slab and epilogue.
 //
 // Epilogue.  A lane's accumulator holds one output row m and runs of 4
 // consecutive n; lanes l and l^32 swap halves (v_permlane32_swap) to own 8
-// consecutive n.  bias / GELU-tanh / gate are applied there, the bf16 result is
-// staged through a wave-private 8 KiB LDS window and written back with 16
-// lanes covering 256 contiguous bytes of a row (the residual is read in that
-// same coalesced layout and added in fp32 before the final rounding).
+// consecutive n.  bias / GELU-tanh are applied there, the bf16 result is staged
+// through a wave-private 8 KiB window inside the LDS stage the last slab just
+// vacated and written back with 16 lanes covering 256 contiguous bytes of a row
+// (gate and residual are applied in that coalesced layout, in fp32).
 //
 // One launch covers up to HDIT_GEMM_MAX_PROBLEMS problems.  Tiles are dealt to
 // workgroups so that the workgroups of one XCD (workgroup id mod 8; each XCD
@@ -42,9 +41,8 @@
 
 namespace {
 
-constexpr int BK = 32;         // k elements per LDS stage
-constexpr int ROW_BYTES = 64;  // BK * sizeof(bf16)
-constexpr int STAGES = 4;
+constexpr int BK = 64;           // k elements per LDS stage
+constexpr int ROW_BYTES = 128;   // BK * sizeof(bf16)
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 8;
 constexpr int NW = 4;
@@ -62,15 +60,14 @@ struct Cfg {
   static constexpr int TM = TM_, TN = TN_;
   static constexpr int BM = 64 * TM, BN = 64 * TN;
   static constexpr int WM = 32 * TM, WN = 32 * TN;
-  static constexpr int A_LOADS = BM / 16 / NW;  // direct-to-LDS wave loads per wave per slab (16 rows each)
-  static constexpr int B_LOADS = BN / 16 / NW;
+  static constexpr int A_LOADS = BM / 8 / NW;  // wave-wide loads (8 rows x 128 bytes) per wave per slab
+  static constexpr int B_LOADS = BN / 8 / NW;
   static constexpr int LOADS = A_LOADS + B_LOADS;
   static constexpr int A_BYTES = BM * ROW_BYTES;
   static constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
-  static constexpr int EPI_OFF = STAGES * STAGE_BYTES;
-  static constexpr int BIAS_OFF = EPI_OFF + NW * EPI_WAVE_BYTES;  // one 1 KiB bias slot per wave
+  static constexpr int BIAS_OFF = 2 * STAGE_BYTES;  // one 1 KiB bias slot per wave
   static constexpr int LDS_BYTES = BIAS_OFF + NW * 1024;
-  static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile/waves mismatch");
+  static_assert(NW * EPI_WAVE_BYTES <= STAGE_BYTES, "the epilogue windows live inside one stage");
   static_assert(TN <= 4, "epilogue staging window is 128 columns wide");
 };
 
@@ -97,10 +94,9 @@ __device__ __forceinline__ TileCoord locate(const GemmTable& tab, int lid) {
 }
 
 // One wave-wide direct-to-LDS copy: lane l's 16 bytes at base + voff land at LDS byte address
-// lds_addr + 16*l.  Written as inline assembly on purpose: the compiler's wait-count insertion treats a
-// `__builtin_amdgcn_global_load_lds` as a pending write to all of LDS and forces vmcnt(0) before the next
-// ds_read, which would drain the whole copy pipeline at every slab; here the copies are only ever
-// waited for with the explicit s_waitcnt before the workgroup barrier.
+// lds_addr + 16*l.  Only used for the bias slots.  Inline assembly, so the compiler's wait-count
+// insertion does not see it: an extra operation in flight only makes the waits it computes for its own
+// loads stricter than needed.
 __device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
@@ -134,17 +130,21 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
   int lid = xcd_begin + blockIdx.x / NUM_XCD;
   if (lid >= xcd_end) return;
 
-  // ---- producer: the slab stream, three slabs ahead of the MFMAs -------------
-  // Lane-constant parts of a direct-to-LDS copy: row-in-group l/4; the chunk a lane fetches is
-  // (l%4) ^ ((row>>2)&3) with row = 16*grp + l/4, i.e. (l%4) ^ ((l>>4)&3).
-  const int ld_row = lane >> 2;
-  const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+  // ---- producer: the slab stream, two slabs ahead of the MFMAs ------------------
+  // A wave-wide load covers rows 8*(wave + NW*i) + lane/8 of the A (or B) tile, chunk lane%8 of the row's
+  // 128-byte slab.  Its LDS destination is row*128 + ((chunk ^ ((row>>1)&7)) << 4); (row>>1)&7 does not
+  // depend on i, so the destinations of one lane differ by the constant NW*8*128 bytes.
+  const int ld_row = lane >> 3;
+  const int ld_chunk = lane & 7;
+  const int st_row = wave * 8 + ld_row;
+  const int st_off = st_row * ROW_BYTES + ((ld_chunk ^ ((st_row >> 1) & 7)) << 4);
   int p_lid = lid;
   bool p_valid = true;
   int p_kt = 0, p_KT = 0;
   const unsigned char* p_abase = nullptr;
   const unsigned char* p_bbase = nullptr;
   unsigned p_off[C::LOADS];
+  i32x4 G[C::LOADS];  // the slab in flight between global memory and LDS
   auto p_setup = [&]() {
     const TileCoord tc = locate<C>(tab, p_lid);
     const hdit_gemm_problem& pr = tab.p[tc.pi];
@@ -154,28 +154,24 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
     p_kt = 0;
 #pragma unroll
     for (int i = 0; i < C::A_LOADS; i++) {
-      const int gr = min(tc.m0 + (wave + i * NW) * 16 + ld_row, pr.m - 1);
+      const int gr = min(tc.m0 + (wave + i * NW) * 8 + ld_row, pr.m - 1);
       p_off[i] = (unsigned)(((int64_t)gr * pr.lda + ld_chunk * 8) * 2);
     }
 #pragma unroll
     for (int i = 0; i < C::B_LOADS; i++) {
-      const int gr = min(tc.n0 + (wave + i * NW) * 16 + ld_row, pr.n - 1);
+      const int gr = min(tc.n0 + (wave + i * NW) * 8 + ld_row, pr.n - 1);
       p_off[C::A_LOADS + i] = (unsigned)(((int64_t)gr * pr.ldb + ld_chunk * 8) * 2);
     }
   };
-  // copies [first, last) of the current producer slab into `stage`.  Unconditional (no branch may split
-  // the MFMA stream it is interleaved with): once the stream is exhausted the last slab is simply copied
-  // again into a stage nobody will read.
-  const unsigned lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds)) + wave * 1024;
-  auto p_issue_one = [&](int stage, int i) {
-    const unsigned dst = lds0 + stage * C::STAGE_BYTES;
-    if (i < C::A_LOADS) lds_dma16(p_abase + (size_t)p_kt * ROW_BYTES, p_off[i], dst + i * NW * 1024);
-    else lds_dma16(p_bbase + (size_t)p_kt * ROW_BYTES, p_off[i], dst + C::A_BYTES + (i - C::A_LOADS) * NW * 1024);
+  // Once the stream is exhausted the last slab is simply loaded again and written to a stage nobody
+  // reads: no branch may split the MFMA stream the loads are interleaved with.
+  auto g_load = [&](int i) {
+    const unsigned char* base = (i < C::A_LOADS ? p_abase : p_bbase) + (size_t)p_kt * ROW_BYTES;
+    G[i] = *(const i32x4*)(base + p_off[i]);
   };
-  auto p_issue = [&](int stage, int first, int last) {
-#pragma unroll
-    for (int i = 0; i < C::LOADS; i++)
-      if (i >= first && i < last) p_issue_one(stage, i);
+  auto l_store = [&](int stage, int i) {
+    const int tile_off = i < C::A_LOADS ? i * (NW * 8 * ROW_BYTES) : C::A_BYTES + (i - C::A_LOADS) * (NW * 8 * ROW_BYTES);
+    *(i32x4*)(lds + stage * C::STAGE_BYTES + tile_off + st_off) = G[i];
   };
   auto p_advance = [&]() {
     if (!p_valid) return;
@@ -188,27 +184,24 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
   };
 
   // ---- consumer ------------------------------------------------------------
-  // fragment read offsets: row r, logical chunk c -> r*64 + ((c ^ ((r>>2)&3)) << 4); fragment rows are
-  // l32 plus a multiple of 32, so (r>>2)&3 == (l32>>2)&3
-  const int swz = (l32 >> 2) & 3;
-  int a_off[2], b_off[2];  // per k-step (chunk = 2*ks + lh)
-#pragma unroll
-  for (int ks = 0; ks < 2; ks++) {
-    a_off[ks] = (wm0 + l32) * ROW_BYTES + (((ks * 2 + lh) ^ swz) << 4);
-    b_off[ks] = C::A_BYTES + (wn0 + l32) * ROW_BYTES + (((ks * 2 + lh) ^ swz) << 4);
-  }
+  // fragment read offsets: row r, logical chunk c -> r*128 + ((c ^ ((r>>1)&7)) << 4); fragment rows are
+  // l32 plus a multiple of 32, so (r>>1)&7 == (l32>>1)&7.  k-step ks uses chunk 2*ks + lh.
+  const int swz = (l32 >> 1) & 7;
+  const int a_row = (wm0 + l32) * ROW_BYTES;
+  const int b_row = C::A_BYTES + (wn0 + l32) * ROW_BYTES;
   bf16x8 fa[2][TM], fb[2][TN];
   auto read_frags = [&](const unsigned char* sbase, int ks, int buf) {
+    const int ch = ((ks * 2 + lh) ^ swz) << 4;
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[buf][i] = *(const bf16x8*)(sbase + a_off[ks] + i * 32 * ROW_BYTES);
+    for (int i = 0; i < TM; i++) fa[buf][i] = *(const bf16x8*)(sbase + a_row + ch + i * 32 * ROW_BYTES);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb[buf][j] = *(const bf16x8*)(sbase + b_off[ks] + j * 32 * ROW_BYTES);
+    for (int j = 0; j < TN; j++) fb[buf][j] = *(const bf16x8*)(sbase + b_row + ch + j * 32 * ROW_BYTES);
   };
 
   // Bias of a tile: every wave copies the 32*TN bias values of its own columns (8 per lane, lanes past the
-  // end clamped) into a private LDS slot when it starts the tile; the copy is older than the tile's slab
-  // copies, so the slab waits cover it.  A problem without bias copies from its B operand and ignores it,
-  // which keeps the number of outstanding copies per tile fixed.
+  // end clamped) into a private LDS slot when it starts the tile; the copy is older than the loads of the
+  // tile's second slab, so the waits for those cover it.  A problem without bias copies from its B
+  // operand and ignores the result.
   const unsigned char* bias_slot = lds + C::BIAS_OFF + wave * 1024;
   const unsigned bias_lds = __builtin_amdgcn_readfirstlane(lds_address(lds)) + C::BIAS_OFF + wave * 1024;
   auto issue_bias = [&](const TileCoord& tc) {
@@ -218,31 +211,36 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
   };
   issue_bias(locate<C>(tab, lid));
 
+  // prologue: slab 0 into stage 0, slab 1 into the registers
   p_setup();
-#pragma unroll 1
-  for (int st = 0; st < STAGES - 1; st++) {
-    p_issue(st, 0, C::LOADS);
-    p_advance();
-  }
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+#pragma unroll
+  for (int i = 0; i < C::LOADS; i++) g_load(i);
+  p_advance();
+#pragma unroll
+  for (int i = 0; i < C::LOADS; i++) l_store(0, i);
+#pragma unroll
+  for (int i = 0; i < C::LOADS; i++) g_load(i);
+  p_advance();
   __syncthreads();
   int stage = 0;
   read_frags(lds, 0, 0);
 
-  // wave-private epilogue staging window
-  unsigned char* epi = lds + C::EPI_OFF + wave * EPI_WAVE_BYTES;
   constexpr int NMMA = TM * TN;
   constexpr int NRD = TM + TN;            // fragment reads per k-step
   constexpr int RD_MFMA = (NRD + 1) / 2;  // MFMAs that are followed by two fragment reads
-  constexpr int L0 = (C::LOADS + 1) / 2;  // copies issued under k-step 0, the rest under k-step 1
-  static_assert(RD_MFMA <= NMMA, "not enough MFMAs to place the fragment reads");
+  constexpr int SLOTS = NMMA - RD_MFMA;   // MFMAs per k-step that can carry a write+load pair
+  constexpr int CP = (C::LOADS + 2) / 3;  // pairs per k-step (k-steps 0..2 of a slab)
+  static_assert(RD_MFMA < NMMA, "not enough MFMAs to place the fragment reads");
 
   bool first_tile = true;
   while (true) {
     const TileCoord tc = locate<C>(tab, lid);
     const hdit_gemm_problem& pr = tab.p[tc.pi];
     const int KT = pr.k / BK;
-    if (!first_tile) issue_bias(tc);
+    if (!first_tile) {
+      __syncthreads();  // every wave has left the previous epilogue, whose staging windows the next writes reuse
+      issue_bias(tc);
+    }
     first_tile = false;
 
     f32x16 acc[TM][TN];
@@ -255,9 +253,10 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
 
     // One k-step: the MFMAs on fragment buffer `buf`.  Under them, pinned in this order: two reads per MFMA
     // of the fragments the next k-step needs (an MFMA goes first, so that its wait for its own fragments
-    // is placed while no younger read is outstanding), then one copy of slab h+3 per MFMA, then the
-    // remaining MFMAs, which give the last read time to return.
-    auto k_step = [&](int buf, const unsigned char* rd_base, int rd_ks, int pstage, int cp_first, int cp_last) {
+    // is placed while no younger read is outstanding), then the write+load pairs [cp_first, cp_last)
+    // spread over the remaining MFMAs: registers of slab h+1 to LDS stage `wstage`, then the same
+    // registers refilled with slab h+2.
+    auto k_step = [&](int buf, const unsigned char* rd_base, int rd_ks, int wstage, int cp_first, int cp_last) {
       read_frags(rd_base, rd_ks, buf ^ 1);
 #pragma unroll
       for (int t = 0; t < NMMA; t++) {
@@ -266,77 +265,86 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
         if (t == RD_MFMA - 1) {
 #pragma unroll
           for (int u = 0; u < RD_MFMA; u++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                              // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // MFMA
             if (2 * u + 2 <= NRD) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // DS reads
             else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           }
           SCHED_FENCE();
         }
-        if (t >= RD_MFMA && cp_first + (t - RD_MFMA) < cp_last) {
-          p_issue_one(pstage, cp_first + (t - RD_MFMA));
+        if (t >= RD_MFMA) {
+#pragma unroll
+          for (int j = 0; j < CP; j++)
+            if (RD_MFMA + (j * SLOTS) / CP == t && cp_first + j < cp_last) {
+              l_store(wstage, cp_first + j);
+              g_load(cp_first + j);
+            }
           SCHED_FENCE();
         }
       }
-      if (cp_first + (NMMA - RD_MFMA) < cp_last) p_issue(pstage, cp_first + (NMMA - RD_MFMA), cp_last);
-      SCHED_FENCE();
     };
 
     for (int kt = 0; kt < KT; kt++) {
-      const int pstage = (stage + STAGES - 1) & (STAGES - 1);  // freed by the previous slab's barrier
-      k_step(0, lds + stage * C::STAGE_BYTES, 1, pstage, 0, L0);
-      // ---- turn the stages over: every wave's copies of slab h+1 must have landed (slab h+2 and the L0
-      // copies of slab h+3 may still be in flight; stores of an epilogue that are younger than those
-      // copies only make the wait conservative), and the fragments read above must be in registers
-      __builtin_amdgcn_s_waitcnt(0x0070 | ((C::LOADS + L0) & 15) | (((C::LOADS + L0) >> 4) << 14));
-      __syncthreads();
-      stage = (stage + 1) & (STAGES - 1);
-      k_step(1, lds + stage * C::STAGE_BYTES, 0, pstage, L0, C::LOADS);
+      const unsigned char* sbase = lds + stage * C::STAGE_BYTES;
+      const int wstage = stage ^ 1;  // held slab h-1; every wave passed the barrier of that slab
+      k_step(0, sbase, 1, wstage, 0, CP);
+      k_step(1, sbase, 2, wstage, CP, 2 * CP);
+      k_step(0, sbase, 3, wstage, 2 * CP, C::LOADS);
       p_advance();
+      // ---- turn the stages over: the fragments of the last k-step are in registers, slab h+1 is written
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      __syncthreads();
+      stage ^= 1;
+      k_step(1, lds + stage * C::STAGE_BYTES, 0, wstage, 0, 0);
     }
+    unsigned char* epi = lds + (stage ^ 1) * C::STAGE_BYTES + wave * EPI_WAVE_BYTES;  // the stage just vacated
 
     // ---- epilogue ---------------------------------------------------------
-    if (KT < 3) __builtin_amdgcn_s_waitcnt(0x0f70);  // the bias copy is only known to have landed after three slab waits
+    if (KT < 2) __builtin_amdgcn_s_waitcnt(0x0f70);  // the bias copy is only known to have landed after the second slab's loads
     auto epilogue = [&](auto mode_tag) {
       constexpr int MODE = decltype(mode_tag)::value;
       constexpr bool GATED = MODE == HDIT_EPI_GATE_RESIDUAL;
-      __bf16* __restrict__ Cp = (__bf16*)pr.c;
-      const __bf16* __restrict__ resid = (const __bf16*)pr.resid;
+      // all addressing below is a uniform base plus a 32-bit byte offset per lane (checked on the host)
+      unsigned char* __restrict__ Cb = (unsigned char*)pr.c;
+      const unsigned char* __restrict__ Rb = (const unsigned char*)pr.resid;
       const float* __restrict__ gate = pr.gate;
       const int M = pr.m, N = pr.n;
-      const int64_t ldc = pr.ldc, ldr = pr.ldr;
+      const int ldc = (int)pr.ldc, ldr = (int)pr.ldr;
       const int ncol0 = tc.n0 + wn0;
-
-      // this wave's bias columns, 8 per 16-byte chunk, from the slot its own copy filled at the start of the
-      // tile (zeros when the problem has no bias)
-      const int bias_mask = pr.bias ? -1 : 0;
-      i32x4 bia[TN * 2];
-#pragma unroll
-      for (int c = 0; c < TN * 2; c++) bia[c] = *(const i32x4*)(bias_slot + ((c * 2 + lh) << 4)) & bias_mask;
+      const int bias_mask = pr.bias ? -1 : 0;  // the slot holds unrelated data when the problem has no bias
 
       // Write-back layout: 16 lanes cover one 256-byte row segment, a wave covers 4 rows per pass, 8 passes
-      // per 32-row block.  The residual rows and the gate columns of a block are requested one block ahead,
-      // before the stores of the block in front of them: vector memory operations retire in order, so a load
+      // per 32-row block, done as two halves of 4.  The residual rows and the gate columns are requested one
+      // block ahead, before the stores in front of them: vector memory operations retire in order, so a load
       // placed behind stores would wait for the stores' round trip.
       const int rchunk = lane & 15;
+      const int wr_row = lane >> 4;
       const int wr_n = ncol0 + rchunk * 8;
       const int wr_nc = min(wr_n, N - 8);
+      const bool wr_ok = rchunk < 4 * TN && wr_n < N;
       i32x4 rres[8];
       f32x4 gte0, gte1;
       bool straddle = false;
-      auto prefetch = [&](int i) {
+      auto prefetch_rows = [&](int i, int half) {
         const int mrow0 = tc.m0 + wm0 + i * 32;
 #pragma unroll
-        for (int it = 0; it < 8; it++) {
-          const int mm = min(mrow0 + it * 4 + (lane >> 4), M - 1);
-          rres[it] = *(const i32x4*)(resid + (int64_t)mm * ldr + wr_nc);
+        for (int it = half * 4; it < half * 4 + 4; it++) {
+          const int mm = min(mrow0 + it * 4 + wr_row, M - 1);
+          rres[it] = *(const i32x4*)(Rb + (unsigned)((mm * ldr + wr_nc) * 2));
         }
+      };
+      auto prefetch_gate = [&](int i) {
+        const int mrow0 = tc.m0 + wm0 + i * 32;
         const int b_lo = min(mrow0, M - 1) / pr.rows_per_batch;
         straddle = min(mrow0 + 31, M - 1) >= (b_lo + 1) * pr.rows_per_batch;
         const float* g = gate + (int64_t)b_lo * pr.gate_stride + wr_nc;
         gte0 = *(const f32x4*)g;
         gte1 = *(const f32x4*)(g + 4);
       };
-      if (GATED) prefetch(0);
+      if (GATED) {
+        prefetch_rows(0, 0);
+        prefetch_rows(0, 1);
+        prefetch_gate(0);
+      }
 
 #pragma unroll
       for (int i = 0; i < TM; i++) {
@@ -356,7 +364,7 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
               v[4 + e] = __int_as_float(sw[1]);
             }
             const int chunk = j * 4 + 2 * gp + lh;  // 16-byte chunk inside the wave's 256-byte row
-            hdit::unpack8(bia[j * 2 + gp], bf);
+            hdit::unpack8(*(const i32x4*)(bias_slot + (chunk << 4)) & bias_mask, bf);
 #pragma unroll
             for (int e = 0; e < 8; e++) v[e] += bf[e];
             if (MODE == HDIT_EPI_BIAS_GELU) {
@@ -365,38 +373,48 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
             }
             *(i32x4*)(epi + l32 * 256 + ((chunk ^ (l32 & 15)) << 4)) = hdit::pack8(v);
           }
+          SCHED_FENCE();  // keeps the scheduler from pulling whole accumulator tiles into VGPRs at once
         }
         // coalesced write-back of this 32 x (32*TN) block
-        i32x4 outv[8];
 #pragma unroll
-        for (int it = 0; it < 8; it++) {
-          const int r = it * 4 + (lane >> 4);
-          i32x4 val = *(const i32x4*)(epi + r * 256 + ((rchunk ^ (r & 15)) << 4));
-          if (GATED) {
-            f32x4 g0 = gte0, g1 = gte1;
-            if (straddle) {  // rows of this block belong to different batch elements: fetch the gate per row
-              const int mm = min(mrow0 + r, M - 1);
-              const float* g = gate + (int64_t)(mm / pr.rows_per_batch) * pr.gate_stride + wr_nc;
-              g0 = *(const f32x4*)g;
-              g1 = *(const f32x4*)(g + 4);
-            }
-            float u[8], rf[8];
-            hdit::unpack8(val, u);
-            hdit::unpack8(rres[it], rf);
+        for (int half = 0; half < 2; half++) {
+          i32x4 outv[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-              u[e] = __builtin_fmaf(g0[e], u[e], rf[e]);
-              u[4 + e] = __builtin_fmaf(g1[e], u[4 + e], rf[4 + e]);
+          for (int q = 0; q < 4; q++) {
+            const int it = half * 4 + q;
+            const int r = it * 4 + wr_row;
+            i32x4 val = *(const i32x4*)(epi + r * 256 + ((rchunk ^ (r & 15)) << 4));
+            if (GATED) {
+              f32x4 g0 = gte0, g1 = gte1;
+              if (straddle) {  // rows of this block belong to different batch elements: fetch the gate per row
+                const int mm = min(mrow0 + r, M - 1);
+                const float* g = gate + (int64_t)(mm / pr.rows_per_batch) * pr.gate_stride + wr_nc;
+                g0 = *(const f32x4*)g;
+                g1 = *(const f32x4*)(g + 4);
+              }
+              float u[8], rf[8];
+              hdit::unpack8(val, u);
+              hdit::unpack8(rres[it], rf);
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                u[e] = __builtin_fmaf(g0[e], u[e], rf[e]);
+                u[4 + e] = __builtin_fmaf(g1[e], u[4 + e], rf[4 + e]);
+              }
+              val = hdit::pack8(u);
             }
-            val = hdit::pack8(u);
+            outv[q] = val;
           }
-          outv[it] = val;
-        }
-        if (GATED && i + 1 < TM) prefetch(i + 1);
+          SCHED_FENCE();
+          if (GATED && i + 1 < TM) {
+            prefetch_rows(i + 1, half);
+            if (half == 1) prefetch_gate(i + 1);
+          }
 #pragma unroll
-        for (int it = 0; it < 8; it++) {
-          const int mm = mrow0 + it * 4 + (lane >> 4);
-          if (rchunk < 4 * TN && mm < M && wr_n < N) *(i32x4*)(Cp + (int64_t)mm * ldc + wr_n) = outv[it];
+          for (int q = 0; q < 4; q++) {
+            const int mm = mrow0 + (half * 4 + q) * 4 + wr_row;
+            if (wr_ok && mm < M) *(i32x4*)(Cb + (unsigned)((mm * ldc + wr_n) * 2)) = outv[q];
+          }
+          SCHED_FENCE();
         }
       }
     };
@@ -426,8 +444,7 @@ int launch(const GemmTable& tab, int total_tiles, hipStream_t stream) {
     }
     attr_set = true;
   }
-  const int per_cu = (2 * C::LDS_BYTES <= 160 * 1024) ? 2 : 1;
-  int max_wgs = (num_cus * per_cu) / NUM_XCD * NUM_XCD;
+  int max_wgs = num_cus / NUM_XCD * NUM_XCD;  // one workgroup per CU: a wave may use the whole register file
   if (max_wgs < NUM_XCD) max_wgs = NUM_XCD;
   const int tiles_per_xcd = (total_tiles + NUM_XCD - 1) / NUM_XCD;
   int wgs_per_xcd = max_wgs / NUM_XCD;
@@ -460,6 +477,7 @@ int build_and_launch(const hdit_gemm_problem* problems, int count, hipStream_t s
   return launch<C>(tab, total, stream);
 }
 
+using Cfg256x256 = Cfg<4, 4>;
 using Cfg256x192 = Cfg<4, 3>;
 using Cfg128x256 = Cfg<2, 4>;
 using Cfg128x128 = Cfg<2, 2>;
@@ -491,11 +509,13 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
     if (p.k % BK != 0 || p.n % 8 != 0) return HDIT_EUNSUPPORTED;
     if (p.lda % 8 || p.ldb % 8 || p.ldc % 8) return HDIT_EINVAL;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uintptr_t)p.c | (uintptr_t)p.bias) & 15) return HDIT_EINVAL;
-    // the direct-to-LDS copies address rows with 32-bit byte offsets from the operand base
+    // rows are addressed with 32-bit byte offsets from the operand base
     if ((int64_t)p.m * p.lda * 2 >= (1ll << 32) || (int64_t)p.n * p.ldb * 2 >= (1ll << 32)) return HDIT_EUNSUPPORTED;
+    if ((int64_t)p.m * p.ldc * 2 >= (1ll << 31)) return HDIT_EUNSUPPORTED;
     if (p.epilogue < HDIT_EPI_BIAS || p.epilogue > HDIT_EPI_GATE_RESIDUAL) return HDIT_EINVAL;
     if (p.epilogue == HDIT_EPI_GATE_RESIDUAL) {
       if (!p.resid || !p.gate || p.rows_per_batch <= 0 || p.ldr % 8) return HDIT_EINVAL;
+      if ((int64_t)p.m * p.ldr * 2 >= (1ll << 31)) return HDIT_EUNSUPPORTED;
       if (((uintptr_t)p.resid & 15) || ((uintptr_t)p.gate & 15) || p.gate_stride % 4) return HDIT_EINVAL;
     }
     live[nlive++] = p;
@@ -515,6 +535,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
   switch (cfg) {
     case 0: return build_and_launch<Cfg256x192>(live, nlive, s);
     case 1: return build_and_launch<Cfg128x256>(live, nlive, s);
+    case 3: return build_and_launch<Cfg256x256>(live, nlive, s);
     default: return build_and_launch<Cfg128x128>(live, nlive, s);
   }
 }
