@@ -484,13 +484,43 @@ using Cfg128x128 = Cfg<2, 2>;
 
 int g_force_cfg = -1;
 
-// Relative cost of a launch with a given tile shape on 256 CUs: rounds of tiles times the time of one tile
-// (proportional to its area; smaller tiles pay more per flop for fragment traffic and epilogue).
-template <class C>
-double launch_cost(const hdit_gemm_problem* problems, int count, double per_flop_penalty, int slots) {
-  const int tiles = count_tiles<C>(problems, count);
-  const int rounds = (tiles + slots - 1) / slots;
-  return (double)rounds * C::BM * C::BN * per_flop_penalty;
+// ---- launch planning ---------------------------------------------------------
+// A launch runs ceil(tiles / CUs) rounds of tiles; a tile costs (k / 64) slab times plus an epilogue.
+// Problems of very different heights (the 8192-row image stream and the 666-row text stream of a joint
+// block) are badly served by one tile shape: the small problem's few large tiles add a nearly empty
+// round.  The planner therefore gives every problem the shape that is cheapest for it alone, launches
+// one kernel per shape, and falls back to a single shape when that is cheaper.
+constexpr int NCFG = 4;
+constexpr int kBM[NCFG] = {256, 128, 128, 256};
+constexpr int kBN[NCFG] = {192, 256, 128, 256};
+// measured on MI355X: microseconds per 64-wide slab and per epilogue of one tile
+constexpr double kSlabUs[NCFG] = {1.35, 1.10, 0.65, 1.99};
+constexpr double kEpiUs[NCFG] = {5.5, 3.5, 2.5, 9.0};
+constexpr double kLaunchUs = 3.0;
+constexpr int kSlots = 256;
+
+int tiles_of(const hdit_gemm_problem& p, int c) { return ((p.m + kBM[c] - 1) / kBM[c]) * ((p.n + kBN[c] - 1) / kBN[c]); }
+
+double launch_time(const hdit_gemm_problem* const* ps, int count, int c) {
+  int tiles = 0;
+  double work = 0;
+  for (int i = 0; i < count; i++) {
+    const int t = tiles_of(*ps[i], c);
+    tiles += t;
+    work += t * ((ps[i]->k / BK) * kSlabUs[c] + kEpiUs[c]);
+  }
+  if (tiles == 0) return 0;
+  const int rounds = (tiles + kSlots - 1) / kSlots;
+  return kLaunchUs + rounds * (work / tiles);
+}
+
+int launch_cfg(int cfg, const hdit_gemm_problem* problems, int count, hipStream_t s) {
+  switch (cfg) {
+    case 0: return build_and_launch<Cfg256x192>(problems, count, s);
+    case 1: return build_and_launch<Cfg128x256>(problems, count, s);
+    case 3: return build_and_launch<Cfg256x256>(problems, count, s);
+    default: return build_and_launch<Cfg128x128>(problems, count, s);
+  }
 }
 
 }  // namespace
@@ -522,20 +552,43 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
   }
   if (nlive == 0) return HDIT_OK;
   hipStream_t s = (hipStream_t)stream;
-  int cfg = g_force_cfg;
-  if (cfg < 0) {
-    const double c0 = launch_cost<Cfg256x192>(live, nlive, 1.00, 256);
-    const double c1 = launch_cost<Cfg128x256>(live, nlive, 1.03, 256);
-    const double c2 = launch_cost<Cfg128x128>(live, nlive, 1.24, 256);
-    cfg = 0;
-    double best = c0;
-    if (c1 < best) best = c1, cfg = 1;
-    if (c2 < best) best = c2, cfg = 2;
+  if (g_force_cfg >= 0) return launch_cfg(g_force_cfg, live, nlive, s);
+
+  // every problem's own best shape
+  int own[HDIT_GEMM_MAX_PROBLEMS];
+  const hdit_gemm_problem* ptr[HDIT_GEMM_MAX_PROBLEMS];
+  for (int i = 0; i < nlive; i++) {
+    const hdit_gemm_problem* one = &live[i];
+    own[i] = 0;
+    double best = launch_time(&one, 1, 0);
+    for (int c = 1; c < NCFG; c++) {
+      const double t = launch_time(&one, 1, c);
+      if (t < best) best = t, own[i] = c;
+    }
   }
-  switch (cfg) {
-    case 0: return build_and_launch<Cfg256x192>(live, nlive, s);
-    case 1: return build_and_launch<Cfg128x256>(live, nlive, s);
-    case 3: return build_and_launch<Cfg256x256>(live, nlive, s);
-    default: return build_and_launch<Cfg128x128>(live, nlive, s);
+  double split_cost = 0;
+  for (int c = 0; c < NCFG; c++) {
+    int n = 0;
+    for (int i = 0; i < nlive; i++)
+      if (own[i] == c) ptr[n++] = &live[i];
+    split_cost += launch_time(ptr, n, c);
   }
+  for (int i = 0; i < nlive; i++) ptr[i] = &live[i];
+  int single = 0;
+  double single_cost = launch_time(ptr, nlive, 0);
+  for (int c = 1; c < NCFG; c++) {
+    const double t = launch_time(ptr, nlive, c);
+    if (t < single_cost) single_cost = t, single = c;
+  }
+  if (single_cost <= split_cost) return launch_cfg(single, live, nlive, s);
+  for (int c = 0; c < NCFG; c++) {
+    hdit_gemm_problem group[HDIT_GEMM_MAX_PROBLEMS];
+    int n = 0;
+    for (int i = 0; i < nlive; i++)
+      if (own[i] == c) group[n++] = live[i];
+    if (n == 0) continue;
+    const int rc = launch_cfg(c, group, n, s);
+    if (rc != HDIT_OK) return rc;
+  }
+  return HDIT_OK;
 }
