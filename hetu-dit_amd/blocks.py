@@ -26,7 +26,7 @@ from torch import nn
 
 from . import ops
 from .cache_manager import get_cache_manager
-from .layers.attention_processor import _rows2d, hetuDiTAttentionWrapper
+from .layers.attention_processor import _PackedProjection, _rows2d, hetuDiTAttentionWrapper
 from .layers.feedforward import hetuDiTFeedForwardWrapper
 from .layers.modules import (
     AdaLayerNormContinuous,
@@ -54,9 +54,37 @@ def _wrap(layer: nn.Module) -> nn.Module:
 
 
 def _adaln(norm: nn.Module, temb: torch.Tensor):
-    """f32 [B, chunks*D] = linear(silu(temb)); chunk views."""
+    """f32 [B, chunks*D] = linear(silu(temb)); chunk views.  Taken from the stack-wide launch of
+    ``StackModulation`` when that ran on this very ``temb``."""
+    cached = getattr(norm, "_stack_emb", None)
+    if cached is not None and cached[0] == temb.data_ptr() and cached[1] == temb._version:
+        return cached[2].chunk(norm.chunks, dim=1)
     emb = ops.adaln_gemv(temb.contiguous(), norm.linear.weight.data, norm.linear.bias.data)
     return emb.chunk(norm.chunks, dim=1)
+
+
+class StackModulation:
+    """``linear(silu(temb))`` of every adaLN module of a block stack in one launch.
+
+    Within a denoise step all blocks are conditioned on the same ``temb``
+    (``transformer_sd3.py:107-152`` passes it unchanged to every block), so the
+    per-block weight streams (56.6 MB per SD3 block) can be read by one
+    bandwidth-bound GEMV over the concatenated weights instead of 48 short ones.
+    The ``nn.Linear`` modules stay addressable: their ``.data`` are row slices of
+    the packed weight, re-packed if a hot-swap re-assigns them."""
+
+    def __init__(self, blocks):
+        kinds = (AdaLayerNormZero, AdaLayerNormZeroSingle, AdaLayerNormContinuous, CogVideoXLayerNormZero)
+        self.norms = [m for b in blocks for m in b.modules() if isinstance(m, kinds)]
+        self.packed = _PackedProjection([n.linear for n in self.norms])
+
+    def precompute(self, temb: torch.Tensor):
+        w, b = self.packed.get()
+        emb = ops.adaln_gemv(temb.contiguous(), w, b)
+        off = 0
+        for norm, rows in zip(self.norms, self.packed.splits):
+            norm._stack_emb = (temb.data_ptr(), temb._version, emb[:, off : off + rows])
+            off += rows
 
 
 def _mlp_both_streams(ff, x2, resid, gate, ff_c=None, xc2=None, resid_c=None, gate_c=None):

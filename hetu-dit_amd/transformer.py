@@ -14,7 +14,8 @@ from typing import List, Optional, Tuple
 import torch
 from torch import nn
 
-from .blocks import CogVideoXBlock, FluxSingleTransformerBlock, FluxTransformerBlock, JointTransformerBlock
+from .blocks import (CogVideoXBlock, FluxSingleTransformerBlock, FluxTransformerBlock, JointTransformerBlock,
+                     StackModulation)
 from .runtime_state import get_runtime_state
 
 
@@ -30,10 +31,12 @@ class SD3TransformerBlocks(nn.Module):
             ]
         )
         self.encoder_hidden_states_cache: List[Optional[torch.Tensor]] = [None] * num_layers
+        self.modulation = StackModulation(self.transformer_blocks)
 
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb):
         rs = get_runtime_state()
+        self.modulation.precompute(temb)
         for i, block in enumerate(self.transformer_blocks):
             if rs.patch_mode and rs.pipeline_patch_idx == 0:
                 self.encoder_hidden_states_cache[i] = encoder_hidden_states
@@ -61,9 +64,11 @@ class FluxTransformerBlocks(nn.Module):
         self.single_transformer_blocks = nn.ModuleList(
             [FluxSingleTransformerBlock(dim, num_attention_heads, attention_head_dim) for _ in range(num_single_layers)]
         )
+        self.modulation = StackModulation(list(self.transformer_blocks) + list(self.single_transformer_blocks))
 
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb):
+        self.modulation.precompute(temb)
         for block in self.transformer_blocks:
             encoder_hidden_states, hidden_states = block(
                 hidden_states=hidden_states, encoder_hidden_states=encoder_hidden_states, temb=temb,
@@ -85,9 +90,11 @@ class CogVideoXTransformerBlocks(nn.Module):
         self.transformer_blocks = nn.ModuleList(
             [CogVideoXBlock(dim, num_attention_heads, attention_head_dim, time_embed_dim) for _ in range(num_layers)]
         )
+        self.modulation = StackModulation(self.transformer_blocks)
 
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None) -> Tuple[torch.Tensor, torch.Tensor]:
+        self.modulation.precompute(temb)
         for block in self.transformer_blocks:
             hidden_states, encoder_hidden_states = block(
                 hidden_states=hidden_states, encoder_hidden_states=encoder_hidden_states, temb=temb,

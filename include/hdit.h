@@ -36,8 +36,10 @@ const char* hdit_last_error(void);
  *
  * A [m, k] row-major (lda), B [n, k] row-major (ldb; an nn.Linear weight),
  * C [m, n] row-major (ldc); fp32 accumulation on MFMA.  Requirements:
- * k % 32 == 0, n % 8 == 0, lda/ldb/ldc/ldr % 8 == 0, every pointer 16-byte
- * aligned, m * lda and n * ldb below 2^31 elements.  Up to
+ * k % 64 == 0, n % 8 == 0, lda/ldb/ldc/ldr % 8 == 0, every pointer 16-byte
+ * aligned, m * lda and n * ldb below 2^31 elements, m * ldc and m * ldr below
+ * 2^30.  Problems of one call may be spread over several kernel launches (one
+ * per tile shape) on the given stream.  Up to
  * HDIT_GEMM_MAX_PROBLEMS problems share one launch (the image and text streams
  * of a joint block, or q|k|v|mlp of a fused projection).
  *
