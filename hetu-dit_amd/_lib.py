@@ -75,6 +75,22 @@ class QkNormJob(C.Structure):
     ]
 
 
+class LnJob(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p),
+        ("y", C.c_void_p),
+        ("shift", C.c_void_p),
+        ("scale", C.c_void_p),
+        ("x_sb", C.c_int64),
+        ("x_st", C.c_int64),
+        ("y_sb", C.c_int64),
+        ("y_st", C.c_int64),
+        ("mod_stride", C.c_int64),
+        ("batch", C.c_int32),
+        ("tokens", C.c_int32),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/hdit.h declares
 SIGNATURES = {
     "hdit_abi_version": (C.c_int, []),
@@ -88,6 +104,10 @@ SIGNATURES = {
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
          C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_void_p],
+    ),
+    "hdit_layernorm_modulate_jobs": (
+        C.c_int,
+        [C.POINTER(LnJob), C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p],
     ),
     "hdit_gate_residual": (
         C.c_int,

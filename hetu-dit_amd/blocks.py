@@ -127,20 +127,19 @@ class JointTransformerBlock(nn.Module):
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor):
         eps = 1e-6
         sh_a, sc_a, g_a, sh_m, sc_m, g_m = _adaln(self.norm1, temb)
-        n = ops.layernorm_modulate(hidden_states, sh_a, sc_a, eps)
         if self.context_pre_only:
             c_sc, c_sh = _adaln(self.norm1_context, temb)  # AdaLayerNormContinuous: scale first
-            nc = ops.layernorm_modulate(encoder_hidden_states, c_sh, c_sc, eps)
+            n, nc = ops.layernorm_modulate_many([(hidden_states, sh_a, sc_a), (encoder_hidden_states, c_sh, c_sc)], eps)
             hidden, _ = self.attn.forward_gated(n, nc, hidden_states, g_a)
         else:
             c_sh_a, c_sc_a, c_g_a, c_sh_m, c_sc_m, c_g_m = _adaln(self.norm1_context, temb)
-            nc = ops.layernorm_modulate(encoder_hidden_states, c_sh_a, c_sc_a, eps)
+            n, nc = ops.layernorm_modulate_many([(hidden_states, sh_a, sc_a), (encoder_hidden_states, c_sh_a, c_sc_a)], eps)
             hidden, encoder = self.attn.forward_gated(n, nc, hidden_states, g_a, encoder_hidden_states, c_g_a)
-        n2 = ops.layernorm_modulate(hidden, sh_m, sc_m, eps)
         if self.context_pre_only:
+            n2 = ops.layernorm_modulate(hidden, sh_m, sc_m, eps)
             _mlp_both_streams(self.ff, _rows2d(n2), hidden, g_m)
             return None, hidden
-        nc2 = ops.layernorm_modulate(encoder, c_sh_m, c_sc_m, eps)
+        n2, nc2 = ops.layernorm_modulate_many([(hidden, sh_m, sc_m), (encoder, c_sh_m, c_sc_m)], eps)
         _mlp_both_streams(self.ff, _rows2d(n2), hidden, g_m, self.ff_context, _rows2d(nc2), encoder, c_g_m)
         return encoder, hidden
 
@@ -166,12 +165,10 @@ class FluxTransformerBlock(nn.Module):
         eps = 1e-6
         sh_a, sc_a, g_a, sh_m, sc_m, g_m = _adaln(self.norm1, temb)
         c_sh_a, c_sc_a, c_g_a, c_sh_m, c_sc_m, c_g_m = _adaln(self.norm1_context, temb)
-        n = ops.layernorm_modulate(hidden_states, sh_a, sc_a, eps)
-        nc = ops.layernorm_modulate(encoder_hidden_states, c_sh_a, c_sc_a, eps)
+        n, nc = ops.layernorm_modulate_many([(hidden_states, sh_a, sc_a), (encoder_hidden_states, c_sh_a, c_sc_a)], eps)
         hidden, encoder = self.attn.forward_gated(n, nc, hidden_states, g_a, encoder_hidden_states, c_g_a,
                                                   image_rotary_emb=image_rotary_emb)
-        n2 = ops.layernorm_modulate(hidden, sh_m, sc_m, eps)
-        nc2 = ops.layernorm_modulate(encoder, c_sh_m, c_sc_m, eps)
+        n2, nc2 = ops.layernorm_modulate_many([(hidden, sh_m, sc_m), (encoder, c_sh_m, c_sc_m)], eps)
         _mlp_both_streams(self.ff, _rows2d(n2), hidden, g_m, self.ff_context, _rows2d(nc2), encoder, c_g_m)
         return encoder, hidden
 
@@ -236,8 +233,8 @@ class CogVideoXBlock(nn.Module):
         Nt = encoder.shape[1]
         joint = torch.empty(B, Nt + N, D, dtype=torch.bfloat16, device=hidden.device)
         w, b = norm.norm.weight.data, norm.norm.bias.data
-        ops.layernorm_modulate(encoder, e_sh, e_sc, norm.norm.eps, w, b, out=joint[:, :Nt])
-        ops.layernorm_modulate(hidden, sh, sc, norm.norm.eps, w, b, out=joint[:, Nt:])
+        ops.layernorm_modulate_many([(encoder, e_sh, e_sc, joint[:, :Nt]), (hidden, sh, sc, joint[:, Nt:])],
+                                    norm.norm.eps, w, b)
         return joint, g, e_g
 
     @staticmethod

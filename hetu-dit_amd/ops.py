@@ -247,6 +247,49 @@ def layernorm_modulate(x, shift=None, scale=None, eps: float = 1e-6, ln_weight=N
     return out
 
 
+def layernorm_modulate_many(items, eps: float = 1e-6, ln_weight=None, ln_bias=None):
+    """LayerNorm + modulate of several tensors of one width in one launch.
+
+    ``items`` is a list of ``(x, shift, scale)`` or ``(x, shift, scale, out)``;
+    returns the outputs in order."""
+    jobs = (_lib.LnJob * len(items))()
+    outs, keep, D0, nbytes = [], [], None, 0.0
+    for i, it in enumerate(items):
+        x, shift, scale = it[0], it[1], it[2]
+        out = it[3] if len(it) > 3 else None
+        B, T, D, xsb, xst = _as3d(x, "x")
+        if D0 is None:
+            D0 = D
+        elif D != D0:
+            raise ValueError("all tensors of one launch must have the same width")
+        if out is None:
+            out = torch.empty(B, T, D, dtype=bf16, device=x.device)
+        Bo, To, Do, ysb, yst = _as3d(out, "out")
+        if (Bo, To, Do) != (B, T, D):
+            raise ValueError("out shape differs from x")
+        sh, st1 = _mod(shift, B, D, "shift")
+        sc, st2 = _mod(scale, B, D, "scale")
+        if sh is not None and sc is not None and st1 != st2:
+            raise ValueError("shift and scale must share a batch stride")
+        j = jobs[i]
+        j.x, j.y, j.shift, j.scale = x.data_ptr(), out.data_ptr(), sh, sc
+        j.x_sb, j.x_st, j.y_sb, j.y_st, j.mod_stride = xsb, xst, ysb, yst, (st1 or st2 or 0)
+        j.batch, j.tokens = B, T
+        outs.append(out)
+        keep.append((x, shift, scale, out))
+        nbytes += 4.0 * B * T * D
+    for w in (ln_weight, ln_bias):
+        if w is not None:
+            _need(w, bf16, "ln affine")
+    check(
+        _run("ln_modulate", nbytes,
+             lambda: _lib.lib().hdit_layernorm_modulate_jobs(jobs, len(items), D0, _ptr(ln_weight), _ptr(ln_bias), eps,
+                                                             _stream())),
+        "hdit_layernorm_modulate_jobs",
+    )
+    return outs
+
+
 def gate_residual(x, y, gate, out=None):
     B, T, D, xsb, xst = _as3d(x, "x")
     By, Ty, Dy, ysb, yst = _as3d(y, "y")

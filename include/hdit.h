@@ -132,6 +132,22 @@ int hdit_layernorm_modulate(const void* x, void* y, const float* shift, const fl
                             int dim, int64_t x_sb, int64_t x_st, int64_t y_sb, int64_t y_st,
                             int64_t mod_stride, float eps, void* stream);
 
+/* The same for up to HDIT_LN_MAX_JOBS tensors of one width in one launch (the
+ * image and the text stream of a joint block: norm1 + norm1_context, or
+ * norm2 + norm2_context, of the blocks cited above). */
+#define HDIT_LN_MAX_JOBS 4
+typedef struct hdit_ln_job {
+  const void* x;      /* bf16 [batch, tokens, dim] */
+  void* y;            /* bf16 [batch, tokens, dim] */
+  const float* shift; /* f32, batch stride mod_stride, or NULL */
+  const float* scale;
+  int64_t x_sb, x_st, y_sb, y_st, mod_stride;
+  int32_t batch, tokens;
+} hdit_ln_job;
+
+int hdit_layernorm_modulate_jobs(const hdit_ln_job* jobs, int count, int dim, const void* ln_weight,
+                                 const void* ln_bias, float eps, void* stream);
+
 /* out = x + gate[b,:] * y   (bf16 [batch, tokens, dim], gate f32).  The gated
  * residual of the same blocks when it is not fused into a GEMM epilogue. */
 int hdit_gate_residual(const void* x, const void* y, const float* gate, void* out, int batch,

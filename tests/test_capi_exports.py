@@ -30,7 +30,7 @@ def library():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for name in ("hdit_gemm_bf16", "hdit_attn_fwd_bf16", "hdit_attn_fwd_fp8", "hdit_attn_absmax",
-                 "hdit_layernorm_modulate", "hdit_gate_residual", "hdit_adaln_gemv", "hdit_gelu_tanh",
+                 "hdit_layernorm_modulate", "hdit_layernorm_modulate_jobs", "hdit_gate_residual", "hdit_adaln_gemv", "hdit_gelu_tanh",
                  "hdit_qk_norm_rope", "hdit_copy_rows", "hdit_abi_version", "hdit_last_error"):
         assert name in syms
 
@@ -79,5 +79,6 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(library):
     a.batch, a.heads, a.head_dim = 1, 1, 96
     assert lib.hdit_attn_fwd_bf16(ctypes.byref(a), None) == -2
     assert lib.hdit_layernorm_modulate(None, None, None, None, None, None, 1, 1, 64, 64, 64, 64, 64, 0, 1e-6, None) == -1
+    assert lib.hdit_layernorm_modulate_jobs(None, 1, 64, None, None, 1e-6, None) == -1
     assert lib.hdit_adaln_gemv(4096, 4096, None, 4096, 9, 16, 64, None) == -2
     assert lib.hdit_qk_norm_rope(None, 1, 1, 1, 64, 1e-6, None) == -1

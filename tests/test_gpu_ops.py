@@ -126,6 +126,23 @@ def test_layernorm_modulate(hdit, dim):
     assert_parity(y, O.layer_norm(x, 1e-5, w, b), what="ln affine")
 
 
+def test_layernorm_modulate_many(hdit):
+    """Two streams of different length in one launch, one of them written into a slice of a joint buffer."""
+    B, D = 2, 1536
+    xs = [rnd(B, 37, D, scale=2.0, seed=11) + 0.5, rnd(B, 5, D, seed=12)]
+    xs = [bf16_round(x) for x in xs]
+    mod = torch.randn(B, 4 * D, generator=torch.Generator().manual_seed(13))
+    md = mod.to(DEV)
+    joint = torch.zeros(B, 42, D, dtype=torch.bfloat16, device=DEV)
+    outs = hdit.ops.layernorm_modulate_many(
+        [(g(xs[0]), md[:, :D], md[:, D:2 * D], joint[:, 5:]), (g(xs[1]), md[:, 2 * D:3 * D], md[:, 3 * D:])], eps=1e-6)
+    torch.cuda.synchronize()
+    assert outs[0].data_ptr() == joint[:, 5:].data_ptr()
+    assert_parity(joint[:, 5:], O.modulate(O.layer_norm(xs[0], 1e-6), mod[:, :D], mod[:, D:2 * D]), what="ln many 0")
+    assert_parity(outs[1], O.modulate(O.layer_norm(xs[1], 1e-6), mod[:, 2 * D:3 * D], mod[:, 3 * D:]), what="ln many 1")
+    assert float(joint[:, :5].float().abs().sum()) == 0.0
+
+
 def test_gate_residual_and_gelu(hdit):
     B, T, D = 2, 33, 1536
     x, y = rnd(B, T, D, seed=1), rnd(B, T, D, seed=2)
