@@ -7,7 +7,8 @@ import os
 import threading
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libhdit.so")
+# HDIT_LIBRARY selects another build of the same ABI (kernel experiments); default: the in-tree library
+LIB_PATH = os.environ.get("HDIT_LIBRARY") or os.path.join(HERE, "libhdit.so")
 
 HDIT_GEMM_MAX_PROBLEMS = 16
 EPI_BIAS, EPI_BIAS_GELU, EPI_GATE_RESIDUAL = 0, 1, 2

@@ -110,10 +110,10 @@ __device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
 
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// All tiles of one shape that this workgroup owns.
 template <class C>
-__global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total_tiles, int tiles_per_xcd,
-                                                  int wgs_per_xcd) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+__device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles, int tiles_per_xcd, int wgs_per_xcd,
+                                          unsigned char* lds) {
   constexpr int TM = C::TM, TN = C::TN;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -428,29 +428,97 @@ __global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total
 }
 
 template <class C>
+__global__ void __launch_bounds__(NT) gemm_kernel(const GemmTable tab, int total_tiles, int tiles_per_xcd,
+                                                  int wgs_per_xcd) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  run_tiles<C>(tab, total_tiles, tiles_per_xcd, wgs_per_xcd, lds);
+}
+
+// Two tile shapes in one launch: the large tiles of the tall problems first, then the small tiles of the
+// short ones (the text stream of a joint block), which a workgroup starts as soon as its large tiles are
+// done: no second launch, and the small tiles fill the tail of the large ones.
+template <class C1, class C2>
+__global__ void __launch_bounds__(NT) gemm_kernel2(const GemmTable tab1, int total1, int per_xcd1, const GemmTable tab2,
+                                                   int total2, int per_xcd2, int wgs_per_xcd) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  run_tiles<C1>(tab1, total1, per_xcd1, wgs_per_xcd, lds);
+  __syncthreads();  // the second phase reuses the LDS of the first
+  run_tiles<C2>(tab2, total2, per_xcd2, wgs_per_xcd, lds);
+}
+
+int g_num_cus = 0;
+
+int max_workgroups() {
+  if (g_num_cus == 0) {
+    int dev = 0, n = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) {
+      hdit_host::set_error(hipGetErrorString(e));
+      return -1;
+    }
+    g_num_cus = n;
+  }
+  int max_wgs = g_num_cus / NUM_XCD * NUM_XCD;  // one workgroup per CU: a wave may use the whole register file
+  return max_wgs < NUM_XCD ? NUM_XCD : max_wgs;
+}
+
+template <class C>
 int launch(const GemmTable& tab, int total_tiles, hipStream_t stream) {
   static bool attr_set = false;
-  static int num_cus = 0;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e == hipSuccess) {
-      int dev = 0;
-      e = hipGetDevice(&dev);
-      if (e == hipSuccess) e = hipDeviceGetAttribute(&num_cus, hipDeviceAttributeMultiprocessorCount, dev);
-    }
     if (e != hipSuccess) {
       hdit_host::set_error(hipGetErrorString(e));
       return HDIT_ELAUNCH;
     }
     attr_set = true;
   }
-  int max_wgs = num_cus / NUM_XCD * NUM_XCD;  // one workgroup per CU: a wave may use the whole register file
-  if (max_wgs < NUM_XCD) max_wgs = NUM_XCD;
+  const int max_wgs = max_workgroups();
+  if (max_wgs < 0) return HDIT_ELAUNCH;
   const int tiles_per_xcd = (total_tiles + NUM_XCD - 1) / NUM_XCD;
   int wgs_per_xcd = max_wgs / NUM_XCD;
   if (wgs_per_xcd > tiles_per_xcd) wgs_per_xcd = tiles_per_xcd;
   hipLaunchKernelGGL(gemm_kernel<C>, dim3(wgs_per_xcd * NUM_XCD), dim3(NT), C::LDS_BYTES, stream, tab, total_tiles,
                      tiles_per_xcd, wgs_per_xcd);
+  return hdit_host::check_launch("hdit_gemm_bf16");
+}
+
+template <class C>
+int fill_table(GemmTable& tab, const hdit_gemm_problem* problems, int count) {
+  tab.count = count;
+  int total = 0;
+  for (int i = 0; i < count; i++) {
+    tab.p[i] = problems[i];
+    tab.tile_start[i] = total;
+    total += ((problems[i].m + C::BM - 1) / C::BM) * ((problems[i].n + C::BN - 1) / C::BN);
+  }
+  for (int i = count; i <= HDIT_GEMM_MAX_PROBLEMS; i++) tab.tile_start[i] = total;
+  return total;
+}
+
+template <class C1, class C2>
+int launch2(const hdit_gemm_problem* p1, int n1, const hdit_gemm_problem* p2, int n2, hipStream_t stream) {
+  constexpr int LDS = C1::LDS_BYTES > C2::LDS_BYTES ? C1::LDS_BYTES : C2::LDS_BYTES;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_kernel2<C1, C2>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    if (e != hipSuccess) {
+      hdit_host::set_error(hipGetErrorString(e));
+      return HDIT_ELAUNCH;
+    }
+    attr_set = true;
+  }
+  const int max_wgs = max_workgroups();
+  if (max_wgs < 0) return HDIT_ELAUNCH;
+  GemmTable t1, t2;
+  const int total1 = fill_table<C1>(t1, p1, n1), total2 = fill_table<C2>(t2, p2, n2);
+  const int per1 = (total1 + NUM_XCD - 1) / NUM_XCD, per2 = (total2 + NUM_XCD - 1) / NUM_XCD;
+  int wgs_per_xcd = max_wgs / NUM_XCD;
+  const int need = per1 > per2 ? per1 : per2;
+  if (wgs_per_xcd > need) wgs_per_xcd = need;
+  hipLaunchKernelGGL((gemm_kernel2<C1, C2>), dim3(wgs_per_xcd * NUM_XCD), dim3(NT), LDS, stream, t1, total1, per1, t2,
+                     total2, per2, wgs_per_xcd);
   return hdit_host::check_launch("hdit_gemm_bf16");
 }
 
@@ -465,14 +533,7 @@ int count_tiles(const hdit_gemm_problem* problems, int count) {
 template <class C>
 int build_and_launch(const hdit_gemm_problem* problems, int count, hipStream_t stream) {
   GemmTable tab;
-  tab.count = count;
-  int total = 0;
-  for (int i = 0; i < count; i++) {
-    tab.p[i] = problems[i];
-    tab.tile_start[i] = total;
-    total += ((problems[i].m + C::BM - 1) / C::BM) * ((problems[i].n + C::BN - 1) / C::BN);
-  }
-  for (int i = count; i <= HDIT_GEMM_MAX_PROBLEMS; i++) tab.tile_start[i] = total;
+  const int total = fill_table<C>(tab, problems, count);
   if (total == 0) return HDIT_OK;
   return launch<C>(tab, total, stream);
 }
@@ -494,14 +555,15 @@ constexpr int NCFG = 4;
 constexpr int kBM[NCFG] = {256, 128, 128, 256};
 constexpr int kBN[NCFG] = {192, 256, 128, 256};
 // measured on MI355X: microseconds per 64-wide slab and per epilogue of one tile
-constexpr double kSlabUs[NCFG] = {1.35, 1.10, 0.65, 1.99};
-constexpr double kEpiUs[NCFG] = {5.5, 3.5, 2.5, 9.0};
+constexpr double kSlabUs[NCFG] = {1.21, 0.72, 0.44, 1.40};
+constexpr double kEpiUs[NCFG] = {13.0, 12.4, 8.0, 16.0};  // epilogue plus the pipeline fill of a tile
 constexpr double kLaunchUs = 3.0;
 constexpr int kSlots = 256;
 
 int tiles_of(const hdit_gemm_problem& p, int c) { return ((p.m + kBM[c] - 1) / kBM[c]) * ((p.n + kBN[c] - 1) / kBN[c]); }
 
-double launch_time(const hdit_gemm_problem* const* ps, int count, int c) {
+// time of all tiles of `ps` under shape c, without launch overhead
+double tiles_time(const hdit_gemm_problem* const* ps, int count, int c) {
   int tiles = 0;
   double work = 0;
   for (int i = 0; i < count; i++) {
@@ -511,7 +573,11 @@ double launch_time(const hdit_gemm_problem* const* ps, int count, int c) {
   }
   if (tiles == 0) return 0;
   const int rounds = (tiles + kSlots - 1) / kSlots;
-  return kLaunchUs + rounds * (work / tiles);
+  return rounds * (work / tiles);
+}
+
+double launch_time(const hdit_gemm_problem* const* ps, int count, int c) {
+  return count == 0 ? 0.0 : kLaunchUs + tiles_time(ps, count, c);
 }
 
 int launch_cfg(int cfg, const hdit_gemm_problem* problems, int count, hipStream_t s) {
@@ -566,13 +632,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
       if (t < best) best = t, own[i] = c;
     }
   }
-  double split_cost = 0;
-  for (int c = 0; c < NCFG; c++) {
-    int n = 0;
-    for (int i = 0; i < nlive; i++)
-      if (own[i] == c) ptr[n++] = &live[i];
-    split_cost += launch_time(ptr, n, c);
-  }
+  // plan A: one shape for everything
   for (int i = 0; i < nlive; i++) ptr[i] = &live[i];
   int single = 0;
   double single_cost = launch_time(ptr, nlive, 0);
@@ -580,15 +640,26 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
     const double t = launch_time(ptr, nlive, c);
     if (t < single_cost) single_cost = t, single = c;
   }
-  if (single_cost <= split_cost) return launch_cfg(single, live, nlive, s);
-  for (int c = 0; c < NCFG; c++) {
-    hdit_gemm_problem group[HDIT_GEMM_MAX_PROBLEMS];
-    int n = 0;
-    for (int i = 0; i < nlive; i++)
-      if (own[i] == c) group[n++] = live[i];
-    if (n == 0) continue;
-    const int rc = launch_cfg(c, group, n, s);
-    if (rc != HDIT_OK) return rc;
+  // plan B: one launch, two shapes -- the problems that want 256-row tiles on the better of the two large
+  // shapes, the others on 128x128
+  hdit_gemm_problem big[HDIT_GEMM_MAX_PROBLEMS], small[HDIT_GEMM_MAX_PROBLEMS];
+  const hdit_gemm_problem* pb[HDIT_GEMM_MAX_PROBLEMS];
+  const hdit_gemm_problem* psm[HDIT_GEMM_MAX_PROBLEMS];
+  int nb = 0, ns = 0;
+  for (int i = 0; i < nlive; i++) {
+    if (own[i] == 0 || own[i] == 3) big[nb] = live[i], pb[nb] = &live[i], nb++;
+    else small[ns] = live[i], psm[ns] = &live[i], ns++;
   }
-  return HDIT_OK;
+  double two_cost = 1e30;
+  int big_cfg = 0;
+  if (nb > 0 && ns > 0) {
+    const double t0 = tiles_time(pb, nb, 0), t3 = tiles_time(pb, nb, 3);
+    big_cfg = t3 < t0 ? 3 : 0;
+    two_cost = kLaunchUs + (t3 < t0 ? t3 : t0) + tiles_time(psm, ns, 2);
+  }
+  if (two_cost < single_cost) {
+    if (big_cfg == 0) return launch2<Cfg256x192, Cfg128x128>(big, nb, small, ns, s);
+    return launch2<Cfg256x256, Cfg128x128>(big, nb, small, ns, s);
+  }
+  return launch_cfg(single, live, nlive, s);
 }

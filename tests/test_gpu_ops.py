@@ -65,6 +65,37 @@ def test_gemm_gelu_and_gate_residual_grouped(hdit):
     assert_parity(res, want, what="gate residual")
 
 
+@pytest.mark.parametrize("epi", ["bias", "gelu", "gate"])
+def test_gemm_tall_and_short_problem_in_one_call(hdit, epi):
+    """An image-sized and a text-sized problem of one call (the planner gives them different tile shapes and,
+    for this pair, runs both shapes in one launch)."""
+    print(f"gemm tall+short epi={epi}", flush=True)
+    B, T1, T2, D, N = 2, 4096, 333, 512, 1536
+    ops = hdit.ops
+    xs = [rnd(B, T1, D, seed=21), rnd(B, T2, D, seed=22)]
+    ws = [rnd(N, D, scale=0.05, seed=23), rnd(N, D, scale=0.05, seed=24)]
+    bs = [rnd(N, seed=25), rnd(N, seed=26)]
+    rs = [rnd(B, T1, N, seed=27), rnd(B, T2, N, seed=28)]
+    gate = torch.randn(B, 2 * N, generator=torch.Generator().manual_seed(29))
+    gd = gate.to(DEV)
+    outs, probs = [], []
+    for i, T in enumerate((T1, T2)):
+        out = g(rs[i]).clone() if epi == "gate" else torch.empty(B, T, N, dtype=torch.bfloat16, device=DEV)
+        outs.append(out)
+        if epi == "gate":
+            probs.append(ops.gemm_problem(g(xs[i]).view(-1, D), g(ws[i]), out.view(-1, N), g(bs[i]), ops.EPI_GATE_RESIDUAL,
+                                          resid=out.view(-1, N), gate=gd[:, i * N:(i + 1) * N], rows_per_batch=T))
+        else:
+            probs.append(ops.gemm_problem(g(xs[i]).view(-1, D), g(ws[i]), out.view(-1, N), g(bs[i]),
+                                          ops.EPI_BIAS_GELU if epi == "gelu" else ops.EPI_BIAS))
+    ops.gemm_launch(probs)
+    torch.cuda.synchronize()
+    for i in range(2):
+        lin = O.linear(xs[i], ws[i], bs[i])
+        want = {"bias": lin, "gelu": O.gelu_tanh(lin), "gate": rs[i] + gate[:, None, i * N:(i + 1) * N] * lin}[epi]
+        assert_parity(outs[i], want, what=f"{epi} problem {i}")
+
+
 @pytest.mark.parametrize("hd", [64, 128])
 @pytest.mark.parametrize("sq,skv", [(256, 256), (77, 333), (300, 1000), (64, 64), (1, 5)])
 def test_attention_single_segment(hdit, hd, sq, skv):
