@@ -36,11 +36,7 @@ def build_stack(cfg, device, seed=0):
 
     with torch.device(device):
         stack = transformer.SD3TransformerBlocks(cfg["layers"], cfg["dim"], cfg["heads"], cfg["head_dim"])
-    gen = torch.Generator(device=device).manual_seed(seed)
-    for _, p in sorted(stack.named_parameters(), key=lambda kv: kv[0]):
-        p.data = (torch.randn(p.shape, generator=gen, device=device) * 0.02).to(torch.bfloat16)
-        p.requires_grad_(False)
-    return stack
+    return randomize_(stack, device, seed)
 
 
 def algorithmic_flops(cfg):
@@ -49,6 +45,91 @@ def algorithmic_flops(cfg):
     gemm = 24.0 * S * D * D * B * cfg["layers"] - 18.0 * Nt * D * D * B  # last block: text stream stops after q|k|v
     attn = 4.0 * S * S * D * B * cfg["layers"]
     return gemm, attn
+
+
+def randomize_(module, device, seed=0):
+    import torch
+
+    gen = torch.Generator(device=device).manual_seed(seed)
+    for _, p in sorted(module.named_parameters(), key=lambda kv: kv[0]):
+        p.data = (torch.randn(p.shape, generator=gen, device=device) * 0.02).to(torch.bfloat16)
+        p.requires_grad_(False)
+    return module
+
+
+WORKLOADS = ("sd3_1024", "sd3_pipefusion", "flux_1024", "cogvideox_5b")
+
+
+def make_workload(name, dev):
+    """(step callable, description, gemm flops, attention flops, blocks per step, attention kernel name) of one of
+    BASELINE.json's configs.  sd3_1024 (configs[1]) is the headline workload; the others are the shapes of
+    configs[3], [2] and [4], selectable for profiling."""
+    import torch
+
+    from hetu_dit_amd import synthetic, transformer
+    from hetu_dit_amd.runtime_state import get_runtime_state, reset_runtime_state
+
+    cfg = synthetic.CONFIGS[name]
+    reset_runtime_state()
+    gen = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *shape: torch.randn(*shape, generator=gen, device=dev).to(torch.bfloat16)
+    B, Ni, Nt, D = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"]
+    S = Ni + Nt
+    if name in ("sd3_1024", "sd3_pipefusion"):
+        stack = build_stack(cfg, dev)
+        e, t = rnd(B, Nt, D), rnd(B, D)
+        if name == "sd3_1024":
+            x = rnd(B, Ni, D)
+            gemm, attn = algorithmic_flops(cfg)
+            desc = ("configs[1]: SD3-shape denoise step, 24 joint blocks, B2 (CFG pair), 4096 image + 333 text "
+                    "tokens, D1536, 24x64 heads, last block context_pre_only")
+            return (lambda: stack(x, e, t)), desc, gemm, attn, cfg["layers"], "attn_fwd_kernel<64>"
+        # PipeFusion shard: a full-sequence pass fills the K/V buffers ("previous step"), then one step is
+        # four patch passes of 1024 image tokens each against the stale full-length buffers
+        P = cfg["patches"]
+        rs = get_runtime_state()
+        rs.set_token_patches([Ni // P * i for i in range(P + 1)])
+        rs.set_patched_mode(False)
+        stack(rnd(B, Ni, D), e, t)
+        rs.set_patched_mode(True)
+        xs = [rnd(B, Ni // P, D) for _ in range(P)]
+
+        def step():
+            out = None
+            for p in range(P):
+                out = stack(xs[p], e, t)
+                rs.next_patch()
+            return out
+
+        L = cfg["layers"]
+        Sq = Ni // P + Nt
+        gemm = (24.0 * Sq * D * D * B * L - 18.0 * Nt * D * D * B) * P
+        attn = 4.0 * Sq * S * D * B * L * P
+        desc = ("configs[3]: SD3 PipeFusion shard, 24 joint blocks x 4 patches, B2, query 1024 image + 333 text tokens "
+                "against the 4096 + 333 stale K/V buffer")
+        return step, desc, gemm, attn, L * P, "attn_fwd_kernel<64>"
+    if name == "flux_1024":
+        with torch.device(dev):
+            stack = transformer.FluxTransformerBlocks(1, 1, D, cfg["heads"], cfg["head_dim"])
+        randomize_(stack, dev)
+        get_runtime_state().max_condition_sequence_length = Nt
+        cos, sin = synthetic.rope_table(synthetic.flux_ids(Nt, *cfg["grid"]), (16, 56, 56))
+        rope = (cos.to(dev), sin.to(dev))
+        x, e, t = rnd(B, Ni, D), rnd(B, Nt, D), rnd(B, D)
+        gemm = 24.0 * S * D * D * B * 2
+        attn = 4.0 * S * S * D * B * 2
+        desc = "configs[2]: Flux-shape, one double-stream + one single-stream block, B1, 4096 image + 512 text tokens, D3072, 24x128 heads"
+        return (lambda: stack(x, e, t, rope)[0]), desc, gemm, attn, 2, "attn_fwd_kernel<128>"
+    with torch.device(dev):
+        stack = transformer.CogVideoXTransformerBlocks(1, D, cfg["heads"], cfg["head_dim"], cfg["temb_dim"])
+    randomize_(stack, dev)
+    cos, sin = synthetic.rope_table(synthetic.cogvideox_positions(*cfg["grid"]), (16, 24, 24))
+    rope = (cos.to(dev), sin.to(dev))
+    x, e, t = rnd(B, Ni, D), rnd(B, Nt, D), rnd(B, cfg["temb_dim"])
+    gemm = 24.0 * S * D * D * B
+    attn = 4.0 * S * S * D * B
+    desc = "configs[4]: CogVideoX-5B-shape block, B1, 226 text + 17550 video tokens, D3072, 48x64 heads"
+    return (lambda: stack(x, e, t, rope)[0]), desc, gemm, attn, 1, "attn_fwd_kernel<64>"
 
 
 def cpu_baseline(runs=3):
@@ -92,6 +173,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--workload", choices=WORKLOADS, default="sd3_1024",
+                    help="sd3_1024 (BASELINE.json configs[1]) is the headline metric; the others are for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only: run with --gpus 1 "
@@ -107,33 +190,37 @@ def main():
     hetu_dit_amd._lib.lib()
     dev = "cuda:0"
     torch.cuda.set_device(0)
-    cfg = synthetic.CONFIGS["sd3_1024"]
-    reset_runtime_state()
-    stack = build_stack(cfg, dev)
-    B, Ni, Nt, D = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"]
-    gen = torch.Generator(device=dev).manual_seed(1)
-    x = torch.randn(B, Ni, D, generator=gen, device=dev).to(torch.bfloat16)
-    e = torch.randn(B, Nt, D, generator=gen, device=dev).to(torch.bfloat16)
-    t = torch.randn(B, D, generator=gen, device=dev).to(torch.bfloat16)
-
-    def step():
-        return stack(x, e, t)
+    step, workload_desc, gemm_fl, attn_fl, n_blocks, attn_kernel = make_workload(args.workload, dev)
+    headline = args.workload == "sd3_1024"
 
     for _ in range(max(args.warmup, 1)):
         out = step()
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all()
 
+    # persistent state a pass reads and mutates (the stale K/V buffers of the PipeFusion workload)
+    from hetu_dit_amd.cache_manager import get_cache_manager
+
+    def kv_buffers():
+        return [t for entry in get_cache_manager().cache.values() for t in entry.tensors if t is not None]
+
     use_graph = not args.no_graph
     if use_graph:
+        saved = [t.clone() for t in kv_buffers()]
+        ref = step().clone()
+        for t, s0 in zip(kv_buffers(), saved):
+            t.copy_(s0)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             g_out = step()
+        for t, s0 in zip(kv_buffers(), saved):
+            t.copy_(s0)
         graph.replay()
         torch.cuda.synchronize()
-        # a replay must reproduce the eager result bit for bit (same kernels, same inputs)
-        if not torch.equal(g_out, out):
+        # from the same buffer state a replay must reproduce the eager result bit for bit
+        if not torch.equal(g_out, ref):
             use_graph = False
+        del saved
         run = graph.replay if use_graph else step
     else:
         run = step
@@ -184,7 +271,6 @@ def main():
         glue[kind] = {"launches_per_step": len(recs) // 3, "largest_launch_bytes": big,
                       "largest_avg_us": round(ms / len(sel) * 1e3, 2), "achieved_GBps": round(nbytes / ms / 1e6, 1),
                       "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
-    gemm_fl, attn_fl = algorithmic_flops(cfg)
     result = {
         "metric": "ms per DiT denoise step (1 GPU)",
         "value": round(ms_step, 3),
@@ -193,36 +279,37 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_step, 3),
-        "ms_per_block": round(ms_step / cfg["layers"], 4),
+        "ms_per_block": round(ms_step / n_blocks, 4),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic (seeded N(0,1) activations, N(0,0.02) random-init weights, resident in HBM)",
-        "config": {"workload": "configs[1]: SD3-shape denoise step, 24 joint blocks, B2 (CFG pair), 4096 image + 333 text "
-                               "tokens, D1536, 24x64 heads, last block context_pre_only",
-                   "launch": "hip-graph replay" if use_graph else "eager"},
+        "config": {"workload": workload_desc, "launch": "hip-graph replay" if use_graph else "eager"},
         "step_tflops": round((gemm_fl + attn_fl) / ms_step / 1e9, 1),
         "roofline": {
             "kernel": "gemm_kernel (grouped bf16 MFMA GEMM, all projection/MLP launches of the step)",
             "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+            "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if headline else None,
             "traffic_note": "rocprofv3 FETCH_SIZE x2.0 + WRITE_SIZE x1.0 (factors from a 256 MiB copy), mean over the "
                             "step's GEMM launches; algorithmic operand+result bytes average 86.6 MB per launch",
             "launches_per_step": n_g // 3, "avg_launch_us": round(ms_g / max(n_g, 1) * 1e3, 2),
             "flops_per_launch": round(fl_g / max(n_g, 1), 1),
         },
         "roofline_attention": {
-            "kernel": "attn_fwd_kernel<64> (joint flash attention)", "bound": "mfma", "achieved": round(attn_tflops, 1),
+            "kernel": attn_kernel + " (joint flash attention)", "bound": "mfma", "achieved": round(attn_tflops, 1),
             "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
-            "traffic": ATTN_TRAFFIC_BYTES_PER_LAUNCH, "launches_per_step": n_a // 3, "avg_launch_us": round(ms_a / max(n_a, 1) * 1e3, 2),
+            "traffic": ATTN_TRAFFIC_BYTES_PER_LAUNCH if headline else None, "launches_per_step": n_a // 3, "avg_launch_us": round(ms_a / max(n_a, 1) * 1e3, 2),
             "flops_per_launch": round(fl_a / max(n_a, 1), 1),
         },
         "roofline_glue": glue,
         "reference_prior": {"ms_per_step": 242.7, "note": "hetu_dit/model_profiler.py:116-121, SD3 1024^2 1 GPU, "
                                                             "hardware unlabelled (README testbed NVIDIA L20); not the same hardware"},
     }
-    if not args.no_cpu_baseline:
+    if not headline:
+        result["metric"] = "ms per pass of the named workload (1 GPU)"
+        result.pop("reference_prior")
+    if not args.no_cpu_baseline and headline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
 
