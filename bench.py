@@ -25,8 +25,8 @@ PEAK_FP8_TFLOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes summarised in
 # profiles/sd3_1024_step_hbm_traffic.txt (hardware counters cannot be read from inside this process)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 376.0e6
-ATTN_TRAFFIC_BYTES_PER_LAUNCH = 516.6e6
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 351.2e6
+ATTN_TRAFFIC_BYTES_PER_LAUNCH = 516.7e6
 
 
 def build_stack(cfg, device, seed=0):
@@ -292,7 +292,7 @@ def main():
             "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
             "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if headline else None,
             "traffic_note": "rocprofv3 FETCH_SIZE x2.0 + WRITE_SIZE x1.0 (factors from a 256 MiB copy), mean over the "
-                            "step's GEMM launches; algorithmic operand+result bytes average 86.6 MB per launch",
+                            "step's hdit_gemm_bf16 calls; algorithmic operand+result bytes average 86.6 MB per call",
             "launches_per_step": n_g // 3, "avg_launch_us": round(ms_g / max(n_g, 1) * 1e3, 2),
             "flops_per_launch": round(fl_g / max(n_g, 1), 1),
         },
