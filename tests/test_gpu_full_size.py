@@ -1,0 +1,162 @@
+"""Parity at the full sizes of BASELINE.json's configs, where the fp32 oracle of the whole problem would
+take minutes: sampled rows against the oracle (a row of a GEMM or of an attention output only needs that
+row of the left operand), and properties that hold at any size -- softmax of a constant V returns V, the
+order of the key/value segments does not matter, adaLN-Zero with a zero modulation projection is the
+identity, a PipeFusion patch against a K/V buffer that holds this very step's values equals the rows of
+the full-sequence pass."""
+import pytest
+import torch
+
+from oracle import ops as O
+from tests.util import assert_parity, bf16_round
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def dev_randn(shape, seed, scale=1.0):
+    gen = torch.Generator(device=DEV).manual_seed(seed)
+    return (torch.randn(shape, generator=gen, device=DEV) * scale).to(torch.bfloat16)
+
+
+@pytest.fixture(autouse=True)
+def fresh_state():
+    from hetu_dit_amd.cache_manager import reset_cache_manager
+    from hetu_dit_amd.runtime_state import reset_runtime_state
+
+    reset_runtime_state()
+    yield
+    reset_cache_manager()
+    reset_runtime_state()
+    torch.cuda.empty_cache()
+
+
+def sample_rows(m, count, seed):
+    gen = torch.Generator().manual_seed(seed)
+    idx = torch.randint(0, m, (count,), generator=gen)
+    idx[0], idx[1] = 0, m - 1  # the corners of the first and the last tile
+    return idx
+
+
+# (image rows, text rows, n, k, epilogue): the four GEMM calls of an SD3 joint block at configs[1], the QKV+MLP
+# call of a Flux single block at configs[2], the FF1 call of a CogVideoX block at configs[4]
+GEMM_CASES = [
+    (8192, 666, 4608, 1536, "bias"),
+    (8192, 666, 1536, 1536, "gate"),
+    (8192, 666, 6144, 1536, "gelu"),
+    (8192, 666, 1536, 6144, "gate"),
+    (4608, 0, 9216, 3072, "bias"),
+    (17776, 0, 12288, 3072, "gelu"),
+]
+
+
+@pytest.mark.parametrize("m_img,m_txt,n,k,epi", GEMM_CASES)
+def test_gemm_full_size_sampled_rows(hdit, m_img, m_txt, n, k, epi):
+    print(f"gemm full size m={m_img}+{m_txt} n={n} k={k} epi={epi}", flush=True)
+    ops = hdit.ops
+    probs, checks = [], []
+    for i, m in enumerate([m for m in (m_img, m_txt) if m]):
+        a, w, b = dev_randn((m, k), 10 + i), dev_randn((n, k), 20 + i, 0.02), dev_randn((n,), 30 + i)
+        rows = sample_rows(m, 48, 40 + i)
+        if epi == "gate":
+            res = dev_randn((m, n), 50 + i)
+            gate = torch.randn(2, n, generator=torch.Generator(device=DEV).manual_seed(60 + i), device=DEV)
+            out = res.clone()
+            probs.append(ops.gemm_problem(a, w, out, b, ops.EPI_GATE_RESIDUAL, resid=out, gate=gate, rows_per_batch=m // 2))
+        else:
+            res = gate = None
+            out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+            probs.append(ops.gemm_problem(a, w, out, b, ops.EPI_BIAS_GELU if epi == "gelu" else ops.EPI_BIAS))
+        checks.append((a, w, b, res, gate, out, rows, m))
+    ops.gemm_launch(probs)
+    torch.cuda.synchronize()
+    for a, w, b, res, gate, out, rows, m in checks:
+        lin = O.linear(a[rows.to(DEV)].float().cpu(), w.float().cpu(), b.float().cpu())
+        if epi == "gelu":
+            want = O.gelu_tanh(lin)
+        elif epi == "gate":
+            g = gate.cpu()[(rows // (m // 2)).clamp(max=1)]
+            want = res[rows.to(DEV)].float().cpu() + g * lin
+        else:
+            want = lin
+        assert_parity(out[rows.to(DEV)], want, what=f"{epi} rows of m={m}")
+        assert torch.isfinite(out.float()).all()
+
+
+# (batch, heads, image tokens, text tokens, head dim): configs[1], [2], [4]
+ATTN_CASES = [(2, 24, 4096, 333, 64), (1, 24, 4096, 512, 128), (1, 48, 17550, 226, 64)]
+
+
+@pytest.mark.parametrize("B,H,n_img,n_txt,hd", ATTN_CASES)
+def test_attention_full_size(hdit, B, H, n_img, n_txt, hd):
+    print(f"attention full size B={B} H={H} {n_img}+{n_txt} hd={hd}", flush=True)
+    ops = hdit.ops
+    qi, qt = dev_randn((B, n_img, H, hd), 1), dev_randn((B, n_txt, H, hd), 2)
+    ki, kt = dev_randn((B, n_img, H, hd), 3), dev_randn((B, n_txt, H, hd), 4)
+    vi, vt = dev_randn((B, n_img, H, hd), 5), dev_randn((B, n_txt, H, hd), 6)
+    oi, ot = ops.attention([qi, qt], [ki, kt], [vi, vt])
+    torch.cuda.synchronize()
+    # sampled (batch, head, query) rows against the oracle: one row needs that query and all keys/values
+    S = n_img + n_txt
+    q = torch.cat([qi, qt], 1)
+    k = torch.cat([ki, kt], 1).float().cpu()
+    v = torch.cat([vi, vt], 1).float().cpu()
+    o = torch.cat([oi, ot], 1)
+    rows = sample_rows(S, 24, 7)
+    rows[2], rows[3] = n_img - 1, n_img  # both sides of the segment boundary
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        want = O.attention(q[b, rows.to(DEV), h].float().cpu()[None, None], k[b, :, h][None, None], v[b, :, h][None, None])[0, 0]
+        assert_parity(o[b, rows.to(DEV), h], want, what=f"attention rows b={b} h={h}")
+    # the order of the key/value segments does not matter (SD3 joins [image, text], Flux [text, image])
+    oi2, ot2 = ops.attention([qi, qt], [kt, ki], [vt, vi])
+    torch.cuda.synchronize()
+    assert_parity(oi2, oi.float(), rel=4e-3, what="segment order (image queries)")
+    assert_parity(ot2, ot.float(), rel=4e-3, what="segment order (text queries)")
+    # a value that is the same for every key comes back unchanged, whatever the scores
+    const = dev_randn((B, 1, H, hd), 8)
+    ci, ct = ops.attention([qi, qt], [ki, kt], [const.expand(B, n_img, H, hd).contiguous(), const.expand(B, n_txt, H, hd).contiguous()])
+    torch.cuda.synchronize()
+    assert_parity(ci, const.expand(B, n_img, H, hd).float(), rel=4e-3, what="constant V (image)")
+    assert_parity(ct, const.expand(B, n_txt, H, hd).float(), rel=4e-3, what="constant V (text)")
+
+
+def test_sd3_stack_full_size_properties(hdit):
+    """configs[1] and configs[3] at full size (24 blocks, B2, 4096 + 333 tokens)."""
+    from hetu_dit_amd import synthetic, transformer
+    from hetu_dit_amd.layers.modules import AdaLayerNormContinuous, AdaLayerNormZero
+    from hetu_dit_amd.runtime_state import get_runtime_state
+
+    cfg = synthetic.CONFIGS["sd3_pipefusion"]
+    B, Ni, Nt, D, L, P = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"], cfg["layers"], cfg["patches"]
+    with torch.device(DEV):
+        stack = transformer.SD3TransformerBlocks(L, D, cfg["heads"], cfg["head_dim"])
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    for _, p in sorted(stack.named_parameters(), key=lambda kv: kv[0]):
+        p.data = (torch.randn(p.shape, generator=gen, device=DEV) * 0.02).to(torch.bfloat16)
+    x, e, t = dev_randn((B, Ni, D), 11), dev_randn((B, Nt, D), 12), dev_randn((B, D), 13)
+
+    # a PipeFusion patch whose K/V buffer holds this very input's keys and values sees what the full pass saw:
+    # its output is the matching rows of the full-sequence output
+    rs = get_runtime_state()
+    rs.set_token_patches([Ni // P * i for i in range(P + 1)])
+    rs.set_patched_mode(False)
+    full = stack(x, e, t)
+    torch.cuda.synchronize()
+    assert torch.isfinite(full.float()).all()
+    rs.set_patched_mode(True)
+    for p in range(P):
+        sl = slice(Ni // P * p, Ni // P * (p + 1))
+        got = stack(x[:, sl].contiguous(), e, t)
+        torch.cuda.synchronize()
+        assert_parity(got, full[:, sl].float(), what=f"patch {p} against the rows of the full pass")
+        rs.next_patch()
+    rs.set_patched_mode(False)
+
+    # adaLN-Zero: with the modulation projections zeroed every gate is zero and the stack is the identity
+    for m in stack.modules():
+        if isinstance(m, (AdaLayerNormZero, AdaLayerNormContinuous)):
+            m.linear.weight.data.zero_()
+            m.linear.bias.data.zero_()
+    out = stack(x, e, t)
+    torch.cuda.synchronize()
+    assert torch.equal(out, x)
