@@ -19,6 +19,7 @@
 // Q, K, V, O are each up to two sequence segments in different buffers, so the
 // joint [image, text] / [text, image] sequences and the "fresh text + stale
 // image buffer" K/V of a PipeFusion patch need no concatenation copy.
+#include <atomic>
 #include <type_traits>
 
 #include "hdit_common.h"
@@ -365,12 +366,12 @@ extern "C" __attribute__((visibility("default"))) int hdit_attn_fwd_bf16(const h
   if (a->head_dim == 64) {
     hipLaunchKernelGGL(attn_fwd_kernel<64>, grid, block, Lds<64>::TOTAL, s, P, q_tiles);
   } else {
-    static bool attr = false;
-    if (!attr) {
+    static std::atomic<bool> attr{false};  // setting the attribute twice from two threads is harmless
+    if (!attr.load(std::memory_order_acquire)) {
       if (hipFuncSetAttribute((const void*)attn_fwd_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               Lds<128>::TOTAL) != hipSuccess)
         return HDIT_ELAUNCH;
-      attr = true;
+      attr.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(attn_fwd_kernel<128>, grid, block, Lds<128>::TOTAL, s, P, q_tiles);
   }

@@ -35,6 +35,7 @@
 // One launch covers up to HDIT_GEMM_MAX_PROBLEMS problems.  Tiles are dealt to
 // workgroups so that the workgroups of one XCD (workgroup id mod 8; each XCD
 // has a private L2) own a contiguous, 8-tile-row-grouped range.
+#include <atomic>
 #include <type_traits>
 
 #include "hdit_common.h"
@@ -446,10 +447,10 @@ __global__ void __launch_bounds__(NT) gemm_kernel2(const GemmTable tab1, int tot
   run_tiles<C2>(tab2, total2, per_xcd2, wgs_per_xcd, lds);
 }
 
-int g_num_cus = 0;
+std::atomic<int> g_num_cus{0};
 
 int max_workgroups() {
-  if (g_num_cus == 0) {
+  if (g_num_cus.load(std::memory_order_acquire) == 0) {
     int dev = 0, n = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
@@ -457,22 +458,22 @@ int max_workgroups() {
       hdit_host::set_error(hipGetErrorString(e));
       return -1;
     }
-    g_num_cus = n;
+    g_num_cus.store(n, std::memory_order_release);
   }
-  int max_wgs = g_num_cus / NUM_XCD * NUM_XCD;  // one workgroup per CU: a wave may use the whole register file
+  int max_wgs = g_num_cus.load(std::memory_order_relaxed) / NUM_XCD * NUM_XCD;  // one workgroup per CU: a wave may use the whole register file
   return max_wgs < NUM_XCD ? NUM_XCD : max_wgs;
 }
 
 template <class C>
 int launch(const GemmTable& tab, int total_tiles, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
+  static std::atomic<bool> attr_set{false};  // setting the attribute twice from two threads is harmless
+  if (!attr_set.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     if (e != hipSuccess) {
       hdit_host::set_error(hipGetErrorString(e));
       return HDIT_ELAUNCH;
     }
-    attr_set = true;
+    attr_set.store(true, std::memory_order_release);
   }
   const int max_wgs = max_workgroups();
   if (max_wgs < 0) return HDIT_ELAUNCH;
@@ -500,14 +501,14 @@ int fill_table(GemmTable& tab, const hdit_gemm_problem* problems, int count) {
 template <class C1, class C2>
 int launch2(const hdit_gemm_problem* p1, int n1, const hdit_gemm_problem* p2, int n2, hipStream_t stream) {
   constexpr int LDS = C1::LDS_BYTES > C2::LDS_BYTES ? C1::LDS_BYTES : C2::LDS_BYTES;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static std::atomic<bool> attr_set{false};  // setting the attribute twice from two threads is harmless
+  if (!attr_set.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_kernel2<C1, C2>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) {
       hdit_host::set_error(hipGetErrorString(e));
       return HDIT_ELAUNCH;
     }
-    attr_set = true;
+    attr_set.store(true, std::memory_order_release);
   }
   const int max_wgs = max_workgroups();
   if (max_wgs < 0) return HDIT_ELAUNCH;
@@ -543,7 +544,7 @@ using Cfg256x192 = Cfg<4, 3>;
 using Cfg128x256 = Cfg<2, 4>;
 using Cfg128x128 = Cfg<2, 2>;
 
-int g_force_cfg = -1;
+std::atomic<int> g_force_cfg{-1};
 
 // ---- launch planning ---------------------------------------------------------
 // A launch runs ceil(tiles / CUs) rounds of tiles; a tile costs (k / 64) slab times plus an epilogue.
@@ -591,7 +592,7 @@ int launch_cfg(int cfg, const hdit_gemm_problem* problems, int count, hipStream_
 
 }  // namespace
 
-extern "C" __attribute__((visibility("default"))) void hdit_gemm_force_config(int cfg) { g_force_cfg = cfg; }
+extern "C" __attribute__((visibility("default"))) void hdit_gemm_force_config(int cfg) { g_force_cfg.store(cfg, std::memory_order_relaxed); }
 
 extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_gemm_problem* problems, int count, void* stream) {
   if (!problems || count < 0 || count > HDIT_GEMM_MAX_PROBLEMS) return HDIT_EINVAL;
@@ -618,7 +619,8 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
   }
   if (nlive == 0) return HDIT_OK;
   hipStream_t s = (hipStream_t)stream;
-  if (g_force_cfg >= 0) return launch_cfg(g_force_cfg, live, nlive, s);
+  const int forced = g_force_cfg.load(std::memory_order_relaxed);
+  if (forced >= 0) return launch_cfg(forced, live, nlive, s);
 
   // every problem's own best shape
   int own[HDIT_GEMM_MAX_PROBLEMS];

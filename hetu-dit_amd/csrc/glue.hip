@@ -363,11 +363,12 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate_jo
   int64_t blocks = 0;
   for (int i = 0; i < count; i++) {
     const hdit_ln_job& j = jobs[i];
-    if (!j.x || !j.y || j.batch < 0 || j.tokens < 0) return HDIT_EINVAL;
+    if (j.batch < 0 || j.tokens < 0) return HDIT_EINVAL;
+    const int64_t rows = (int64_t)j.batch * j.tokens;
+    if (rows == 0) continue;  // an empty tensor may come with a null pointer
+    if (!j.x || !j.y) return HDIT_EINVAL;
     if (j.x_sb % 8 || j.x_st % 8 || j.y_sb % 8 || j.y_st % 8 || j.mod_stride % 4) return HDIT_EINVAL;
     if (!aligned16(j.x) || !aligned16(j.y) || !aligned16(j.shift) || !aligned16(j.scale)) return HDIT_EINVAL;
-    const int64_t rows = (int64_t)j.batch * j.tokens;
-    if (rows == 0) continue;
     tab.block_start[tab.count] = (int)blocks;
     tab.j[tab.count++] = j;
     blocks += (rows + 7) / 8;  // 4 waves x 2 rows

@@ -280,3 +280,38 @@ def test_torch_library_ops_dispatch_to_the_hip_kernels(hdit):
     torch.cuda.synchronize()
     assert_parity(y, O.gelu_tanh(O.linear(x, w, b)), what="torch.ops.hdit.linear")
     assert_parity(n, O.layer_norm(x, 1e-6), what="torch.ops.hdit.layernorm_modulate")
+
+
+def test_empty_and_ragged_inputs(hdit):
+    """Zero-row problems and zero-length segments are no-ops, not errors; odd sizes go through the edge paths."""
+    ops = hdit.ops
+    D, N = 128, 200  # n is a multiple of 8 but of no tile width
+    a, w, b = rnd(37, D, seed=1), rnd(N, D, scale=0.05, seed=2), rnd(N, seed=3)
+    out = torch.empty(37, N, dtype=torch.bfloat16, device=DEV)
+    empty_a = torch.empty(0, D, dtype=torch.bfloat16, device=DEV)
+    empty_out = torch.empty(0, N, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_launch([ops.gemm_problem(empty_a, g(w), empty_out, g(b)), ops.gemm_problem(g(a), g(w), out, g(b))])
+    ops.gemm_launch([ops.gemm_problem(empty_a, g(w), empty_out, g(b))])
+    torch.cuda.synchronize()
+    assert_parity(out, O.linear(a, w, b), what="ragged gemm next to an empty problem")
+    # LayerNorm of an empty stream next to a one-row stream
+    x1 = rnd(1, 1, 256, seed=4)
+    y0, y1 = ops.layernorm_modulate_many([(torch.empty(1, 0, 256, dtype=torch.bfloat16, device=DEV), None, None),
+                                          (g(x1), None, None)])
+    torch.cuda.synchronize()
+    assert y0.shape == (1, 0, 256)
+    assert_parity(y1, O.layer_norm(x1, 1e-6), what="one-row layernorm")
+    # attention: empty text segment on every operand; one query against three keys
+    q, k, v = rnd(1, 1, 2, 64, seed=5), rnd(1, 3, 2, 64, seed=6), rnd(1, 3, 2, 64, seed=7)
+    e = torch.empty(1, 0, 2, 64, dtype=torch.bfloat16, device=DEV)
+    o, o_e = ops.attention([g(q), e], [g(k), e], [g(v), e])
+    torch.cuda.synchronize()
+    assert o_e.shape == (1, 0, 2, 64)
+    want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
+    assert_parity(o, want, what="one query, three keys")
+    # no queries at all: nothing to do
+    (o0,) = ops.attention([e], [g(k)], [g(v)])
+    assert o0.shape == (1, 0, 2, 64)
+    # queries without any key are refused
+    with pytest.raises(hdit._lib.HditError):
+        ops.attention([g(q)], [e], [e])
