@@ -1,0 +1,144 @@
+// Head and tail of a denoise step around the block stack: patchify / unpatchify of the latent, the
+// sinusoidal timestep projection, SiLU, and classifier-free guidance fused with the flow-match Euler
+// update.  All of them touch about a megabyte per step; one thread per element (or per 8) is plenty.
+#include "hdit_common.h"
+
+namespace {
+
+using hdit::pack8;
+using hdit::unpack8;
+
+inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+// out[b, hy*w + wx, (c*p + py)*p + px] = latent[b, c, hy*p + py, wx*p + px]: the im2col of a p x p, stride p
+// convolution, columns in the order of the flattened conv weight [out, c, py, px]
+__global__ void __launch_bounds__(256) patchify_kernel(const __bf16* __restrict__ latent, __bf16* __restrict__ out,
+                                                       int64_t total, int C, int H, int W, int p) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int K = C * p * p, w = W / p, h = H / p;
+  const int col = (int)(i % K);
+  const int64_t tok = i / K;
+  const int px = col % p, py = (col / p) % p, c = col / (p * p);
+  const int wx = (int)(tok % w), hy = (int)((tok / w) % h);
+  const int64_t b = tok / ((int64_t)w * h);
+  out[i] = latent[((b * C + c) * H + hy * p + py) * W + wx * p + px];
+}
+
+// out[b, c, hy*p + py, wx*p + px] = x[b, hy*w + wx, (py*p + px)*C + c]
+__global__ void __launch_bounds__(256) unpatchify_kernel(const __bf16* __restrict__ x, __bf16* __restrict__ out,
+                                                         int64_t total, int C, int H, int W, int p) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int w = W / p, h = H / p;
+  const int X = (int)(i % W), Y = (int)((i / W) % H), c = (int)((i / ((int64_t)W * H)) % C);
+  const int64_t b = i / ((int64_t)W * H * C);
+  const int wx = X / p, px = X % p, hy = Y / p, py = Y % p;
+  out[i] = x[((b * h + hy) * w + wx) * (int64_t)(p * p * C) + (py * p + px) * C + c];
+}
+
+// out[b, :half] = cos(t[b] * f_i), out[b, half:] = sin(t[b] * f_i), f_i = exp(-ln(max_period) * i / half)
+__global__ void __launch_bounds__(256) timestep_embedding_kernel(const float* __restrict__ t, __bf16* __restrict__ out,
+                                                                 int batch, int dim, float max_period) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int half = dim / 2;
+  if (i >= batch * half) return;
+  const int b = i / half, k = i % half;
+  const float freq = expf(-logf(max_period) * (float)k / (float)half);
+  const float arg = t[b] * freq;
+  out[(int64_t)b * dim + k] = (__bf16)cosf(arg);
+  out[(int64_t)b * dim + half + k] = (__bf16)sinf(arg);
+}
+
+__global__ void __launch_bounds__(256) silu_kernel(const __bf16* __restrict__ x, __bf16* __restrict__ y, int64_t chunks) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= chunks) return;
+  float f[8];
+  unpack8(*(const i32x4*)(x + i * 8), f);
+#pragma unroll
+  for (int e = 0; e < 8; e++) f[e] = f[e] / (1.0f + expf(-f[e]));
+  *(i32x4*)(y + i * 8) = pack8(f);
+}
+
+__device__ __forceinline__ float round_bf16(float v) { return (float)(__bf16)v; }
+
+// Classifier-free guidance and the flow-match Euler update, in the rounding sequence of the bf16 tensor
+// expressions they replace:
+//   noise = uncond + s * (cond - uncond)                      (three bf16 tensor operations)
+//   x32 = float(sample); denoised = x32 - bf16(noise * sigma); derivative = (x32 - denoised) / sigma
+//   prev = bf16(x32 + derivative * (sigma_next - sigma))       (fp32 arithmetic, no fused multiply-add)
+__global__ void __launch_bounds__(256) cfg_euler_kernel(const __bf16* __restrict__ uncond, const __bf16* __restrict__ cond,
+                                                        const __bf16* __restrict__ sample, __bf16* __restrict__ out,
+                                                        int64_t total, float guidance, float sigma, float sigma_next) {
+#pragma clang fp contract(off)
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const float u = (float)uncond[i], c = (float)cond[i];
+  const float diff = round_bf16(c - u);
+  const float scaled = round_bf16(guidance * diff);
+  const float noise = round_bf16(u + scaled);
+  const float x = (float)sample[i];
+  const float denoised = x - round_bf16(noise * sigma);
+  const float derivative = (x - denoised) / sigma;
+  const float dt = sigma_next - sigma;
+  out[i] = (__bf16)(x + derivative * dt);
+}
+
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int hdit_patchify(const void* latent, void* out, int batch, int channels, int height, int width,
+                                             int patch, void* stream) {
+  if (batch < 0 || channels <= 0 || height <= 0 || width <= 0 || patch <= 0) return HDIT_EINVAL;
+  if (height % patch || width % patch) return HDIT_EINVAL;
+  const int64_t total = (int64_t)batch * channels * height * width;
+  if (total == 0) return HDIT_OK;
+  if (!latent || !out) return HDIT_EINVAL;
+  hipLaunchKernelGGL(patchify_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __bf16*)latent, (__bf16*)out, total, channels, height, width, patch);
+  return hdit_host::check_launch("hdit_patchify");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_unpatchify(const void* x, void* out, int batch, int channels, int height, int width,
+                                               int patch, void* stream) {
+  if (batch < 0 || channels <= 0 || height <= 0 || width <= 0 || patch <= 0) return HDIT_EINVAL;
+  if (height % patch || width % patch) return HDIT_EINVAL;
+  const int64_t total = (int64_t)batch * channels * height * width;
+  if (total == 0) return HDIT_OK;
+  if (!x || !out) return HDIT_EINVAL;
+  hipLaunchKernelGGL(unpatchify_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __bf16*)x, (__bf16*)out, total, channels, height, width, patch);
+  return hdit_host::check_launch("hdit_unpatchify");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_timestep_embedding(const float* timesteps, void* out, int batch, int dim,
+                                                       float max_period, void* stream) {
+  if (batch < 0 || dim <= 0 || dim % 2 || max_period <= 1.0f) return HDIT_EINVAL;
+  if (batch == 0) return HDIT_OK;
+  if (!timesteps || !out) return HDIT_EINVAL;
+  const int n = batch * (dim / 2);
+  hipLaunchKernelGGL(timestep_embedding_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     timesteps, (__bf16*)out, batch, dim, max_period);
+  return hdit_host::check_launch("hdit_timestep_embedding");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_silu(const void* x, void* y, int64_t count, void* stream) {
+  if (count < 0 || count % 8) return HDIT_EINVAL;
+  if (count == 0) return HDIT_OK;
+  if (!x || !y || !aligned16(x) || !aligned16(y)) return HDIT_EINVAL;
+  const int64_t chunks = count / 8;
+  hipLaunchKernelGGL(silu_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __bf16*)x, (__bf16*)y, chunks);
+  return hdit_host::check_launch("hdit_silu");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_cfg_euler_step(const void* noise_uncond, const void* noise_cond, const void* sample,
+                                                   void* out, int64_t count, float guidance, float sigma,
+                                                   float sigma_next, void* stream) {
+  if (count < 0 || !(sigma > 0.0f)) return HDIT_EINVAL;
+  if (count == 0) return HDIT_OK;
+  if (!noise_uncond || !noise_cond || !sample || !out) return HDIT_EINVAL;
+  hipLaunchKernelGGL(cfg_euler_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __bf16*)noise_uncond, (const __bf16*)noise_cond, (const __bf16*)sample, (__bf16*)out, count,
+                     guidance, sigma, sigma_next);
+  return hdit_host::check_launch("hdit_cfg_euler_step");
+}

@@ -36,6 +36,8 @@
 // workgroups so that the workgroups of one XCD (workgroup id mod 8; each XCD
 // has a private L2) own a contiguous, 8-tile-row-grouped range.
 #include <atomic>
+#include <cstdio>
+#include <cstdlib>
 #include <type_traits>
 
 #include "hdit_common.h"
@@ -658,6 +660,12 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
     const double t0 = tiles_time(pb, nb, 0), t3 = tiles_time(pb, nb, 3);
     big_cfg = t3 < t0 ? 3 : 0;
     two_cost = kLaunchUs + (t3 < t0 ? t3 : t0) + tiles_time(psm, ns, 2);
+  }
+  static const bool debug = getenv("HDIT_GEMM_DEBUG") != nullptr;
+  if (debug) {
+    fprintf(stderr, "hdit_gemm_bf16 plan:");
+    for (int i = 0; i < nlive; i++) fprintf(stderr, " [%dx%dx%d epi%d own%d]", live[i].m, live[i].n, live[i].k, live[i].epilogue, own[i]);
+    fprintf(stderr, " single cfg%d %.1f us, two-shape(big cfg%d) %.1f us\n", single, single_cost, big_cfg, two_cost);
   }
   if (two_cost < single_cost) {
     if (big_cfg == 0) return launch2<Cfg256x192, Cfg128x128>(big, nb, small, ns, s);

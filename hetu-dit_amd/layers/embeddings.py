@@ -1,0 +1,70 @@
+"""Patch-embedding wrapper with the interface of the reference's ``layers/embeddings.py:20-112``
+(``hetuDiTPatchEmbedWrapper``): projects the latent, adds the (cropped) position table, and in patch mode
+adds only the rows of the table that belong to the current pipeline patch.
+
+The p x p, stride-p convolution is a GEMM over the im2col rows (``hdit_patchify``); the position rows ride
+the GEMM's residual epilogue, so tokens leave the matrix core already position-encoded."""
+import torch
+
+from .. import ops
+from ..registry import hetuDiTLayerWrappersRegister
+from ..runtime_state import get_runtime_state
+from .base_layer import hetuDiTDiffusionLayerBaseWrapper
+from .modules import PatchEmbed
+
+
+@hetuDiTLayerWrappersRegister.register(PatchEmbed)
+class hetuDiTPatchEmbedWrapper(hetuDiTDiffusionLayerBaseWrapper):
+    def __init__(self, patch_embedding: PatchEmbed):
+        super().__init__(module=patch_embedding)
+        self._pos_cache = {}
+        self._ones = None
+
+    def _pos_rows(self, height: int, width: int, start: int, end: int, device) -> torch.Tensor:
+        """bf16 rows [start, end) of the table cropped for a latent of height x width pixels."""
+        key = (height, width, start, end, self.module.pos_embed.data_ptr())
+        rows = self._pos_cache.get(key)
+        if rows is None:
+            table = self.module.cropped_pos_embed(height, width)[0]
+            if end > table.shape[0]:
+                raise ValueError(f"pipeline patch ends at token {end} but the position table has {table.shape[0]} rows")
+            rows = table[start:end].to(device=device, dtype=torch.bfloat16).contiguous()
+            if len(self._pos_cache) >= 16:
+                self._pos_cache.clear()
+            self._pos_cache[key] = rows
+        return rows
+
+    @torch.no_grad()
+    def forward(self, latent: torch.Tensor) -> torch.Tensor:
+        m = self.module
+        rs = get_runtime_state()
+        p = m.patch_size
+        B, C, H, W = latent.shape
+        D = m.proj.weight.shape[0]
+        x = ops.patchify(latent.contiguous(), p)  # [B, T, C p p]
+        T = x.shape[1]
+        w2 = m.proj.weight.data.reshape(D, C * p * p)
+        bias = m.proj.bias.data if m.proj.bias is not None else None
+        out = torch.empty(B, T, D, dtype=torch.bfloat16, device=latent.device)
+        if m.pos_embed is None:
+            ops.gemm_launch([ops.gemm_problem(x.view(-1, C * p * p), w2, out.view(-1, D), bias)])
+            return out
+        if rs.patch_mode:
+            # the latent holds the rows of the current pipeline patch; the table is that of the whole image
+            if not rs.latents_height:
+                raise ValueError("patch mode needs the latent height of the whole image (runtime state set_patches)")
+            height = rs.latents_height
+            start, end = rs.pp_patches_token_start_end_idx_global[rs.pipeline_patch_idx]
+        else:
+            height, start, end = H, 0, T
+        if end - start != T:
+            raise ValueError(f"latent has {T} tokens but the pipeline patch covers {end - start}")
+        pos = self._pos_rows(height, W, start, end, latent.device)
+        if self._ones is None or self._ones.device != latent.device or self._ones.shape[1] != D:
+            self._ones = torch.ones(1, D, dtype=torch.float32, device=latent.device)
+        problems = [
+            ops.gemm_problem(x[b], w2, out[b], bias, ops.EPI_GATE_RESIDUAL, resid=pos, gate=self._ones, rows_per_batch=T)
+            for b in range(B)
+        ]
+        ops.gemm_launch(problems)
+        return out

@@ -151,3 +151,71 @@ class CogVideoXLayerNormZero(nn.Module):
         self.silu = nn.SiLU()
         self.linear = nn.Linear(conditioning_dim, 6 * embedding_dim, bias=True)
         self.norm = nn.LayerNorm(embedding_dim, eps=eps, elementwise_affine=True)
+
+
+def sincos_pos_embed_2d(embed_dim: int, grid_size: int, base_size: int, interpolation_scale: float = 1.0) -> torch.Tensor:
+    """diffusers ``get_2d_sincos_pos_embed``: [grid_size^2, embed_dim] fp32, first half of the channels from
+    the column coordinate, second half from the row coordinate, each [sin | cos] of pos * 10000^(-2i/d);
+    positions are scaled by base_size / grid_size."""
+    coord = torch.arange(grid_size, dtype=torch.float64) * (base_size / grid_size) / interpolation_scale
+    omega = 1.0 / 10000.0 ** (torch.arange(embed_dim // 4, dtype=torch.float64) / (embed_dim / 4.0))
+
+    def one_axis(pos):
+        ang = pos.reshape(-1)[:, None] * omega[None]
+        return torch.cat([ang.sin(), ang.cos()], dim=1)
+
+    cols = coord[None, :].expand(grid_size, grid_size)
+    rows = coord[:, None].expand(grid_size, grid_size)
+    return torch.cat([one_axis(cols), one_axis(rows)], dim=1).float()
+
+
+class PatchEmbed(nn.Module):
+    """diffusers ``PatchEmbed`` as SD3 configures it: p x p stride-p convolution, flatten, and a fixed sin-cos
+    position table of ``pos_embed_max_size``^2 entries that is centre-cropped to the latent's token grid."""
+
+    def __init__(self, height: int = 128, width: int = 128, patch_size: int = 2, in_channels: int = 16,
+                 embed_dim: int = 1536, pos_embed_max_size: int = 192):
+        super().__init__()
+        self.patch_size, self.height, self.width = patch_size, height // patch_size, width // patch_size
+        self.base_size = height // patch_size
+        self.pos_embed_max_size = pos_embed_max_size
+        self.flatten, self.layer_norm = True, False
+        self.proj = nn.Conv2d(in_channels, embed_dim, kernel_size=patch_size, stride=patch_size, bias=True)
+        table = sincos_pos_embed_2d(embed_dim, pos_embed_max_size, self.base_size)
+        self.register_buffer("pos_embed", table[None], persistent=True)
+
+    def cropped_pos_embed(self, height: int, width: int) -> torch.Tensor:
+        """[1, tokens, D] centre crop of the table for a latent of height x width pixels."""
+        height, width = height // self.patch_size, width // self.patch_size
+        m = self.pos_embed_max_size
+        if height > m or width > m:
+            raise ValueError(f"token grid {height}x{width} exceeds pos_embed_max_size {m}")
+        top, left = (m - height) // 2, (m - width) // 2
+        t = self.pos_embed.reshape(1, m, m, -1)[:, top : top + height, left : left + width]
+        return t.reshape(1, height * width, -1)
+
+
+class TimestepEmbedding(nn.Module):
+    def __init__(self, in_channels: int, time_embed_dim: int):
+        super().__init__()
+        self.linear_1 = nn.Linear(in_channels, time_embed_dim)
+        self.act = nn.SiLU()
+        self.linear_2 = nn.Linear(time_embed_dim, time_embed_dim)
+
+
+class PixArtAlphaTextProjection(nn.Module):
+    def __init__(self, in_features: int, hidden_size: int):
+        super().__init__()
+        self.linear_1 = nn.Linear(in_features, hidden_size)
+        self.act_1 = nn.SiLU()
+        self.linear_2 = nn.Linear(hidden_size, hidden_size)
+
+
+class CombinedTimestepTextProjEmbeddings(nn.Module):
+    """temb = timestep_embedder(sincos_256(t)) + text_embedder(pooled_projection)."""
+
+    def __init__(self, embedding_dim: int, pooled_projection_dim: int, frequency_dim: int = 256):
+        super().__init__()
+        self.frequency_dim = frequency_dim
+        self.timestep_embedder = TimestepEmbedding(frequency_dim, embedding_dim)
+        self.text_embedder = PixArtAlphaTextProjection(pooled_projection_dim, embedding_dim)

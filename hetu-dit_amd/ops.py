@@ -382,3 +382,57 @@ def copy_rows(src: torch.Tensor, dst: torch.Tensor):
     check(_lib.lib().hdit_copy_rows(src.data_ptr(), dst.data_ptr(), B, T, D, src.stride(0), src.stride(1), dst.stride(0),
                                     dst.stride(1), _stream()), "hdit_copy_rows")
     return dst
+
+
+def patchify(latent: torch.Tensor, patch: int) -> torch.Tensor:
+    """bf16 [B, C, H, W] -> [B, (H/p)(W/p), C p p]: rows for the patch-embedding GEMM."""
+    _need(latent, bf16, "latent")
+    if latent.dim() != 4 or not latent.is_contiguous():
+        raise ValueError("latent must be a contiguous [B, C, H, W] tensor")
+    B, Cc, H, W = latent.shape
+    out = torch.empty(B, (H // patch) * (W // patch), Cc * patch * patch, dtype=bf16, device=latent.device)
+    check(_lib.lib().hdit_patchify(latent.data_ptr(), out.data_ptr(), B, Cc, H, W, patch, _stream()), "hdit_patchify")
+    return out
+
+
+def unpatchify(x: torch.Tensor, channels: int, height: int, width: int, patch: int) -> torch.Tensor:
+    """bf16 [B, (H/p)(W/p), p p C] -> [B, C, H, W]."""
+    _need(x, bf16, "x")
+    B = x.shape[0]
+    if not x.is_contiguous() or tuple(x.shape) != (B, (height // patch) * (width // patch), patch * patch * channels):
+        raise ValueError("unpatchify input shape does not match the latent geometry")
+    out = torch.empty(B, channels, height, width, dtype=bf16, device=x.device)
+    check(_lib.lib().hdit_unpatchify(x.data_ptr(), out.data_ptr(), B, channels, height, width, patch, _stream()),
+          "hdit_unpatchify")
+    return out
+
+
+def timestep_embedding(timesteps: torch.Tensor, dim: int, max_period: float = 10000.0) -> torch.Tensor:
+    """f32 [B] -> bf16 [B, dim] = [cos | sin]."""
+    _need(timesteps, torch.float32, "timesteps")
+    t = timesteps.contiguous()
+    out = torch.empty(t.shape[0], dim, dtype=bf16, device=t.device)
+    check(_lib.lib().hdit_timestep_embedding(t.data_ptr(), out.data_ptr(), t.shape[0], dim, max_period, _stream()),
+          "hdit_timestep_embedding")
+    return out
+
+
+def silu(x: torch.Tensor) -> torch.Tensor:
+    _need(x, bf16, "x")
+    if not x.is_contiguous():
+        raise ValueError("silu input must be contiguous")
+    y = torch.empty_like(x)
+    check(_lib.lib().hdit_silu(x.data_ptr(), y.data_ptr(), x.numel(), _stream()), "hdit_silu")
+    return y
+
+
+def cfg_euler_step(noise_uncond, noise_cond, sample, guidance: float, sigma: float, sigma_next: float) -> torch.Tensor:
+    """bf16: sample + d/dsigma step of the guided prediction (see include/hdit.h)."""
+    for t, n in ((noise_uncond, "noise_uncond"), (noise_cond, "noise_cond"), (sample, "sample")):
+        _need(t, bf16, n)
+        if not t.is_contiguous() or t.shape != sample.shape:
+            raise ValueError("cfg_euler_step operands must be contiguous and of one shape")
+    out = torch.empty_like(sample)
+    check(_lib.lib().hdit_cfg_euler_step(noise_uncond.data_ptr(), noise_cond.data_ptr(), sample.data_ptr(), out.data_ptr(),
+                                         sample.numel(), guidance, sigma, sigma_next, _stream()), "hdit_cfg_euler_step")
+    return out

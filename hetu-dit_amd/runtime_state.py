@@ -15,6 +15,11 @@ class DiTRuntimeState:
         self.pp_patches_start_idx_local: List[int] = [0]
         self.pp_patches_token_start_idx_local: List[int] = [0]
         self.pp_patches_token_num: List[int] = []
+        # [start, end) token range of every pipeline patch within the whole image (runtime_state.py:106); with one
+        # sequence-parallel rank the global ranges are the local ones
+        self.pp_patches_token_start_end_idx_global: List[List[int]] = []
+        # latent rows of the whole image (the reference's input_config.height // vae_scale_factor); 0 = unknown
+        self.latents_height: int = 0
         self.max_condition_sequence_length: int = 0
         # forced False by the reference (runtime_state.py:188,:225)
         self.split_text_embed_in_sp: bool = False
@@ -58,6 +63,8 @@ class DiTRuntimeState:
         self.pp_patches_start_idx_local = starts
         self.pp_patches_token_start_idx_local = tok
         self.pp_patches_token_num = [tok[i + 1] - tok[i] for i in range(n)]
+        self.pp_patches_token_start_end_idx_global = [[tok[i], tok[i + 1]] for i in range(n)]
+        self.latents_height = latents_height
         self.pipeline_patch_idx = 0
 
     def set_token_patches(self, token_starts: List[int]):
@@ -65,6 +72,10 @@ class DiTRuntimeState:
         self.num_pipeline_patch = len(token_starts) - 1
         self.pp_patches_token_start_idx_local = list(token_starts)
         self.pp_patches_token_num = [token_starts[i + 1] - token_starts[i] for i in range(self.num_pipeline_patch)]
+        self.pp_patches_token_start_end_idx_global = [
+            [token_starts[i], token_starts[i + 1]] for i in range(self.num_pipeline_patch)
+        ]
+        self.latents_height = 0
         self.pipeline_patch_idx = 0
 
 

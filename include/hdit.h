@@ -194,6 +194,43 @@ int hdit_qk_norm_rope(const hdit_qknorm_job* jobs, int count, int batch, int hea
 int hdit_copy_rows(const void* src, void* dst, int batch, int tokens, int dim, int64_t src_sb,
                    int64_t src_st, int64_t dst_sb, int64_t dst_st, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Head and tail of a denoise step around the block stack (about a megabyte
+ * each; the projections between them are hdit_gemm_bf16 problems).
+ * ---------------------------------------------------------------------- */
+
+/* out[b, hy*(W/p) + wx, (c*p + py)*p + px] = latent[b, c, hy*p + py, wx*p + px]
+ * (bf16): the rows a p x p, stride-p convolution multiplies with its flattened
+ * weight [out, c*p*p], i.e. the A operand that turns `self.module.proj(latent)`
+ * + flatten + transpose of layers/embeddings.py:53-55 into a GEMM. */
+int hdit_patchify(const void* latent, void* out, int batch, int channels, int height, int width, int patch,
+                  void* stream);
+
+/* out[b, c, hy*p + py, wx*p + px] = x[b, hy*(W/p) + wx, (py*p + px)*C + c] (bf16):
+ * the reshape + einsum("nhwpqc->nchpwq") + reshape of
+ * models/transformers/transformer_sd3.py:160-182. */
+int hdit_unpatchify(const void* x, void* out, int batch, int channels, int height, int width, int patch,
+                    void* stream);
+
+/* out[b, :dim/2] = cos(t[b] f_i), out[b, dim/2:] = sin(t[b] f_i), f_i =
+ * max_period^(-i / (dim/2)); t f32 [batch], out bf16 [batch, dim].  diffusers
+ * Timesteps(flip_sin_to_cos=True, downscale_freq_shift=0) inside the
+ * time_text_embed called at transformer_sd3.py:101. */
+int hdit_timestep_embedding(const float* timesteps, void* out, int batch, int dim, float max_period, void* stream);
+
+/* y = silu(x) elementwise (bf16, count % 8 == 0): the activation between the
+ * two linears of the timestep / pooled-text embedders of the same module. */
+int hdit_silu(const void* x, void* y, int64_t count, void* stream);
+
+/* Classifier-free guidance fused with the flow-match Euler update (bf16 in/out,
+ * fp32 inside, in the rounding sequence of the tensor expressions replaced):
+ *   noise = uncond + guidance * (cond - uncond)
+ *     (model_executor/pipelines/pipeline_stable_diffusion_3.py:1703-1713)
+ *   out = sample + ((sample - (sample - noise * sigma)) / sigma) * (sigma_next - sigma)
+ *     (schedulers/scheduling_flow_match_euler_discrete.py:74-118 with gamma = 0) */
+int hdit_cfg_euler_step(const void* noise_uncond, const void* noise_cond, const void* sample, void* out,
+                        int64_t count, float guidance, float sigma, float sigma_next, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

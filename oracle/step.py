@@ -1,0 +1,128 @@
+"""CPU oracle (test infrastructure only) for the head and tail of an SD3 denoise step around the block
+stack: patch embedding with the cropped sin-cos position table, the timestep / pooled-text conditioning
+embedding, the context projection, ``norm_out`` + ``proj_out`` + unpatchify, classifier-free guidance and the
+flow-match Euler update.
+
+What the reference owns: the order of these calls (``hetu_dit/model_executor/diffusion_executor/models/
+transformers/transformer_sd3.py:92-185``), the patch-embedding wrapper (``.../layers/embeddings.py:32-112``),
+the guidance expression (``hetu_dit/model_executor/pipelines/pipeline_stable_diffusion_3.py:1703-1713``) and the
+scheduler step (``.../schedulers/scheduling_flow_match_euler_discrete.py:74-118``).  The modules it wraps
+(``PatchEmbed``, ``get_2d_sincos_pos_embed``, ``CombinedTimestepTextProjEmbeddings``, ``AdaLayerNormContinuous``)
+live in diffusers, which is absent: their published formulas are restated here.
+
+Pinning: ``patch_embed`` against ``F.conv2d``; ``unpatchify`` against the reference's reshape/einsum
+expression; ``timestep_embedding`` against the closed form (t = 0 gives [1.., 0..], first frequency is 1);
+``cfg_euler_step`` IS the reference's tensor expression sequence in bf16 / fp32 torch arithmetic.
+``sincos_pos_embed_2d`` (which axis comes first, the base_size scaling, the centre crop) and the order of
+the [cos | sin] halves are **parity unpinned**: only an import of diffusers could confirm them.
+"""
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import ops as O
+
+P = Dict[str, torch.Tensor]
+
+
+def patch_embed(latent: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, pos_embed: Optional[torch.Tensor]) -> torch.Tensor:
+    """latent [B, C, H, W], conv weight [D, C, p, p] (stride p) -> tokens [B, (H/p)(W/p), D] (+ pos_embed [T, D])."""
+    B, C, H, W = latent.shape
+    D, _, p, _ = weight.shape
+    x = latent.float().reshape(B, C, H // p, p, W // p, p).permute(0, 2, 4, 1, 3, 5).reshape(B, (H // p) * (W // p), C * p * p)
+    tok = O.linear(x, weight.float().reshape(D, C * p * p), bias)
+    if pos_embed is not None:
+        tok = tok + pos_embed.float()[None]
+    return tok
+
+
+def _sincos_1d(embed_dim: int, pos: torch.Tensor) -> torch.Tensor:
+    omega = torch.arange(embed_dim // 2, dtype=torch.float64) / (embed_dim / 2.0)
+    omega = 1.0 / 10000.0 ** omega
+    out = pos.reshape(-1).double()[:, None] * omega[None]
+    return torch.cat([out.sin(), out.cos()], dim=1)
+
+
+def sincos_pos_embed_2d(embed_dim: int, grid_size: int, base_size: int, interpolation_scale: float = 1.0) -> torch.Tensor:
+    """[grid_size^2, embed_dim] fp32 table; positions scaled by base_size / grid_size."""
+    coord = torch.arange(grid_size, dtype=torch.float64) / (grid_size / base_size) / interpolation_scale
+    gw, gh = torch.meshgrid(coord, coord, indexing="xy")  # gw varies along the row (w first)
+    emb_a = _sincos_1d(embed_dim // 2, gw)
+    emb_b = _sincos_1d(embed_dim // 2, gh)
+    return torch.cat([emb_a, emb_b], dim=1).float()
+
+
+def cropped_pos_embed(table: torch.Tensor, max_size: int, height: int, width: int) -> torch.Tensor:
+    """Centre crop of the [max_size^2, D] table to [height*width, D]."""
+    top, left = (max_size - height) // 2, (max_size - width) // 2
+    t = table.reshape(max_size, max_size, -1)[top : top + height, left : left + width]
+    return t.reshape(height * width, -1)
+
+
+def timestep_embedding(t: torch.Tensor, dim: int, max_period: float = 10000.0) -> torch.Tensor:
+    half = dim // 2
+    freq = torch.exp(-math.log(max_period) * torch.arange(half, dtype=torch.float32) / half)
+    arg = t.float()[:, None] * freq[None]
+    return torch.cat([arg.cos(), arg.sin()], dim=1)
+
+
+def combined_timestep_text_embed(p: P, prefix: str, timestep: torch.Tensor, pooled: torch.Tensor, freq_dim: int = 256) -> torch.Tensor:
+    """temb = linear_2(silu(linear_1(sincos(t)))) + linear_2(silu(linear_1(pooled)))."""
+    tp = timestep_embedding(timestep, freq_dim)
+    te = O.linear(O.silu(O.linear(tp, p[prefix + "timestep_embedder.linear_1.weight"], p[prefix + "timestep_embedder.linear_1.bias"])),
+                  p[prefix + "timestep_embedder.linear_2.weight"], p[prefix + "timestep_embedder.linear_2.bias"])
+    pe = O.linear(O.silu(O.linear(pooled.float(), p[prefix + "text_embedder.linear_1.weight"], p[prefix + "text_embedder.linear_1.bias"])),
+                  p[prefix + "text_embedder.linear_2.weight"], p[prefix + "text_embedder.linear_2.bias"])
+    return te + pe
+
+
+def norm_out_proj(p: P, hidden: torch.Tensor, temb: torch.Tensor) -> torch.Tensor:
+    """AdaLayerNormContinuous (scale first) then proj_out."""
+    scale, shift = O.adaln_modulation(temb, p["norm_out.linear.weight"], p["norm_out.linear.bias"], 2)
+    x = O.modulate(O.layer_norm(hidden, 1e-6), shift, scale)
+    return O.linear(x, p["proj_out.weight"], p["proj_out.bias"])
+
+
+def unpatchify(x: torch.Tensor, channels: int, height: int, width: int, patch: int) -> torch.Tensor:
+    """transformer_sd3.py:160-182: [B, h*w, p*p*C] -> [B, C, h*p, w*p]."""
+    B = x.shape[0]
+    h, w = height // patch, width // patch
+    x = x.reshape(B, h, w, patch, patch, channels)
+    x = torch.einsum("nhwpqc->nchpwq", x)
+    return x.reshape(B, channels, h * patch, w * patch)
+
+
+def cfg_euler_step(noise_uncond: torch.Tensor, noise_cond: torch.Tensor, sample: torch.Tensor, guidance: float,
+                   sigma: float, sigma_next: float) -> torch.Tensor:
+    """The reference's expressions on bf16 tensors (each tensor operation rounds to bf16; the scheduler works
+    in fp32 with 0-dim fp32 sigmas)."""
+    u, c, x = noise_uncond.bfloat16(), noise_cond.bfloat16(), sample.bfloat16()
+    noise = u + guidance * (c - u)
+    sig, sig_next = torch.tensor(sigma, dtype=torch.float32), torch.tensor(sigma_next, dtype=torch.float32)
+    x32 = x.to(torch.float32)
+    denoised = x32 - noise * sig
+    derivative = (x32 - denoised) / sig
+    prev = x32 + derivative * (sig_next - sig)
+    return prev.to(torch.bfloat16)
+
+
+def sd3_transformer(p: P, latent: torch.Tensor, encoder: torch.Tensor, pooled: torch.Tensor, timestep: torch.Tensor,
+                    heads: int, layers: int, patch: int, pos_embed_max_size: int) -> torch.Tensor:
+    """transformer_sd3.py:92-185 outside patch mode: latent [B, C, H, W] -> predicted noise [B, C_out, H, W].
+    ``p`` uses the unwrapped parameter names (``pos_embed.proj.weight``, ``pos_embed.pos_embed`` [1, max^2, D],
+    ``time_text_embed.*``, ``context_embedder.*``, ``transformer_blocks.N.*``, ``norm_out.linear.*``, ``proj_out.*``)."""
+    from . import blocks as BL
+
+    B, _, H, W = latent.shape
+    pos = cropped_pos_embed(p["pos_embed.pos_embed"][0], pos_embed_max_size, H // patch, W // patch)
+    hidden = patch_embed(latent, p["pos_embed.proj.weight"], p["pos_embed.proj.bias"], pos)
+    temb = combined_timestep_text_embed(p, "time_text_embed.", timestep, pooled)
+    enc = O.linear(encoder.float(), p["context_embedder.weight"], p["context_embedder.bias"])
+    for i in range(layers):
+        pre = f"transformer_blocks.{i}."
+        bp = {k[len(pre):]: v for k, v in p.items() if k.startswith(pre)}
+        enc, hidden = BL.sd3_joint_block(bp, hidden, enc, temb, heads, context_pre_only=(i == layers - 1))
+    out = norm_out_proj(p, hidden, temb)
+    channels = p["proj_out.weight"].shape[0] // (patch * patch)
+    return unpatchify(out, channels, H, W, patch)

@@ -1,0 +1,149 @@
+"""Head and tail of an SD3 denoise step on the HIP path against the oracle: patchify / unpatchify (bit-exact
+data movement), timestep projection, SiLU, guidance + Euler update (bit-exact against the bf16 / fp32 tensor
+expressions), the patch-embedding wrapper with and without pipeline patches, and the whole transformer
+from latent to predicted noise."""
+import pytest
+import torch
+
+from oracle import step as S
+from tests.util import assert_parity
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(autouse=True)
+def fresh_state():
+    from hetu_dit_amd.cache_manager import reset_cache_manager
+    from hetu_dit_amd.runtime_state import reset_runtime_state
+
+    reset_runtime_state()
+    yield
+    reset_cache_manager()
+    reset_runtime_state()
+
+
+def step_params(model) -> dict:
+    """fp32 parameters and buffers under the unwrapped names the oracle uses."""
+    from tests.util import oracle_params
+
+    out = {}
+    for i, blk in enumerate(model.transformer_blocks):
+        for k, v in oracle_params(blk).items():
+            out[f"transformer_blocks.{i}.{k}"] = v
+    for name, p in list(model.named_parameters()) + list(model.named_buffers()):
+        if not name.startswith("transformer_blocks."):
+            out[name.replace(".module.", ".")] = p.detach().float().cpu()
+    return out
+
+
+@pytest.mark.parametrize("B,C,H,W,p", [(2, 16, 32, 48, 2), (1, 3, 8, 16, 4), (3, 5, 6, 6, 1), (1, 16, 128, 128, 2)])
+def test_patchify_unpatchify_exact(hdit, B, C, H, W, p):
+    print(f"patchify {B} {C} {H} {W} {p}", flush=True)
+    ops = hdit.ops
+    torch.manual_seed(0)
+    lat = torch.randn(B, C, H, W).bfloat16()
+    got = ops.patchify(lat.to(DEV), p)
+    want = lat.reshape(B, C, H // p, p, W // p, p).permute(0, 2, 4, 1, 3, 5).reshape(B, (H // p) * (W // p), C * p * p)
+    assert torch.equal(got.cpu(), want)
+    x = torch.randn(B, (H // p) * (W // p), p * p * C).bfloat16()
+    got = ops.unpatchify(x.to(DEV), C, H, W, p)
+    assert torch.equal(got.cpu(), S.unpatchify(x, C, H, W, p))
+
+
+def test_patchify_refuses_ragged_grid(hdit):
+    from hetu_dit_amd._lib import HditError
+
+    with pytest.raises((HditError, ValueError)):
+        hdit.ops.patchify(torch.zeros(1, 4, 7, 8, dtype=torch.bfloat16, device=DEV), 2)
+    assert hdit.ops.patchify(torch.zeros(0, 4, 8, 8, dtype=torch.bfloat16, device=DEV), 2).shape == (0, 16, 16)
+
+
+def test_timestep_embedding_and_silu(hdit):
+    ops = hdit.ops
+    t = torch.tensor([0.0, 1.0, 17.5, 500.0, 999.0, 1000.0])
+    got = ops.timestep_embedding(t.to(DEV), 256).float().cpu()
+    want = S.timestep_embedding(t, 256)
+    # bf16 rounding of values in [-1, 1]: absolute error below 2^-9
+    assert (got - want).abs().max() < 2.0 ** -8
+    assert_parity(got, want, what="timestep embedding")
+    assert torch.equal(got[0, :128], torch.ones(128)) and torch.equal(got[0, 128:], torch.zeros(128))
+    x = (torch.randn(7, 1536) * 3).bfloat16()
+    y = ops.silu(x.to(DEV))
+    assert_parity(y, torch.nn.functional.silu(x.float()), rel=4e-3, what="silu")
+
+
+@pytest.mark.parametrize("guidance,sigma,sigma_next", [(7.0, 1.0, 0.9644), (4.5, 0.3127, 0.25), (1.0, 0.0421, 0.0), (0.0, 0.5, 0.5)])
+def test_cfg_euler_step_bit_exact(hdit, guidance, sigma, sigma_next):
+    torch.manual_seed(3)
+    u, c, x = (torch.randn(2, 16, 64, 64).bfloat16() for _ in range(3))
+    got = hdit.ops.cfg_euler_step(u.to(DEV), c.to(DEV), x.to(DEV), guidance, sigma, sigma_next)
+    want = S.cfg_euler_step(u, c, x, guidance, sigma, sigma_next)
+    assert torch.equal(got.cpu(), want)
+
+
+def test_patch_embed_wrapper_full_and_patches(hdit):
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.layers.embeddings import hetuDiTPatchEmbedWrapper
+    from hetu_dit_amd.layers.modules import PatchEmbed
+    from hetu_dit_amd.registry import hetuDiTLayerWrappersRegister
+    from hetu_dit_amd.runtime_state import get_runtime_state
+
+    pe = PatchEmbed(64, 64, 2, 16, 256, pos_embed_max_size=48)
+    synthetic.init_module_(pe, 5)
+    assert hetuDiTLayerWrappersRegister.get_wrapper(pe) is hetuDiTPatchEmbedWrapper
+    wrap = hetuDiTPatchEmbedWrapper(pe).to(DEV)
+    w, b = pe.proj.weight.detach().float().cpu(), pe.proj.bias.detach().float().cpu()
+    table = pe.pos_embed[0].float().cpu()
+    lat = synthetic.randn_bf16((2, 16, 48, 40), 6)  # 24 x 20 tokens, not the module's own 32 x 32
+    want = S.patch_embed(lat.float(), w, b, S.cropped_pos_embed(table, 48, 24, 20))
+    got = wrap(lat.to(DEV))
+    assert_parity(got, want, what="patch embed (full image)")
+
+    # pipeline patches: rows [0, 16), [16, 32), [32, 48) of the latent get rows of the whole image's table
+    rs = get_runtime_state()
+    rs.set_patches(48, 40, 2, 3)
+    rs.set_patched_mode(True)
+    for i in range(rs.num_pipeline_patch):
+        r0, r1 = rs.pp_patches_start_idx_local[i], rs.pp_patches_start_idx_local[i + 1]
+        t0, t1 = rs.pp_patches_token_start_end_idx_global[i]
+        got = wrap(lat[:, :, r0:r1].contiguous().to(DEV))
+        assert_parity(got, want[:, t0:t1], what=f"patch embed (pipeline patch {i})")
+        rs.next_patch()
+    rs.set_patched_mode(False)
+    with pytest.raises(ValueError):
+        wrap(torch.zeros(1, 16, 100, 40, dtype=torch.bfloat16, device=DEV))  # 50 token rows > max 48
+
+
+def test_sd3_transformer_latent_to_noise(hdit):
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.transformer_sd3 import SD3Transformer2DModel
+
+    L, heads = 3, 4
+    model = SD3Transformer2DModel(sample_size=32, patch_size=2, in_channels=16, num_layers=L, attention_head_dim=64,
+                                  num_attention_heads=heads, joint_attention_dim=128, caption_projection_dim=256,
+                                  pooled_projection_dim=64, out_channels=16, pos_embed_max_size=24)
+    synthetic.init_module_(model, 7)
+    params = step_params(model)
+    model = model.to(DEV)
+    B = 2
+    lat = synthetic.randn_bf16((B, 16, 32, 40), 8)
+    enc = synthetic.randn_bf16((B, 77, 128), 9)
+    pooled = synthetic.randn_bf16((B, 64), 10)
+    t = torch.tensor([981.0, 981.0])
+    got = model(lat.to(DEV), enc.to(DEV), pooled.to(DEV), t.to(DEV))
+    torch.cuda.synchronize()
+    want = S.sd3_transformer(params, lat.float(), enc.float(), pooled.float(), t, heads, L, 2, 24)
+    assert got.shape == lat.shape
+    assert_parity(got, want, what="sd3 transformer")
+
+    # conditioning vector on its own
+    temb = model.conditioning(t.to(DEV), pooled.to(DEV))
+    assert_parity(temb, S.combined_timestep_text_embed(params, "time_text_embed.", t, pooled.float()), what="temb")
+
+    # one guided step: [uncond, cond] batch, guidance and Euler update against the oracle's expressions
+    lat1 = lat[:1]
+    new = model.denoise_step(lat1.to(DEV), enc.to(DEV), pooled.to(DEV), t[:1].to(DEV), 7.0, 0.981, 0.95)
+    noise = S.sd3_transformer(params, torch.cat([lat1, lat1]).float(), enc.float(), pooled.float(), t, heads, L, 2, 24)
+    want = S.cfg_euler_step(noise[:1], noise[1:], lat1, 7.0, 0.981, 0.95)
+    assert_parity(new, want.float(), what="denoise step")
