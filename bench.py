@@ -57,7 +57,7 @@ def randomize_(module, device, seed=0):
     return module
 
 
-WORKLOADS = ("sd3_1024", "sd3_pipefusion", "flux_1024", "cogvideox_5b")
+WORKLOADS = ("sd3_1024", "sd3_1024_transformer", "sd3_pipefusion", "flux_1024", "cogvideox_5b")
 
 
 def make_workload(name, dev):
@@ -69,10 +69,27 @@ def make_workload(name, dev):
     from hetu_dit_amd import synthetic, transformer
     from hetu_dit_amd.runtime_state import get_runtime_state, reset_runtime_state
 
-    cfg = synthetic.CONFIGS[name]
     reset_runtime_state()
     gen = torch.Generator(device=dev).manual_seed(1)
     rnd = lambda *shape: torch.randn(*shape, generator=gen, device=dev).to(torch.bfloat16)
+    if name == "sd3_1024_transformer":
+        # the same 24 blocks inside the whole transformer: latent in, guided and Euler-updated latent out
+        from hetu_dit_amd.transformer_sd3 import SD3Transformer2DModel
+
+        cfg = synthetic.CONFIGS["sd3_1024"]
+        with torch.device(dev):
+            model = SD3Transformer2DModel()  # SD3-medium geometry: 128 x 128 x 16 latent, patch 2, text 4096 -> 1536
+        randomize_(model, dev)
+        lat, enc, pooled = rnd(1, 16, 128, 128), rnd(2, cfg["n_txt"], 4096), rnd(2, 2048)
+        ts = torch.full((1,), 981.0, device=dev)
+        gemm, attn = algorithmic_flops(cfg)
+        D, T, Nt = cfg["dim"], cfg["n_img"], cfg["n_txt"]
+        gemm += 2.0 * 2 * (T * 64 * D * 2 + Nt * 4096 * D + 256 * D + D * D + 2048 * D + D * D)
+        desc = ("configs[1] inside the whole SD3 transformer: patch embedding + position table, timestep/text conditioning, "
+                "context projection, 24 joint blocks, norm_out + proj_out + unpatchify, guidance 7.0 and the Euler update")
+        return (lambda: model.denoise_step(lat, enc, pooled, ts, 7.0, 0.981, 0.95)), desc, gemm, attn, cfg["layers"], \
+            "attn_fwd_kernel<64>"
+    cfg = synthetic.CONFIGS[name]
     B, Ni, Nt, D = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"]
     S = Ni + Nt
     if name in ("sd3_1024", "sd3_pipefusion"):

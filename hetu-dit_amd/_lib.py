@@ -126,6 +126,10 @@ SIGNATURES = {
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_float, C.c_float, C.c_void_p],
     ),
+    "hdit_rope_table": (
+        C.c_int,
+        [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int, C.c_double, C.c_void_p, C.c_void_p, C.c_void_p],
+    ),
     "hdit_copy_rows": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_void_p],

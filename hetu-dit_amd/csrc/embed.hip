@@ -60,6 +60,30 @@ __global__ void __launch_bounds__(256) silu_kernel(const __bf16* __restrict__ x,
   *(i32x4*)(y + i * 8) = pack8(f);
 }
 
+struct RopeAxes {
+  int n;
+  int dim[HDIT_ROPE_MAX_AXES];
+};
+
+// cos/sin[row, off_a + 2i] = cos/sin[row, off_a + 2i + 1] = cos/sin(pos[row, a] * theta^(-2i / dim_a)), in float64
+// like the table it replaces, stored as f32; one thread per rotation pair
+__global__ void __launch_bounds__(256) rope_table_kernel(const float* __restrict__ pos, float* __restrict__ cos_out,
+                                                         float* __restrict__ sin_out, int rows, RopeAxes ax, int width,
+                                                         double theta) {
+  const int pairs = width / 2;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)rows * pairs) return;
+  const int row = (int)(i / pairs);
+  int pr = (int)(i % pairs), a = 0;
+  while (pr >= ax.dim[a] / 2) pr -= ax.dim[a++] / 2;  // ax.dim sums to width, so a stays below ax.n
+  const double freq = 1.0 / pow(theta, (double)(2 * pr) / (double)ax.dim[a]);
+  const double ang = (double)pos[(int64_t)row * ax.n + a] * freq;
+  const float c = (float)cos(ang), sn = (float)sin(ang);
+  const int64_t o = (int64_t)row * width + (i % pairs) * 2;
+  *(float2*)(cos_out + o) = make_float2(c, c);
+  *(float2*)(sin_out + o) = make_float2(sn, sn);
+}
+
 __device__ __forceinline__ float round_bf16(float v) { return (float)(__bf16)v; }
 
 // Classifier-free guidance and the flow-match Euler update, in the rounding sequence of the bf16 tensor
@@ -141,4 +165,23 @@ extern "C" __attribute__((visibility("default"))) int hdit_cfg_euler_step(const 
                      (const __bf16*)noise_uncond, (const __bf16*)noise_cond, (const __bf16*)sample, (__bf16*)out, count,
                      guidance, sigma, sigma_next);
   return hdit_host::check_launch("hdit_cfg_euler_step");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_rope_table(const float* positions, int rows, const int* axes_dim, int n_axes,
+                                               double theta, float* cos_out, float* sin_out, void* stream) {
+  if (rows < 0 || !axes_dim || n_axes <= 0 || n_axes > HDIT_ROPE_MAX_AXES || !(theta > 1.0)) return HDIT_EINVAL;
+  RopeAxes ax{};
+  ax.n = n_axes;
+  int width = 0;
+  for (int a = 0; a < n_axes; a++) {
+    if (axes_dim[a] <= 0 || axes_dim[a] % 2) return HDIT_EINVAL;
+    ax.dim[a] = axes_dim[a];
+    width += axes_dim[a];
+  }
+  if (rows == 0) return HDIT_OK;
+  if (!positions || !cos_out || !sin_out || (((uintptr_t)cos_out | (uintptr_t)sin_out) & 7)) return HDIT_EINVAL;
+  const int64_t n = (int64_t)rows * (width / 2);
+  hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, positions,
+                     cos_out, sin_out, rows, ax, width, theta);
+  return hdit_host::check_launch("hdit_rope_table");
 }

@@ -68,3 +68,51 @@ class hetuDiTPatchEmbedWrapper(hetuDiTDiffusionLayerBaseWrapper):
         ]
         ops.gemm_launch(problems)
         return out
+
+
+def project(x2: torch.Tensor, lin, **epilogue) -> torch.Tensor:
+    """bf16 [m, k] -> [m, n] through one launch of the grouped GEMM (bias in the epilogue)."""
+    out = torch.empty(x2.shape[0], lin.weight.shape[0], dtype=torch.bfloat16, device=x2.device)
+    ops.gemm_launch([ops.gemm_problem(x2, lin.weight.data, out, lin.bias.data, **epilogue)])
+    return out
+
+
+def conditioning_embedding(tte, timestep: torch.Tensor, pooled_projection: torch.Tensor, guidance=None) -> torch.Tensor:
+    """bf16 [B, D] conditioning vector of ``CombinedTimestepTextProjEmbeddings`` /
+    ``CombinedTimestepGuidanceTextProjEmbeddings`` (called at ``transformer_sd3.py:101`` and
+    ``transformer_flux.py:108-112``): each embedder is linear -> SiLU -> linear; the sum of the embedders
+    rides the residual epilogue of the second linears."""
+    B = timestep.shape[0]
+    D = tte.timestep_embedder.linear_2.weight.shape[0]
+    ones = getattr(tte, "_unit_gate", None)
+    if ones is None or ones.device != timestep.device:
+        ones = torch.ones(1, D, dtype=torch.float32, device=timestep.device)
+        object.__setattr__(tte, "_unit_gate", ones)
+    acc = None
+
+    def add(embedder_in: torch.Tensor, lin1, lin2):
+        nonlocal acc
+        h = ops.silu(project(embedder_in, lin1))
+        if acc is None:
+            acc = project(h, lin2)
+        else:
+            acc = project(h, lin2, epilogue=ops.EPI_GATE_RESIDUAL, resid=acc, gate=ones, rows_per_batch=B)
+
+    add(ops.timestep_embedding(timestep.to(torch.float32), tte.frequency_dim), tte.timestep_embedder.linear_1,
+        tte.timestep_embedder.linear_2)
+    if guidance is not None:
+        add(ops.timestep_embedding(guidance.to(torch.float32), tte.frequency_dim), tte.guidance_embedder.linear_1,
+            tte.guidance_embedder.linear_2)
+    add(pooled_projection.contiguous(), tte.text_embedder.linear_1, tte.text_embedder.linear_2)
+    return acc
+
+
+def norm_out_project(norm_out, proj_out, hidden_states: torch.Tensor, temb: torch.Tensor) -> torch.Tensor:
+    """``proj_out(norm_out(hidden_states, temb))`` (``transformer_sd3.py:156-157``, ``transformer_flux.py:203-205``):
+    AdaLayerNormContinuous (chunk order scale, shift) fused into one normalise-and-modulate pass, then a GEMM."""
+    from ..blocks import _adaln
+
+    scale, shift = _adaln(norm_out, temb)
+    x = ops.layernorm_modulate(hidden_states, shift, scale, norm_out.norm.eps)
+    B, T, D = x.shape
+    return project(x.view(-1, D), proj_out).view(B, T, -1)

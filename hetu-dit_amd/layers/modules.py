@@ -219,3 +219,22 @@ class CombinedTimestepTextProjEmbeddings(nn.Module):
         self.frequency_dim = frequency_dim
         self.timestep_embedder = TimestepEmbedding(frequency_dim, embedding_dim)
         self.text_embedder = PixArtAlphaTextProjection(pooled_projection_dim, embedding_dim)
+
+
+class CombinedTimestepGuidanceTextProjEmbeddings(nn.Module):
+    """temb = timestep_embedder(sincos_256(t)) + guidance_embedder(sincos_256(g)) + text_embedder(pooled)."""
+
+    def __init__(self, embedding_dim: int, pooled_projection_dim: int, frequency_dim: int = 256):
+        super().__init__()
+        self.frequency_dim = frequency_dim
+        self.timestep_embedder = TimestepEmbedding(frequency_dim, embedding_dim)
+        self.guidance_embedder = TimestepEmbedding(frequency_dim, embedding_dim)
+        self.text_embedder = PixArtAlphaTextProjection(pooled_projection_dim, embedding_dim)
+
+
+class FluxPosEmbed(nn.Module):
+    """Rotary table from (text | image) position ids, one rotary axis per id column."""
+
+    def __init__(self, theta: float = 10000.0, axes_dim=(16, 56, 56)):
+        super().__init__()
+        self.theta, self.axes_dim = theta, tuple(axes_dim)

@@ -436,3 +436,18 @@ def cfg_euler_step(noise_uncond, noise_cond, sample, guidance: float, sigma: flo
     check(_lib.lib().hdit_cfg_euler_step(noise_uncond.data_ptr(), noise_cond.data_ptr(), sample.data_ptr(), out.data_ptr(),
                                          sample.numel(), guidance, sigma, sigma_next, _stream()), "hdit_cfg_euler_step")
     return out
+
+
+def rope_table(positions: torch.Tensor, axes_dim, theta: float = 10000.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """f32 positions [S, len(axes_dim)] -> (cos, sin) f32 [S, sum(axes_dim)], the ``image_rotary_emb`` the blocks take."""
+    _need(positions, torch.float32, "positions")
+    axes = [int(a) for a in axes_dim]
+    if positions.dim() != 2 or positions.shape[1] != len(axes) or not positions.is_contiguous():
+        raise ValueError("positions must be a contiguous [tokens, axes] tensor with one column per rotary axis")
+    rows = positions.shape[0]
+    cos = torch.empty(rows, sum(axes), dtype=torch.float32, device=positions.device)
+    sin = torch.empty_like(cos)
+    arr = (C.c_int * len(axes))(*axes)
+    check(_lib.lib().hdit_rope_table(positions.data_ptr(), rows, arr, len(axes), float(theta), cos.data_ptr(), sin.data_ptr(),
+                                     _stream()), "hdit_rope_table")
+    return cos, sin

@@ -5,14 +5,11 @@ blocks, ``norm_out`` / ``proj_out`` and unpatchify -- plus the guidance and sche
 the pipeline (``pipeline_stable_diffusion_3.py:1703-1713``,
 ``schedulers/scheduling_flow_match_euler_discrete.py:74-118``).  Every projection is a launch of the grouped
 GEMM; the small glue steps have their own kernels (``csrc/embed.hip``)."""
-from typing import Optional
-
 import torch
 from torch import nn
 
 from . import ops
-from .blocks import _adaln
-from .layers.embeddings import hetuDiTPatchEmbedWrapper
+from .layers.embeddings import conditioning_embedding, hetuDiTPatchEmbedWrapper, norm_out_project, project
 from .layers.modules import AdaLayerNormContinuous, CombinedTimestepTextProjEmbeddings, PatchEmbed
 from .transformer import SD3TransformerBlocks
 
@@ -34,25 +31,9 @@ class SD3Transformer2DModel(nn.Module):
         self.transformer_blocks = self._runner.transformer_blocks
         self.norm_out = AdaLayerNormContinuous(D, D, eps=1e-6)
         self.proj_out = nn.Linear(D, patch_size * patch_size * out_channels)
-        self._ones: Optional[torch.Tensor] = None
-
-    def _linear(self, x2: torch.Tensor, lin: nn.Linear, **epilogue) -> torch.Tensor:
-        out = torch.empty(x2.shape[0], lin.weight.shape[0], dtype=torch.bfloat16, device=x2.device)
-        ops.gemm_launch([ops.gemm_problem(x2, lin.weight.data, out, lin.bias.data, **epilogue)])
-        return out
 
     def conditioning(self, timestep: torch.Tensor, pooled_projections: torch.Tensor) -> torch.Tensor:
-        """bf16 [B, D]: timestep_embedder(sincos(t)) + text_embedder(pooled); the sum rides the last GEMM's
-        residual epilogue."""
-        tte = self.time_text_embed
-        B = timestep.shape[0]
-        if self._ones is None or self._ones.device != timestep.device:
-            self._ones = torch.ones(1, self.inner_dim, dtype=torch.float32, device=timestep.device)
-        t_proj = ops.timestep_embedding(timestep.to(torch.float32), tte.frequency_dim)
-        t_emb = self._linear(ops.silu(self._linear(t_proj, tte.timestep_embedder.linear_1)), tte.timestep_embedder.linear_2)
-        h = ops.silu(self._linear(pooled_projections.contiguous(), tte.text_embedder.linear_1))
-        return self._linear(h, tte.text_embedder.linear_2, epilogue=ops.EPI_GATE_RESIDUAL, resid=t_emb, gate=self._ones,
-                            rows_per_batch=B)
+        return conditioning_embedding(self.time_text_embed, timestep, pooled_projections)
 
     @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, pooled_projections: torch.Tensor,
@@ -63,11 +44,9 @@ class SD3Transformer2DModel(nn.Module):
         tokens = self.pos_embed(hidden_states)
         temb = self.conditioning(timestep, pooled_projections)
         enc = encoder_hidden_states.contiguous()
-        enc = self._linear(enc.view(-1, enc.shape[-1]), self.context_embedder).view(B, enc.shape[1], -1)
+        enc = project(enc.view(-1, enc.shape[-1]), self.context_embedder).view(B, enc.shape[1], -1)
         tokens = self._runner(tokens, enc, temb)
-        scale, shift = _adaln(self.norm_out, temb)  # AdaLayerNormContinuous: scale first
-        x = ops.layernorm_modulate(tokens, shift, scale, self.norm_out.norm.eps)
-        x = self._linear(x.view(-1, self.inner_dim), self.proj_out).view(B, tokens.shape[1], -1)
+        x = norm_out_project(self.norm_out, self.proj_out, tokens, temb)
         return ops.unpatchify(x, self.out_channels, H, W, self.patch_size)
 
     @torch.no_grad()

@@ -199,6 +199,16 @@ int hdit_copy_rows(const void* src, void* dst, int batch, int tokens, int dim, i
  * each; the projections between them are hdit_gemm_bf16 problems).
  * ---------------------------------------------------------------------- */
 
+/* Rotary table from token positions: positions f32 [rows, n_axes]; per axis a
+ * of width axes_dim[a] (even), angle = pos * theta^(-2i / axes_dim[a]) in float64,
+ * each value written twice (rotation pair), axes concatenated: cos_out, sin_out
+ * f32 [rows, sum(axes_dim)].  This is `self.pos_embed(ids)` of
+ * models/transformers/transformer_flux.py:130-131 (axes (16, 56, 56) over
+ * (0, row, col) ids) and the table the CogVideoX pipeline hands its blocks. */
+#define HDIT_ROPE_MAX_AXES 4
+int hdit_rope_table(const float* positions, int rows, const int* axes_dim, int n_axes, double theta, float* cos_out,
+                    float* sin_out, void* stream);
+
 /* out[b, hy*(W/p) + wx, (c*p + py)*p + px] = latent[b, c, hy*p + py, wx*p + px]
  * (bf16): the rows a p x p, stride-p convolution multiplies with its flattened
  * weight [out, c*p*p], i.e. the A operand that turns `self.module.proj(latent)`

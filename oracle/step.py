@@ -13,8 +13,11 @@ live in diffusers, which is absent: their published formulas are restated here.
 Pinning: ``patch_embed`` against ``F.conv2d``; ``unpatchify`` against the reference's reshape/einsum
 expression; ``timestep_embedding`` against the closed form (t = 0 gives [1.., 0..], first frequency is 1);
 ``cfg_euler_step`` IS the reference's tensor expression sequence in bf16 / fp32 torch arithmetic.
-``sincos_pos_embed_2d`` (which axis comes first, the base_size scaling, the centre crop) and the order of
-the [cos | sin] halves are **parity unpinned**: only an import of diffusers could confirm them.
+``sincos_pos_embed_2d`` (which axis comes first, the base_size scaling, the centre crop), the order of the
+[cos | sin] halves of the timestep projection and ``flow_match_sigmas`` (diffusers' schedule, checked only
+against its closed form and the published SD3 28-step values 1.0, 0.9874, ...) are **parity unpinned**: only an
+import of diffusers could confirm them.  ``flux_conditioning`` / ``flux_transformer`` compose functions pinned
+elsewhere in the order of ``transformer_flux.py:101-207``.
 """
 import math
 from typing import Dict, Optional, Tuple
@@ -126,3 +129,52 @@ def sd3_transformer(p: P, latent: torch.Tensor, encoder: torch.Tensor, pooled: t
     out = norm_out_proj(p, hidden, temb)
     channels = p["proj_out.weight"].shape[0] // (patch * patch)
     return unpatchify(out, channels, H, W, patch)
+
+
+def flux_conditioning(p: P, prefix: str, timestep: torch.Tensor, pooled: torch.Tensor, guidance: Optional[torch.Tensor],
+                      freq_dim: int = 256) -> torch.Tensor:
+    """transformer_flux.py:104-112: the timestep (and guidance) is scaled by 1000 in the model's dtype (bf16)
+    before the sinusoidal projection; the embedders' outputs are summed."""
+    def embed(name, x):
+        return O.linear(O.silu(O.linear(x, p[f"{prefix}{name}.linear_1.weight"], p[f"{prefix}{name}.linear_1.bias"])),
+                        p[f"{prefix}{name}.linear_2.weight"], p[f"{prefix}{name}.linear_2.bias"])
+
+    t = (timestep.to(torch.bfloat16) * 1000).float()
+    out = embed("timestep_embedder", timestep_embedding(t, freq_dim))
+    if guidance is not None:
+        g = (guidance.to(torch.bfloat16) * 1000).float()
+        out = out + embed("guidance_embedder", timestep_embedding(g, freq_dim))
+    return out + embed("text_embedder", pooled.float())
+
+
+def flux_transformer(p: P, hidden: torch.Tensor, encoder: torch.Tensor, pooled: torch.Tensor, timestep: torch.Tensor,
+                     img_ids: torch.Tensor, txt_ids: torch.Tensor, guidance: Optional[torch.Tensor], heads: int, layers: int,
+                     single_layers: int, axes_dim=(16, 56, 56)) -> torch.Tensor:
+    """transformer_flux.py:101-207 on one stage: packed latent [B, N_img, C] -> [B, N_img, C]."""
+    from . import blocks as BL
+
+    def sub(prefix):
+        return {k[len(prefix):]: v for k, v in p.items() if k.startswith(prefix)}
+
+    x = O.linear(hidden.float(), p["x_embedder.weight"], p["x_embedder.bias"])
+    temb = flux_conditioning(p, "time_text_embed.", timestep, pooled, guidance)
+    enc = O.linear(encoder.float(), p["context_embedder.weight"], p["context_embedder.bias"])
+    rope = O.flux_rope_table(torch.cat([txt_ids, img_ids], 0), axes_dim)
+    for i in range(layers):
+        enc, x = BL.flux_double_block(sub(f"transformer_blocks.{i}."), x, enc, temb, rope, heads)
+    n_txt = enc.shape[1]
+    joint = torch.cat([enc, x], dim=1)
+    for i in range(single_layers):
+        joint = BL.flux_single_block(sub(f"single_transformer_blocks.{i}."), joint, temb, rope, heads, n_text=n_txt)
+    return norm_out_proj(p, joint[:, n_txt:], temb)
+
+
+def flow_match_sigmas(num_inference_steps: int, shift: float = 3.0, num_train_timesteps: int = 1000) -> torch.Tensor:
+    """diffusers ``FlowMatchEulerDiscreteScheduler.set_timesteps`` (static shift): t evenly spaced from sigma_max
+    to sigma_min of the shifted training schedule, shifted again, with a final 0.  fp32 [steps + 1]."""
+    def sh(s):
+        return shift * s / (1 + (shift - 1) * s)
+
+    s_max, s_min = sh(1.0), float(torch.tensor(sh(1.0 / num_train_timesteps), dtype=torch.float32))
+    t = torch.linspace(s_max, s_min, num_inference_steps, dtype=torch.float64)
+    return torch.cat([sh(t).float(), torch.zeros(1)])

@@ -32,7 +32,8 @@ def test_header_declares_the_expected_entry_points():
     for name in ("hdit_gemm_bf16", "hdit_attn_fwd_bf16", "hdit_attn_fwd_fp8", "hdit_attn_absmax",
                  "hdit_layernorm_modulate", "hdit_layernorm_modulate_jobs", "hdit_gate_residual", "hdit_adaln_gemv", "hdit_gelu_tanh",
                  "hdit_qk_norm_rope", "hdit_copy_rows", "hdit_patchify", "hdit_unpatchify", "hdit_timestep_embedding",
-                 "hdit_silu", "hdit_cfg_euler_step", "hdit_abi_version", "hdit_last_error"):
+                 "hdit_silu", "hdit_cfg_euler_step",
+    "hdit_rope_table", "hdit_abi_version", "hdit_last_error"):
         assert name in syms
 
 

@@ -147,3 +147,89 @@ def test_sd3_transformer_latent_to_noise(hdit):
     noise = S.sd3_transformer(params, torch.cat([lat1, lat1]).float(), enc.float(), pooled.float(), t, heads, L, 2, 24)
     want = S.cfg_euler_step(noise[:1], noise[1:], lat1, 7.0, 0.981, 0.95)
     assert_parity(new, want.float(), what="denoise step")
+
+
+def test_rope_table_kernel(hdit):
+    from hetu_dit_amd import synthetic
+    from oracle import ops as O
+
+    ids = synthetic.flux_ids(37, 12, 20)
+    cos, sin = hdit.ops.rope_table(ids.float().to(DEV), (16, 56, 56))
+    ocos, osin = O.flux_rope_table(ids, (16, 56, 56))
+    assert cos.shape == ocos.shape == (37 + 240, 128)
+    assert (cos.cpu() - ocos).abs().max() < 2e-6 and (sin.cpu() - osin).abs().max() < 2e-6
+    assert torch.equal(cos[:37].cpu(), torch.ones(37, 128)) and torch.equal(sin[:37].cpu(), torch.zeros(37, 128))
+    # CogVideoX: (frame, row, col) positions over axes (16, 24, 24)
+    pos = synthetic.cogvideox_positions(3, 6, 10)
+    cos, sin = hdit.ops.rope_table(pos.float().to(DEV), (16, 24, 24))
+    ocos, osin = O.cogvideox_rope_table(3, 6, 10, 64)
+    assert (cos.cpu() - ocos).abs().max() < 2e-6 and (sin.cpu() - osin).abs().max() < 2e-6
+    with pytest.raises(Exception):
+        hdit.ops.rope_table(pos.float().to(DEV), (16, 24, 23))
+
+
+def test_flux_transformer_packed_latent_to_noise(hdit):
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.transformer_flux import FluxTransformer2DModel
+
+    heads, L, Ls, gh, gw, Nt = 2, 2, 2, 12, 16, 64
+    model = FluxTransformer2DModel(num_layers=L, num_single_layers=Ls, attention_head_dim=128, num_attention_heads=heads,
+                                   joint_attention_dim=192, pooled_projection_dim=64)
+    synthetic.init_module_(model, 21)
+    params = step_params(model)
+    for i, blk in enumerate(model.single_transformer_blocks):
+        from tests.util import oracle_params
+
+        for k, v in oracle_params(blk).items():
+            params[f"single_transformer_blocks.{i}.{k}"] = v
+    model = model.to(DEV)
+    B = 1
+    lat = synthetic.randn_bf16((B, gh * gw, 64), 22)
+    enc = synthetic.randn_bf16((B, Nt, 192), 23)
+    pooled = synthetic.randn_bf16((B, 64), 24)
+    t, g = torch.tensor([0.7071]), torch.tensor([3.5])
+    ids = synthetic.flux_ids(Nt, gh, gw)
+    txt_ids, img_ids = ids[:Nt], ids[Nt:]
+    got = model(lat.to(DEV), enc.to(DEV), pooled.to(DEV), t.to(DEV), img_ids.to(DEV), txt_ids.to(DEV), g.to(DEV))
+    torch.cuda.synchronize()
+    want = S.flux_transformer(params, lat.float(), enc.float(), pooled.float(), t, img_ids, txt_ids, g, heads, L, Ls)
+    assert got.shape == lat.shape
+    assert_parity(got, want, what="flux transformer")
+    temb = model.conditioning(t.to(DEV), pooled.to(DEV), g.to(DEV))
+    assert_parity(temb, S.flux_conditioning(params, "time_text_embed.", t, pooled.float(), g), what="flux temb")
+    with pytest.raises(ValueError):
+        model.conditioning(t.to(DEV), pooled.to(DEV), None)
+
+
+def test_scheduler_steps_match_oracle_expressions(hdit):
+    from hetu_dit_amd.runtime_state import get_runtime_state
+    from hetu_dit_amd.schedulers import FlowMatchEulerDiscreteScheduler
+
+    torch.manual_seed(5)
+    sch = FlowMatchEulerDiscreteScheduler(shift=3.0)
+    sch.set_timesteps(6, device=DEV)
+    sig = S.flow_match_sigmas(6)
+    x = torch.randn(1, 16, 32, 32).bfloat16()
+    ref = x.clone()
+    cur = x.to(DEV)
+    for i, t in enumerate(sch.timesteps):
+        u, c = torch.randn_like(x), torch.randn_like(x)
+        if i % 2 == 0:  # guidance fused with the update
+            cur = sch.step_with_guidance(u.to(DEV), c.to(DEV), 5.0, t, cur)
+            ref = S.cfg_euler_step(u, c, ref, 5.0, float(sig[i]), float(sig[i + 1]))
+        else:           # the reference's two-call form: guidance by tensor expressions, then scheduler.step
+            noise = u + 5.0 * (c - u)
+            cur = sch.step(noise.to(DEV), t, cur, return_dict=False)[0]
+            ref = S.cfg_euler_step(noise, noise, ref, 0.0, float(sig[i]), float(sig[i + 1]))
+        assert sch.step_index == i + 1
+        assert torch.equal(cur.cpu(), ref), f"step {i}"
+    # patch mode: the index moves after the last patch only
+    rs = get_runtime_state()
+    sch.set_timesteps(4, device=DEV)
+    rs.set_patches(32, 32, 2, 2)
+    rs.set_patched_mode(True)
+    t0 = sch.timesteps[0]
+    for patch, expect in ((0, 0), (1, 1)):
+        sch.step(x[:, :, :16].contiguous().to(DEV), t0, x[:, :, :16].contiguous().to(DEV))
+        assert sch.step_index == expect
+        rs.next_patch()

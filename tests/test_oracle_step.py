@@ -115,3 +115,65 @@ def test_combined_embedding_and_norm_out_against_torch_modules():
     scale, shift = lin(F.silu(temb)).chunk(2, dim=1)
     want = proj(F.layer_norm(hidden, (D,), eps=1e-6) * (1 + scale[:, None]) + shift[:, None])
     assert torch.allclose(S.norm_out_proj(q, hidden, temb), want, atol=1e-5)
+
+
+def test_flow_match_sigmas_closed_form_and_scheduler_host_logic():
+    from hetu_dit_amd.runtime_state import get_runtime_state, reset_runtime_state
+    from hetu_dit_amd.schedulers import FlowMatchEulerDiscreteScheduler
+
+    sig = S.flow_match_sigmas(28)
+    assert sig.shape == (29,) and sig[0] == 1.0 and sig[-1] == 0.0
+    assert torch.all(sig[1:] < sig[:-1])
+    # published SD3 schedule (shift 3, 28 steps): second sigma 0.9874, last non-zero 3 s / (1 + 2 s) at s = sigma_min
+    assert abs(float(sig[1]) - 0.9874) < 1e-4
+    s_min = 3 * 0.001 / 1.002
+    assert abs(float(sig[-2]) - 3 * s_min / (1 + 2 * s_min)) < 1e-6
+    # un-shifting gives back evenly spaced points
+    un = sig[:-1].double() / (3 - 2 * sig[:-1].double())
+    assert torch.allclose(un[1:] - un[:-1], (un[-1] - un[0]) / 27 * torch.ones(27, dtype=torch.float64), atol=1e-6)
+
+    sch = FlowMatchEulerDiscreteScheduler(shift=3.0)
+    sch.set_timesteps(28)
+    assert torch.allclose(sch.sigmas, sig, atol=1e-7)
+    assert torch.allclose(sch.timesteps, sig[:-1] * 1000, atol=1e-4)
+    assert sch.step_index is None and sch.index_for_timestep(sch.timesteps[3]) == 3
+    with pytest.raises(ValueError):
+        sch._sigma_pair(3)
+    with pytest.raises(ValueError):
+        sch.index_for_timestep(123.456)
+    # the step index advances once per step: after every call outside patch mode, after the last patch inside
+    reset_runtime_state()
+    rs = get_runtime_state()
+    assert sch._sigma_pair(sch.timesteps[0]) == (float(sig[0]), float(sig[1]))
+    sch._advance()
+    assert sch.step_index == 1
+    rs.set_token_patches([0, 4, 8, 12])
+    rs.set_patched_mode(True)
+    for expect in (1, 1, 2):
+        sch._advance()
+        assert sch.step_index == expect
+        rs.next_patch()
+    reset_runtime_state()
+
+
+def test_flux_conditioning_against_torch_modules():
+    torch.manual_seed(4)
+    D, Pd = 32, 24
+    lins = {n: (torch.nn.Linear(256 if n != "text_embedder" else Pd, D), torch.nn.Linear(D, D))
+            for n in ("timestep_embedder", "guidance_embedder", "text_embedder")}
+    p = {}
+    for n, (l1, l2) in lins.items():
+        p[f"e.{n}.linear_1.weight"], p[f"e.{n}.linear_1.bias"] = l1.weight.detach(), l1.bias.detach()
+        p[f"e.{n}.linear_2.weight"], p[f"e.{n}.linear_2.bias"] = l2.weight.detach(), l2.bias.detach()
+    t, g, pooled = torch.tensor([0.7071, 0.25]), torch.tensor([3.5, 3.5]), torch.randn(2, Pd)
+
+    def emb(n, x):
+        return lins[n][1](F.silu(lins[n][0](x)))
+
+    tb = (t.bfloat16() * 1000).float()  # 0.7071 -> bf16 0.70703125 -> 707.03125 -> bf16 708
+    assert tb[0] == 708.0
+    want = emb("timestep_embedder", S.timestep_embedding(tb, 256)) + emb("guidance_embedder", S.timestep_embedding(
+        torch.tensor([3504.0, 3504.0]), 256)) + emb("text_embedder", pooled)  # 3500 rounds to 3504 in bf16
+    assert torch.allclose(S.flux_conditioning(p, "e.", t, pooled, g), want, atol=1e-5)
+    want = emb("timestep_embedder", S.timestep_embedding(tb, 256)) + emb("text_embedder", pooled)
+    assert torch.allclose(S.flux_conditioning(p, "e.", t, pooled, None), want, atol=1e-5)
