@@ -46,6 +46,12 @@ therefore pinned by what mathematics and PyTorch's own library routines fix
   sites fix (joint ordering, return order, split points, argument names) and
   the adaLN-"Zero" identity property (zero modulation weights => block is the
   identity on the residual stream).
+* head and tail of a step (``oracle/step.py``): patch embedding -- ``F.conv2d``;
+  unpatchify -- ``F.fold`` and index checks; timestep projection and the 2-D
+  sin-cos table -- closed forms; conditioning embedders and ``norm_out`` +
+  ``proj_out`` -- ``torch.nn`` modules; guidance + Euler update -- fp64
+  identities.  The layout conventions of diffusers' position table, timestep
+  projection and sigma schedule are **parity unpinned** (see that file's header).
 """
 
 from .ops import (  # noqa: F401
@@ -69,3 +75,4 @@ from .blocks import (  # noqa: F401
     feed_forward,
 )
 from .kv_cache import StaleKVBuffer  # noqa: F401
+from . import step  # noqa: F401
