@@ -76,6 +76,10 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   constexpr int DB = HD / 32;       // 32-wide d blocks of O^T
   constexpr int CPR = HD / 8;       // 16-byte chunks per row
   constexpr int NCH = BKV * CPR / 256;  // chunks per thread per tile (K and V each)
+  // FOLD: the softmax scale is multiplied into Q once and the running reference m is subtracted inside the
+  // score MFMA (its first k-step accumulates onto -m), so the accumulators feed exp2 directly: one FMA less
+  // per score in a loop that is bound by the VALU.  Costs 32 registers; the d = 128 kernel has none to spare.
+  constexpr bool FOLD = HD == 64;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
@@ -91,7 +95,18 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     int r = min(q0 + qb * 32 + l32, P.sq - 1);
     const __bf16* rp = row_ptr(P.q, b, h, r);
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[qb][ks] = *(const bf16x8*)(rp + ks * 16 + lh * 8);
+    for (int ks = 0; ks < KS; ks++) {
+      const i32x4 raw = *(const i32x4*)(rp + ks * 16 + lh * 8);
+      if constexpr (FOLD) {
+        float f[8];
+        hdit::unpack8(raw, f);
+#pragma unroll
+        for (int e = 0; e < 8; e++) f[e] *= P.scale_log2;
+        qf[qb][ks] = __builtin_bit_cast(bf16x8, hdit::pack8(f));
+      } else {
+        qf[qb][ks] = __builtin_bit_cast(bf16x8, raw);
+      }
+    }
   }
 
   // ---- K/V tile staging: global -> registers -> LDS.  A tile that lies inside one segment is addressed as
@@ -157,8 +172,17 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) oacc[i][j][v] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY};
+  // running reference m of the online softmax (log2 units) and running sum per query column.  With FOLD the
+  // accumulators of a score block start from negm = -m (the same value in all 16 entries: a lane owns one
+  // query column per qb) and m starts at 0 until the first tile sets it to that tile's column maxima.
+  float m_run[2] = {FOLD ? 0.f : -INFINITY, FOLD ? 0.f : -INFINITY};
   float l_run[2] = {0.f, 0.f};
+  f32x16 negm[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) negm[qb][v] = 0.f;
+  bool first = true;
 
   // lane-constant part of the V^T transpose-read address:
   // 16-lane group G = lane/16, x = lane%16: key row 4*(G/2) + x/4, column 16*(G%2) + 4*(x%4)
@@ -180,7 +204,7 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
         bf16x8 kf = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + ks * 32);
 #pragma unroll
         for (int qb = 0; qb < 2; qb++)
-          sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], ks == 0 ? zero16 : sacc[kb][qb], 0, 0, 0);
+          sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], ks == 0 ? (FOLD ? negm[qb] : zero16) : sacc[kb][qb], 0, 0, 0);
       }
     }
     if (MASK) {
@@ -199,28 +223,64 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     // ---- online softmax in the log2 domain.  A lane owns one query column per qb and 32 of its 64 keys;
     // the other 32 live in lane^32.
     bf16x8 pf[2][4];  // [qb][u], u = 2*kb + half: the 16 keys of PV k-step u
-    float mcand[2];
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-      float mx = fmaxf(sacc[0][qb][0], sacc[1][qb][0]);
-#pragma unroll
-      for (int v = 1; v < 16; v++) mx = fmaxf(mx, fmaxf(sacc[0][qb][v], sacc[1][qb][v]));
-      auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(mx), __float_as_int(mx), false, false);
-      mx = fmaxf(__int_as_float(sw[0]), __int_as_float(sw[1]));
-      mcand[qb] = fmaxf(m_run[qb], mx * P.scale_log2);
-    }
-    // raise the running maxima (and rescale) only if some row outgrew the threshold: wave-uniform branch
-    const bool grow = (mcand[0] - m_run[0] > RESCALE_THRESHOLD) || (mcand[1] - m_run[1] > RESCALE_THRESHOLD);
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+    if constexpr (FOLD) {
+      float mrel[2];  // column maxima relative to the running reference
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
-        const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - mcand[qb]);
-        m_run[qb] = mcand[qb];
-        l_run[qb] *= alpha;
+        float mx = fmaxf(sacc[0][qb][0], sacc[1][qb][0]);
 #pragma unroll
-        for (int db = 0; db < DB; db++)
+        for (int v = 1; v < 16; v++) mx = fmaxf(fmaxf(mx, sacc[0][qb][v]), sacc[1][qb][v]);  // one v_max3 per step
+        auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(mx), __float_as_int(mx), false, false);
+        mrel[qb] = fmaxf(__int_as_float(sw[0]), __int_as_float(sw[1]));
+      }
+      // move the reference (and rescale) only if some column outgrew the threshold: wave-uniform branch
+      const bool grow = first || mrel[0] > RESCALE_THRESHOLD || mrel[1] > RESCALE_THRESHOLD;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
-          for (int v = 0; v < 16; v++) oacc[db][qb][v] *= alpha;
+        for (int qb = 0; qb < 2; qb++) {
+          const float d = first ? mrel[qb] : fmaxf(mrel[qb], 0.f);
+          m_run[qb] += d;
+          if (!first) {
+            const float alpha = __builtin_amdgcn_exp2f(-d);
+            l_run[qb] *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+              for (int v = 0; v < 16; v++) oacc[db][qb][v] *= alpha;
+          }
+#pragma unroll
+          for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) sacc[kb][qb][v] -= d;
+#pragma unroll
+          for (int v = 0; v < 16; v++) negm[qb][v] = -m_run[qb];
+        }
+        first = false;
+      }
+    } else {
+      float mcand[2];
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        float mx = fmaxf(sacc[0][qb][0], sacc[1][qb][0]);
+#pragma unroll
+        for (int v = 1; v < 16; v++) mx = fmaxf(fmaxf(mx, sacc[0][qb][v]), sacc[1][qb][v]);  // one v_max3 per step
+        auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(mx), __float_as_int(mx), false, false);
+        mx = fmaxf(__int_as_float(sw[0]), __int_as_float(sw[1]));
+        mcand[qb] = fmaxf(m_run[qb], mx * P.scale_log2);
+      }
+      // raise the running maxima (and rescale) only if some row outgrew the threshold: wave-uniform branch
+      const bool grow = (mcand[0] - m_run[0] > RESCALE_THRESHOLD) || (mcand[1] - m_run[1] > RESCALE_THRESHOLD);
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+          const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - mcand[qb]);
+          m_run[qb] = mcand[qb];
+          l_run[qb] *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) oacc[db][qb][v] *= alpha;
+        }
       }
     }
 #pragma unroll
@@ -234,8 +294,9 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
           i32x4 pk;
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][qb][hh * 8 + 2 * e], P.scale_log2, -m));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][qb][hh * 8 + 2 * e + 1], P.scale_log2, -m));
+            const float s0 = sacc[kb][qb][hh * 8 + 2 * e], s1 = sacc[kb][qb][hh * 8 + 2 * e + 1];
+            const float p0 = __builtin_amdgcn_exp2f(FOLD ? s0 : __builtin_fmaf(s0, P.scale_log2, -m));
+            const float p1 = __builtin_amdgcn_exp2f(FOLD ? s1 : __builtin_fmaf(s1, P.scale_log2, -m));
             const uint32_t pp = hdit::pack2(p0, p1);
             pk[e] = (int)pp;
             // row sum of exactly the bf16 values that enter the PV product
