@@ -16,6 +16,13 @@ _lib_def.define("gate_residual(Tensor x, Tensor y, Tensor gate) -> Tensor")
 _lib_def.define("adaln_gemv(Tensor temb, Tensor weight, Tensor? bias=None) -> Tensor")
 _lib_def.define("gelu_tanh(Tensor x, Tensor? bias=None) -> Tensor")
 _lib_def.define("attention(Tensor[] q, Tensor[] k, Tensor[] v, float scale=0.0, bool fp8=False) -> Tensor[]")
+_lib_def.define("patchify(Tensor latent, int patch) -> Tensor")
+_lib_def.define("unpatchify(Tensor x, int channels, int height, int width, int patch) -> Tensor")
+_lib_def.define("timestep_embedding(Tensor timesteps, int dim, float max_period=10000.0) -> Tensor")
+_lib_def.define("silu(Tensor x) -> Tensor")
+_lib_def.define("rope_table(Tensor positions, int[] axes_dim, float theta=10000.0) -> (Tensor, Tensor)")
+_lib_def.define("cfg_euler_step(Tensor noise_uncond, Tensor noise_cond, Tensor sample, float guidance, float sigma, "
+                "float sigma_next) -> Tensor")
 
 
 def _linear(x, weight, bias=None, gelu=False):
@@ -37,6 +44,13 @@ _impl.impl("gate_residual", lambda x, y, gate: ops.gate_residual(x, y, gate))
 _impl.impl("adaln_gemv", lambda temb, weight, bias=None: ops.adaln_gemv(temb, weight, bias))
 _impl.impl("gelu_tanh", lambda x, bias=None: ops.gelu_tanh(x, bias))
 _impl.impl("attention", _attention)
+_impl.impl("patchify", lambda latent, patch: ops.patchify(latent, patch))
+_impl.impl("unpatchify", lambda x, channels, height, width, patch: ops.unpatchify(x, channels, height, width, patch))
+_impl.impl("timestep_embedding", lambda t, dim, max_period=10000.0: ops.timestep_embedding(t, dim, max_period))
+_impl.impl("silu", lambda x: ops.silu(x))
+_impl.impl("rope_table", lambda positions, axes_dim, theta=10000.0: ops.rope_table(positions, list(axes_dim), theta))
+_impl.impl("cfg_euler_step", lambda u, c, x, guidance, sigma, sigma_next: ops.cfg_euler_step(u, c, x, guidance, sigma,
+                                                                                          sigma_next))
 
 
 @torch.library.register_fake("hdit::linear")
@@ -67,3 +81,35 @@ def _(x, bias=None):
 @torch.library.register_fake("hdit::attention")
 def _(q, k, v, scale=0.0, fp8=False):
     return [t.new_empty(t.shape) for t in q]
+
+
+@torch.library.register_fake("hdit::patchify")
+def _(latent, patch):
+    B, C, H, W = latent.shape
+    return latent.new_empty(B, (H // patch) * (W // patch), C * patch * patch)
+
+
+@torch.library.register_fake("hdit::unpatchify")
+def _(x, channels, height, width, patch):
+    return x.new_empty(x.shape[0], channels, height, width)
+
+
+@torch.library.register_fake("hdit::timestep_embedding")
+def _(timesteps, dim, max_period=10000.0):
+    return timesteps.new_empty(timesteps.shape[0], dim, dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("hdit::silu")
+def _(x):
+    return x.new_empty(x.shape)
+
+
+@torch.library.register_fake("hdit::rope_table")
+def _(positions, axes_dim, theta=10000.0):
+    width = sum(axes_dim)
+    return positions.new_empty(positions.shape[0], width), positions.new_empty(positions.shape[0], width)
+
+
+@torch.library.register_fake("hdit::cfg_euler_step")
+def _(noise_uncond, noise_cond, sample, guidance, sigma, sigma_next):
+    return sample.new_empty(sample.shape)

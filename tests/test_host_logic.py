@@ -173,3 +173,14 @@ def test_torch_library_ops_have_fake_kernels():
         q = torch.empty(2, 7, 1, 64, dtype=torch.bfloat16, device="cuda")
         (o,) = torch.ops.hdit.attention([q], [q], [q])
         assert o.shape == q.shape
+        lat = torch.empty(2, 16, 8, 12, dtype=torch.bfloat16, device="cuda")
+        tok = torch.ops.hdit.patchify(lat, 2)
+        assert tok.shape == (2, 24, 64)
+        assert torch.ops.hdit.unpatchify(tok, 16, 8, 12, 2).shape == lat.shape
+        ts = torch.empty(3, dtype=torch.float32, device="cuda")
+        emb = torch.ops.hdit.timestep_embedding(ts, 256)
+        assert emb.shape == (3, 256) and emb.dtype == torch.bfloat16
+        assert torch.ops.hdit.silu(emb).shape == emb.shape
+        cos, sin = torch.ops.hdit.rope_table(torch.empty(9, 3, dtype=torch.float32, device="cuda"), [16, 56, 56])
+        assert cos.shape == sin.shape == (9, 128) and cos.dtype == torch.float32
+        assert torch.ops.hdit.cfg_euler_step(lat, lat, lat, 7.0, 1.0, 0.9).shape == lat.shape
