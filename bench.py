@@ -195,7 +195,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only: run with --gpus 1 "
-              "(every box of this build has one GPU; how the path shards is described in DESIGN.md)", file=sys.stderr)
+              "(the path is built and measured on a single GPU; nothing here launches collectives)", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -243,11 +243,18 @@ def main():
         run = step
 
     torch.cuda.synchronize()
+    clk0 = ops.clock_sample()  # enqueued in front of the timed passes, on their stream
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         run()
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    clk1 = ops.clock_sample()
+    torch.cuda.synchronize()
+    d_clk = (clk1 - clk0).tolist()
+    # average shader clock over the timed passes: shader-clock ticks per tick of the constant 100 MHz counter
+    shader_clock_ghz = d_clk[0] / d_clk[1] * 0.1 if d_clk[1] > 0 else None
 
     # one plain device copy of known size (256 MiB read + 256 MiB written): the scale reference for the
     # FETCH_SIZE / WRITE_SIZE hardware counters when this command runs under `rocprofv3 --pmc`
@@ -304,6 +311,9 @@ def main():
         "data": "synthetic (seeded N(0,1) activations, N(0,0.02) random-init weights, resident in HBM)",
         "config": {"workload": workload_desc, "launch": "hip-graph replay" if use_graph else "eager"},
         "step_tflops": round((gemm_fl + attn_fl) / ms_step / 1e9, 1),
+        "shader_clock_ghz": round(shader_clock_ghz, 3) if shader_clock_ghz else None,
+        "shader_clock_note": "average over the timed passes, from the shader-clock and 100 MHz counters sampled on the "
+                             "launch stream before and after them; the published peaks are quoted at 2.4 GHz",
         "roofline": {
             "kernel": "gemm_kernel (grouped bf16 MFMA GEMM, all projection/MLP launches of the step)",
             "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",

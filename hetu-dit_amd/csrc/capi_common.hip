@@ -25,3 +25,19 @@ int check_launch(const char* what) {
 
 extern "C" __attribute__((visibility("default"))) int hdit_abi_version(void) { return 1; }
 extern "C" __attribute__((visibility("default"))) const char* hdit_last_error(void) { return g_err; }
+
+namespace {
+// one lane stores the shader-clock counter and the constant 100 MHz counter
+__global__ void clock_sample_kernel(unsigned long long* out) {
+  if (threadIdx.x == 0) {
+    out[0] = __builtin_amdgcn_s_memtime();
+    out[1] = __builtin_amdgcn_s_memrealtime();
+  }
+}
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int hdit_clock_sample(void* out, void* stream) {
+  if (!out || (((uintptr_t)out) & 7)) return HDIT_EINVAL;
+  hipLaunchKernelGGL(clock_sample_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)out);
+  return hdit_host::check_launch("hdit_clock_sample");
+}

@@ -451,3 +451,10 @@ def rope_table(positions: torch.Tensor, axes_dim, theta: float = 10000.0) -> Tup
     check(_lib.lib().hdit_rope_table(positions.data_ptr(), rows, arr, len(axes), float(theta), cos.data_ptr(), sin.data_ptr(),
                                      _stream()), "hdit_rope_table")
     return cos, sin
+
+
+def clock_sample() -> torch.Tensor:
+    """int64 [2] on the device, filled on the current stream with (shader-clock counter, 100 MHz counter)."""
+    out = torch.zeros(2, dtype=torch.int64, device="cuda")
+    check(_lib.lib().hdit_clock_sample(out.data_ptr(), _stream()), "hdit_clock_sample")
+    return out

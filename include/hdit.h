@@ -30,6 +30,12 @@ extern "C" {
 int hdit_abi_version(void);
 /* Static string describing the last HDIT_ELAUNCH on this thread ("" if none). */
 const char* hdit_last_error(void);
+/* Measurement aid without a counterpart in the reference: enqueues a one-wave
+ * kernel that stores two 64-bit counters to out[0..1] (device memory, 8-byte
+ * aligned): the shader-clock counter and the constant 100 MHz counter.  Two
+ * samples on one stream, around the work being timed, give the average shader
+ * clock the work ran at: (d out[0]) / (d out[1]) x 100 MHz. */
+int hdit_clock_sample(void* out, void* stream);
 
 /* ------------------------------------------------------------------------
  * Grouped bf16 GEMM with fused epilogue:  C = epilogue(A . B^T + bias)

@@ -33,7 +33,7 @@ def test_header_declares_the_expected_entry_points():
                  "hdit_layernorm_modulate", "hdit_layernorm_modulate_jobs", "hdit_gate_residual", "hdit_adaln_gemv", "hdit_gelu_tanh",
                  "hdit_qk_norm_rope", "hdit_copy_rows", "hdit_patchify", "hdit_unpatchify", "hdit_timestep_embedding",
                  "hdit_silu", "hdit_cfg_euler_step",
-    "hdit_rope_table", "hdit_abi_version", "hdit_last_error"):
+    "hdit_rope_table", "hdit_clock_sample", "hdit_abi_version", "hdit_last_error"):
         assert name in syms
 
 

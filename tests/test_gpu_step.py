@@ -233,3 +233,16 @@ def test_scheduler_steps_match_oracle_expressions(hdit):
         sch.step(x[:, :, :16].contiguous().to(DEV), t0, x[:, :, :16].contiguous().to(DEV))
         assert sch.step_index == expect
         rs.next_patch()
+
+
+def test_clock_sample_counts_forward(hdit):
+    a = hdit.ops.clock_sample()
+    x = torch.randn(4096, 4096, device=DEV)
+    for _ in range(5):
+        x = x @ x * 1e-3
+    b = hdit.ops.clock_sample()
+    torch.cuda.synchronize()
+    d = (b - a).tolist()
+    assert d[0] > 0 and d[1] > 0
+    ghz = d[0] / d[1] * 0.1
+    assert 0.05 < ghz < 3.5, ghz  # a plausible shader clock
