@@ -121,10 +121,13 @@ def gemm_problem(
 
 
 def gemm_launch(problems: Sequence[GemmProblem]):
-    n = len(problems)
-    arr = (GemmProblem * n)(*problems)
-    flops = sum(2.0 * p.m * p.n * p.k for p in problems) if _TIMER is not None else 0.0
-    check(_run("gemm", flops, lambda: _lib.lib().hdit_gemm_bf16(arr, n, _stream())), "hdit_gemm_bf16")
+    """One call of the grouped GEMM per HDIT_GEMM_MAX_PROBLEMS problems (a call plans its problems together)."""
+    for first in range(0, len(problems), _lib.HDIT_GEMM_MAX_PROBLEMS):
+        chunk = problems[first : first + _lib.HDIT_GEMM_MAX_PROBLEMS]
+        n = len(chunk)
+        arr = (GemmProblem * n)(*chunk)
+        flops = sum(2.0 * p.m * p.n * p.k for p in chunk) if _TIMER is not None else 0.0
+        check(_run("gemm", flops, lambda: _lib.lib().hdit_gemm_bf16(arr, n, _stream())), "hdit_gemm_bf16")
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, gelu: bool = False,

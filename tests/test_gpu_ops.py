@@ -315,3 +315,15 @@ def test_empty_and_ragged_inputs(hdit):
     # queries without any key are refused
     with pytest.raises(hdit._lib.HditError):
         ops.attention([g(q)], [e], [e])
+
+
+def test_gemm_more_problems_than_one_call_takes(hdit):
+    """20 problems (the C entry point takes 16 per call): the wrapper splits them over calls."""
+    ops = hdit.ops
+    ws = [rnd(64, 128, scale=0.05, seed=100 + i) for i in range(20)]
+    xs = [rnd(33 + i, 128, seed=200 + i) for i in range(20)]
+    outs = [torch.empty(33 + i, 64, dtype=torch.bfloat16, device=DEV) for i in range(20)]
+    ops.gemm_launch([ops.gemm_problem(g(x), g(w), o) for x, w, o in zip(xs, ws, outs)])
+    torch.cuda.synchronize()
+    for x, w, o in zip(xs, ws, outs):
+        assert_parity(o, O.linear(x, w), what="one of 20 problems")
