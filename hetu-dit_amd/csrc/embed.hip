@@ -25,7 +25,9 @@ __global__ void __launch_bounds__(256) patchify_kernel(const __bf16* __restrict_
   out[i] = latent[((b * C + c) * H + hy * p + py) * W + wx * p + px];
 }
 
-// out[b, c, hy*p + py, wx*p + px] = x[b, hy*w + wx, (py*p + px)*C + c]
+// out[b, c, hy*p + py, wx*p + px] = x[b, hy*w + wx, (py*p + px)*C + c]   (channel innermost), or
+//                                 = x[b, hy*w + wx, (c*p + py)*p + px]   (CHANNEL_MAJOR)
+template <bool CHANNEL_MAJOR>
 __global__ void __launch_bounds__(256) unpatchify_kernel(const __bf16* __restrict__ x, __bf16* __restrict__ out,
                                                          int64_t total, int C, int H, int W, int p) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -34,7 +36,8 @@ __global__ void __launch_bounds__(256) unpatchify_kernel(const __bf16* __restric
   const int X = (int)(i % W), Y = (int)((i / W) % H), c = (int)((i / ((int64_t)W * H)) % C);
   const int64_t b = i / ((int64_t)W * H * C);
   const int wx = X / p, px = X % p, hy = Y / p, py = Y % p;
-  out[i] = x[((b * h + hy) * w + wx) * (int64_t)(p * p * C) + (py * p + px) * C + c];
+  const int col = CHANNEL_MAJOR ? (c * p + py) * p + px : (py * p + px) * C + c;
+  out[i] = x[((b * h + hy) * w + wx) * (int64_t)(p * p * C) + col];
 }
 
 // out[b, :half] = cos(t[b] * f_i), out[b, half:] = sin(t[b] * f_i), f_i = exp(-ln(max_period) * i / half)
@@ -123,14 +126,18 @@ extern "C" __attribute__((visibility("default"))) int hdit_patchify(const void* 
 }
 
 extern "C" __attribute__((visibility("default"))) int hdit_unpatchify(const void* x, void* out, int batch, int channels, int height, int width,
-                                               int patch, void* stream) {
+                                               int patch, int channel_major, void* stream) {
   if (batch < 0 || channels <= 0 || height <= 0 || width <= 0 || patch <= 0) return HDIT_EINVAL;
   if (height % patch || width % patch) return HDIT_EINVAL;
   const int64_t total = (int64_t)batch * channels * height * width;
   if (total == 0) return HDIT_OK;
   if (!x || !out) return HDIT_EINVAL;
-  hipLaunchKernelGGL(unpatchify_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const __bf16*)x, (__bf16*)out, total, channels, height, width, patch);
+  if (channel_major)
+    hipLaunchKernelGGL(unpatchify_kernel<true>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const __bf16*)x, (__bf16*)out, total, channels, height, width, patch);
+  else
+    hipLaunchKernelGGL(unpatchify_kernel<false>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const __bf16*)x, (__bf16*)out, total, channels, height, width, patch);
   return hdit_host::check_launch("hdit_unpatchify");
 }
 

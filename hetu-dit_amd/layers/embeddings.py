@@ -116,3 +116,39 @@ def norm_out_project(norm_out, proj_out, hidden_states: torch.Tensor, temb: torc
     x = ops.layernorm_modulate(hidden_states, shift, scale, norm_out.norm.eps)
     B, T, D = x.shape
     return project(x.view(-1, D), proj_out).view(B, T, -1)
+
+
+from .modules import CogVideoXPatchEmbed  # noqa: E402
+
+
+@hetuDiTLayerWrappersRegister.register(CogVideoXPatchEmbed)
+class hetuDiTCogVideoXPatchEmbedWrapper(hetuDiTDiffusionLayerBaseWrapper):
+    """``layers/embeddings.py:115-232`` of the reference for the rotary-embedding models (CogVideoX-5B): text
+    projection and per-frame patch convolution written side by side into one joint [text, video] sequence --
+    all projections of all batch elements in one grouped-GEMM launch, no ``cat``."""
+
+    def __init__(self, patch_embedding: CogVideoXPatchEmbed):
+        super().__init__(module=patch_embedding)
+
+    @torch.no_grad()
+    def forward(self, text_embeds: torch.Tensor, image_embeds: torch.Tensor) -> torch.Tensor:
+        m = self.module
+        if m.patch_size_t is not None or m.use_positional_embeddings or m.use_learned_positional_embeddings:
+            raise NotImplementedError("only the CogVideoX-5B patch embedding (2-D patches, rotary positions) is built")
+        B, F, C, H, W = image_embeds.shape
+        p = m.patch_size
+        D = m.proj.weight.shape[0]
+        n_txt = text_embeds.shape[1]
+        x = ops.patchify(image_embeds.contiguous().view(B * F, C, H, W), p)  # [B F, h w, C p p]
+        n_img = F * x.shape[1]
+        x = x.view(B, n_img, C * p * p)
+        w2 = m.proj.weight.data.reshape(D, C * p * p)
+        bias = m.proj.bias.data if m.proj.bias is not None else None
+        text = text_embeds.contiguous()
+        out = torch.empty(B, n_txt + n_img, D, dtype=torch.bfloat16, device=image_embeds.device)
+        problems = []
+        for b in range(B):
+            problems.append(ops.gemm_problem(text[b], m.text_proj.weight.data, out[b, :n_txt], m.text_proj.bias.data))
+            problems.append(ops.gemm_problem(x[b], w2, out[b, n_txt:], bias))
+        ops.gemm_launch(problems)
+        return out

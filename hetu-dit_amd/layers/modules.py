@@ -238,3 +238,29 @@ class FluxPosEmbed(nn.Module):
     def __init__(self, theta: float = 10000.0, axes_dim=(16, 56, 56)):
         super().__init__()
         self.theta, self.axes_dim = theta, tuple(axes_dim)
+
+
+class CogVideoXPatchEmbed(nn.Module):
+    """diffusers ``CogVideoXPatchEmbed`` as CogVideoX-5B configures it: a p x p stride-p convolution per frame,
+    a text projection, no learned or sin-cos position table (the model uses rotary embeddings)."""
+
+    def __init__(self, patch_size: int = 2, in_channels: int = 16, embed_dim: int = 3072, text_embed_dim: int = 4096,
+                 bias: bool = True):
+        super().__init__()
+        self.patch_size, self.patch_size_t = patch_size, None
+        self.use_positional_embeddings = False
+        self.use_learned_positional_embeddings = False
+        self.proj = nn.Conv2d(in_channels, embed_dim, kernel_size=patch_size, stride=patch_size, bias=bias)
+        self.text_proj = nn.Linear(text_embed_dim, embed_dim)
+
+
+class AdaLayerNorm(nn.Module):
+    """temb -> (shift, scale) -- shift first (``chunk_dim=1``); the LayerNorm carries affine weights."""
+
+    chunks = 2
+
+    def __init__(self, embedding_dim: int, output_dim: int, eps: float = 1e-5):
+        super().__init__()
+        self.silu = nn.SiLU()
+        self.linear = nn.Linear(embedding_dim, output_dim)
+        self.norm = nn.LayerNorm(output_dim // 2, eps=eps, elementwise_affine=True)

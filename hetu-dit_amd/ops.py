@@ -398,15 +398,17 @@ def patchify(latent: torch.Tensor, patch: int) -> torch.Tensor:
     return out
 
 
-def unpatchify(x: torch.Tensor, channels: int, height: int, width: int, patch: int) -> torch.Tensor:
-    """bf16 [B, (H/p)(W/p), p p C] -> [B, C, H, W]."""
+def unpatchify(x: torch.Tensor, channels: int, height: int, width: int, patch: int,
+               channel_major: bool = False) -> torch.Tensor:
+    """bf16 [B, (H/p)(W/p), p p C] -> [B, C, H, W]; token columns ordered (py, px, c), or (c, py, px) if
+    ``channel_major``."""
     _need(x, bf16, "x")
     B = x.shape[0]
     if not x.is_contiguous() or tuple(x.shape) != (B, (height // patch) * (width // patch), patch * patch * channels):
         raise ValueError("unpatchify input shape does not match the latent geometry")
     out = torch.empty(B, channels, height, width, dtype=bf16, device=x.device)
-    check(_lib.lib().hdit_unpatchify(x.data_ptr(), out.data_ptr(), B, channels, height, width, patch, _stream()),
-          "hdit_unpatchify")
+    check(_lib.lib().hdit_unpatchify(x.data_ptr(), out.data_ptr(), B, channels, height, width, patch, int(channel_major),
+                                     _stream()), "hdit_unpatchify")
     return out
 
 

@@ -17,7 +17,7 @@ _lib_def.define("adaln_gemv(Tensor temb, Tensor weight, Tensor? bias=None) -> Te
 _lib_def.define("gelu_tanh(Tensor x, Tensor? bias=None) -> Tensor")
 _lib_def.define("attention(Tensor[] q, Tensor[] k, Tensor[] v, float scale=0.0, bool fp8=False) -> Tensor[]")
 _lib_def.define("patchify(Tensor latent, int patch) -> Tensor")
-_lib_def.define("unpatchify(Tensor x, int channels, int height, int width, int patch) -> Tensor")
+_lib_def.define("unpatchify(Tensor x, int channels, int height, int width, int patch, bool channel_major=False) -> Tensor")
 _lib_def.define("timestep_embedding(Tensor timesteps, int dim, float max_period=10000.0) -> Tensor")
 _lib_def.define("silu(Tensor x) -> Tensor")
 _lib_def.define("rope_table(Tensor positions, int[] axes_dim, float theta=10000.0) -> (Tensor, Tensor)")
@@ -45,7 +45,8 @@ _impl.impl("adaln_gemv", lambda temb, weight, bias=None: ops.adaln_gemv(temb, we
 _impl.impl("gelu_tanh", lambda x, bias=None: ops.gelu_tanh(x, bias))
 _impl.impl("attention", _attention)
 _impl.impl("patchify", lambda latent, patch: ops.patchify(latent, patch))
-_impl.impl("unpatchify", lambda x, channels, height, width, patch: ops.unpatchify(x, channels, height, width, patch))
+_impl.impl("unpatchify", lambda x, channels, height, width, patch, channel_major=False: ops.unpatchify(
+    x, channels, height, width, patch, channel_major))
 _impl.impl("timestep_embedding", lambda t, dim, max_period=10000.0: ops.timestep_embedding(t, dim, max_period))
 _impl.impl("silu", lambda x: ops.silu(x))
 _impl.impl("rope_table", lambda positions, axes_dim, theta=10000.0: ops.rope_table(positions, list(axes_dim), theta))
@@ -90,7 +91,7 @@ def _(latent, patch):
 
 
 @torch.library.register_fake("hdit::unpatchify")
-def _(x, channels, height, width, patch):
+def _(x, channels, height, width, patch, channel_major=False):
     return x.new_empty(x.shape[0], channels, height, width)
 
 

@@ -222,11 +222,14 @@ int hdit_rope_table(const float* positions, int rows, const int* axes_dim, int n
 int hdit_patchify(const void* latent, void* out, int batch, int channels, int height, int width, int patch,
                   void* stream);
 
-/* out[b, c, hy*p + py, wx*p + px] = x[b, hy*(W/p) + wx, (py*p + px)*C + c] (bf16):
- * the reshape + einsum("nhwpqc->nchpwq") + reshape of
- * models/transformers/transformer_sd3.py:160-182. */
+/* out[b, c, hy*p + py, wx*p + px] = x[b, hy*(W/p) + wx, col] (bf16) with
+ * col = (py*p + px)*C + c: the reshape + einsum("nhwpqc->nchpwq") + reshape of
+ * models/transformers/transformer_sd3.py:160-182; or, channel_major != 0,
+ * col = (c*p + py)*p + px: the reshape + permute(0, 1, 4, 2, 5, 3, 6) of
+ * models/transformers/cogvideox_transformer_3d.py:143-146 with the frames of a
+ * video counted into `batch`. */
 int hdit_unpatchify(const void* x, void* out, int batch, int channels, int height, int width, int patch,
-                    void* stream);
+                    int channel_major, void* stream);
 
 /* out[b, :dim/2] = cos(t[b] f_i), out[b, dim/2:] = sin(t[b] f_i), f_i =
  * max_period^(-i / (dim/2)); t f32 [batch], out bf16 [batch, dim].  diffusers

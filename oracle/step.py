@@ -17,7 +17,9 @@ expression; ``timestep_embedding`` against the closed form (t = 0 gives [1.., 0.
 [cos | sin] halves of the timestep projection and ``flow_match_sigmas`` (diffusers' schedule, checked only
 against its closed form and the published SD3 28-step values 1.0, 0.9874, ...) are **parity unpinned**: only an
 import of diffusers could confirm them.  ``flux_conditioning`` / ``flux_transformer`` compose functions pinned
-elsewhere in the order of ``transformer_flux.py:101-207``.
+elsewhere in the order of ``transformer_flux.py:101-207``.  ``cogvideox_patch_embed`` is pinned by ``F.conv2d`` and the
+wrapper's own flatten/transpose/cat expressions, ``ada_layer_norm`` by ``torch.nn`` modules (its shift-first chunk order
+is diffusers' and unpinned), ``unpatchify_channel_major`` by ``F.fold``.
 """
 import math
 from typing import Dict, Optional, Tuple
@@ -178,3 +180,53 @@ def flow_match_sigmas(num_inference_steps: int, shift: float = 3.0, num_train_ti
     s_max, s_min = sh(1.0), float(torch.tensor(sh(1.0 / num_train_timesteps), dtype=torch.float32))
     t = torch.linspace(s_max, s_min, num_inference_steps, dtype=torch.float64)
     return torch.cat([sh(t).float(), torch.zeros(1)])
+
+
+def cogvideox_patch_embed(p: P, prefix: str, text: torch.Tensor, video: torch.Tensor) -> torch.Tensor:
+    """layers/embeddings.py:126-165 (2-D patches, no position table): text [B, N_t, E], video [B, F, C, H, W] ->
+    [B, N_t + F (H/p)(W/p), D], text rows first."""
+    B, F, C, H, W = video.shape
+    w, b = p[prefix + "proj.weight"], p[prefix + "proj.bias"]
+    img = patch_embed(video.reshape(B * F, C, H, W), w, b, None)          # [B F, h w, D]
+    img = img.reshape(B, F * img.shape[1], -1)
+    txt = O.linear(text.float(), p[prefix + "text_proj.weight"], p[prefix + "text_proj.bias"])
+    return torch.cat([txt, img], dim=1)
+
+
+def ada_layer_norm(p: P, prefix: str, x: torch.Tensor, temb: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
+    """diffusers ``AdaLayerNorm`` with ``chunk_dim=1``: (shift, scale) = linear(silu(temb)).chunk(2); affine
+    LayerNorm, then * (1 + scale) + shift."""
+    shift, scale = O.adaln_modulation(temb, p[prefix + "linear.weight"], p[prefix + "linear.bias"], 2)
+    n = O.layer_norm(x, eps, p[prefix + "norm.weight"], p[prefix + "norm.bias"])
+    return O.modulate(n, shift, scale)
+
+
+def unpatchify_channel_major(x: torch.Tensor, frames: int, channels: int, height: int, width: int, patch: int) -> torch.Tensor:
+    """cogvideox_transformer_3d.py:143-146: [B, F h w, C p p] -> [B, F, C, H, W]."""
+    B = x.shape[0]
+    out = x.reshape(B, frames, height // patch, width // patch, channels, patch, patch)
+    return out.permute(0, 1, 4, 2, 5, 3, 6).flatten(5, 6).flatten(3, 4)
+
+
+def cogvideox_transformer(p: P, video: torch.Tensor, text: torch.Tensor, timestep: torch.Tensor, rope, heads: int,
+                          layers: int, patch: int) -> torch.Tensor:
+    """cogvideox_transformer_3d.py:72-160 for the rotary-embedding model: [B, F, C, H, W] -> [B, F, C_out, H, W]."""
+    from . import blocks as BL
+
+    B, F, _, H, W = video.shape
+    D = p["patch_embed.proj.weight"].shape[0]
+    t_emb = timestep_embedding(timestep, D)
+    emb = O.linear(O.silu(O.linear(t_emb, p["time_embedding.linear_1.weight"], p["time_embedding.linear_1.bias"])),
+                   p["time_embedding.linear_2.weight"], p["time_embedding.linear_2.bias"])
+    joint = cogvideox_patch_embed(p, "patch_embed.", text, video)
+    n_txt = text.shape[1]
+    enc, hid = joint[:, :n_txt], joint[:, n_txt:]
+    for i in range(layers):
+        pre = f"transformer_blocks.{i}."
+        bp = {k[len(pre):]: v for k, v in p.items() if k.startswith(pre)}
+        hid, enc = BL.cogvideox_block(bp, hid, enc, emb, rope, heads)
+    joint = O.layer_norm(torch.cat([enc, hid], dim=1), 1e-5, p["norm_final.weight"], p["norm_final.bias"])
+    hid = ada_layer_norm(p, "norm_out.", joint[:, n_txt:], emb)
+    out = O.linear(hid, p["proj_out.weight"], p["proj_out.bias"])
+    channels = p["proj_out.weight"].shape[0] // (patch * patch)
+    return unpatchify_channel_major(out, F, channels, H, W, patch)

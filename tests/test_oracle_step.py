@@ -177,3 +177,38 @@ def test_flux_conditioning_against_torch_modules():
     assert torch.allclose(S.flux_conditioning(p, "e.", t, pooled, g), want, atol=1e-5)
     want = emb("timestep_embedder", S.timestep_embedding(tb, 256)) + emb("text_embedder", pooled)
     assert torch.allclose(S.flux_conditioning(p, "e.", t, pooled, None), want, atol=1e-5)
+
+
+def test_cogvideox_head_tail_against_torch():
+    torch.manual_seed(6)
+    B, Fr, C, H, W, D, E, Nt, p = 2, 3, 4, 6, 8, 24, 10, 5, 2
+    conv, tproj = torch.nn.Conv2d(C, D, p, stride=p), torch.nn.Linear(E, D)
+    prm = {"pe.proj.weight": conv.weight.detach(), "pe.proj.bias": conv.bias.detach(),
+           "pe.text_proj.weight": tproj.weight.detach(), "pe.text_proj.bias": tproj.bias.detach()}
+    text, video = torch.randn(B, Nt, E), torch.randn(B, Fr, C, H, W)
+    # the wrapper's own expressions: conv per frame, flatten(3).transpose(2, 3), flatten(1, 2), cat [text, video]
+    img = conv(video.reshape(-1, C, H, W)).view(B, Fr, D, H // p, W // p).flatten(3).transpose(2, 3).flatten(1, 2)
+    want = torch.cat([tproj(text), img], dim=1)
+    assert torch.allclose(S.cogvideox_patch_embed(prm, "pe.", text, video), want, atol=1e-5)
+
+    # AdaLayerNorm (shift first, affine LayerNorm)
+    lin, ln = torch.nn.Linear(7, 2 * D), torch.nn.LayerNorm(D, eps=1e-5)
+    with torch.no_grad():
+        ln.weight.normal_(1, 0.1), ln.bias.normal_(0, 0.1)
+    q = {"n.linear.weight": lin.weight.detach(), "n.linear.bias": lin.bias.detach(), "n.norm.weight": ln.weight.detach(),
+         "n.norm.bias": ln.bias.detach()}
+    x, temb = torch.randn(B, 9, D), torch.randn(B, 7)
+    shift, scale = lin(F.silu(temb)).chunk(2, dim=1)
+    want = ln(x) * (1 + scale[:, None]) + shift[:, None]
+    assert torch.allclose(S.ada_layer_norm(q, "n.", x, temb), want, atol=1e-5)
+
+    # channel-major unpatchify: token (f, hy, wx), column (c, py, px) -> out[b, f, c, hy p + py, wx p + px]
+    h, w = H // p, W // p
+    tok = torch.arange(B * Fr * h * w * C * p * p, dtype=torch.float32).reshape(B, Fr * h * w, C * p * p)
+    out = S.unpatchify_channel_major(tok, Fr, C, H, W, p)
+    assert out.shape == (B, Fr, C, H, W)
+    for (b, f, c, hy, py, wx, px) in [(0, 0, 0, 0, 0, 0, 0), (1, 2, 3, 2, 1, 3, 0), (0, 1, 2, 1, 0, 2, 1)]:
+        assert out[b, f, c, hy * p + py, wx * p + px] == tok[b, (f * h + hy) * w + wx, (c * p + py) * p + px]
+    # F.fold takes exactly channel-major columns
+    cols = tok.reshape(B * Fr, h * w, C * p * p).transpose(1, 2)
+    assert torch.equal(F.fold(cols, (H, W), kernel_size=p, stride=p).view(B, Fr, C, H, W), out)
