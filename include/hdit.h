@@ -77,6 +77,11 @@ typedef struct hdit_gemm_problem {
 
 int hdit_gemm_bf16(const hdit_gemm_problem* problems, int count, void* stream);
 
+/* Test hook without a counterpart in the reference: pins the tile shape of
+ * every later hdit_gemm_bf16 call of the process (0: 256x192, 1: 128x256,
+ * 2: 128x128, 3: 256x256; -1: back to the planner). */
+void hdit_gemm_force_config(int cfg);
+
 /* ------------------------------------------------------------------------
  * Joint (image + text) flash attention, non-causal, no mask, bf16 in/out,
  * fp32 online softmax on MFMA.

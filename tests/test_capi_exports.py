@@ -33,7 +33,7 @@ def test_header_declares_the_expected_entry_points():
                  "hdit_layernorm_modulate", "hdit_layernorm_modulate_jobs", "hdit_gate_residual", "hdit_adaln_gemv", "hdit_gelu_tanh",
                  "hdit_qk_norm_rope", "hdit_copy_rows", "hdit_patchify", "hdit_unpatchify", "hdit_timestep_embedding",
                  "hdit_silu", "hdit_cfg_euler_step",
-    "hdit_rope_table", "hdit_clock_sample", "hdit_abi_version", "hdit_last_error"):
+    "hdit_rope_table", "hdit_clock_sample", "hdit_gemm_force_config", "hdit_abi_version", "hdit_last_error"):
         assert name in syms
 
 
@@ -84,3 +84,17 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(library):
     assert lib.hdit_layernorm_modulate_jobs(None, 1, 64, None, None, 1e-6, None) == -1
     assert lib.hdit_adaln_gemv(4096, 4096, None, 4096, 9, 16, 64, None) == -2
     assert lib.hdit_qk_norm_rope(None, 1, 1, 1, 64, 1e-6, None) == -1
+
+
+def test_library_exports_nothing_the_header_does_not_declare(library):
+    import shutil
+    import subprocess
+
+    import hetu_dit_amd
+
+    nm = shutil.which("nm")
+    if nm is None:
+        pytest.skip("nm not available")
+    out = subprocess.run([nm, "-D", "--defined-only", hetu_dit_amd.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted({line.split()[-1] for line in out.splitlines() if " T " in line and line.split()[-1].startswith("hdit_")})
+    assert exported == declared_symbols()
