@@ -80,12 +80,56 @@ def build(name):
     return blk, params, {k: (v.numpy() if isinstance(v, torch.Tensor) else v) for k, v in out.items()}
 
 
+STEP_CFG = dict(sample_size=16, patch_size=2, in_channels=16, num_layers=2, attention_head_dim=64, num_attention_heads=2,
+                joint_attention_dim=64, caption_projection_dim=128, pooled_projection_dim=64, out_channels=16,
+                pos_embed_max_size=12)
+
+
+def step_params(model):
+    """fp32 parameters and buffers of a whole-transformer model under the unwrapped names the oracle uses."""
+    out = {}
+    for stack in ("transformer_blocks", "single_transformer_blocks"):
+        for i, blk in enumerate(getattr(model, stack, [])):
+            for k, v in oracle_params(blk).items():
+                out[f"{stack}.{i}.{k}"] = v
+    for name, p in list(model.named_parameters()) + list(model.named_buffers()):
+        if "transformer_blocks." not in name:
+            out[name.replace(".module.", ".")] = p.detach().float().cpu()
+    return out
+
+
+def build_step():
+    """A tiny SD3 transformer from latent to predicted noise, the guided Euler update and the sigma schedule."""
+    from hetu_dit_amd.transformer_sd3 import SD3Transformer2DModel
+    from oracle import step as S
+
+    reset_cache_manager()
+    model = SD3Transformer2DModel(**STEP_CFG)
+    synthetic.init_module_(model, 201)
+    params = step_params(model)
+    checksum = float(sum(v.double().abs().sum() for k, v in params.items() if not k.endswith("pos_embed.pos_embed")))
+    lat = synthetic.randn_bf16((2, 16, 16, 24), 2011).float()
+    enc = synthetic.randn_bf16((2, 11, 64), 2012).float()
+    pooled = synthetic.randn_bf16((2, 64), 2013).float()
+    t = torch.tensor([640.0, 640.0])
+    noise = S.sd3_transformer(params, lat, enc, pooled, t, STEP_CFG["num_attention_heads"], STEP_CFG["num_layers"],
+                              STEP_CFG["patch_size"], STEP_CFG["pos_embed_max_size"])
+    new = S.cfg_euler_step(noise[:1], noise[1:], lat[:1], 7.0, 0.9, 0.8)
+    out = dict(weights_abs_sum=np.float64(checksum), latent=lat, encoder_hidden_states=enc, pooled=pooled, timestep=t,
+               noise=noise, guided_step=new.float(), sigmas_10=S.flow_match_sigmas(10))
+    return model, params, {k: (v.numpy() if isinstance(v, torch.Tensor) else v) for k, v in out.items()}
+
+
 def main():
     for name in CASES:
         _, _, arrays = build(name)
         path = os.path.join(HERE, name + ".npz")
         np.savez_compressed(path, **arrays)
         print(f"{path}: {os.path.getsize(path) / 1024:.1f} KiB")
+    _, _, arrays = build_step()
+    path = os.path.join(HERE, "sd3_step.npz")
+    np.savez_compressed(path, **arrays)
+    print(f"{path}: {os.path.getsize(path) / 1024:.1f} KiB")
 
 
 if __name__ == "__main__":
