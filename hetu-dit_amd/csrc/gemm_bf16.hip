@@ -645,7 +645,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
     if (t < single_cost) single_cost = t, single = c;
   }
   // plan B: one launch, two shapes -- the problems that want 256-row tiles on the better of the two large
-  // shapes, the others on 128x128
+  // shapes, the others on the better of the two 128-row shapes
   hdit_gemm_problem big[HDIT_GEMM_MAX_PROBLEMS], small[HDIT_GEMM_MAX_PROBLEMS];
   const hdit_gemm_problem* pb[HDIT_GEMM_MAX_PROBLEMS];
   const hdit_gemm_problem* psm[HDIT_GEMM_MAX_PROBLEMS];
@@ -655,21 +655,27 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
     else small[ns] = live[i], psm[ns] = &live[i], ns++;
   }
   double two_cost = 1e30;
-  int big_cfg = 0;
+  int big_cfg = 0, small_cfg = 2;
   if (nb > 0 && ns > 0) {
     const double t0 = tiles_time(pb, nb, 0), t3 = tiles_time(pb, nb, 3);
     big_cfg = t3 < t0 ? 3 : 0;
-    two_cost = kLaunchUs + (t3 < t0 ? t3 : t0) + tiles_time(psm, ns, 2);
+    // the short problems on 128x128 or, when that needs a second round, on 128x256
+    const double s2 = tiles_time(psm, ns, 2), s1 = tiles_time(psm, ns, 1);
+    small_cfg = s1 < s2 ? 1 : 2;
+    two_cost = kLaunchUs + (t3 < t0 ? t3 : t0) + (s1 < s2 ? s1 : s2);
   }
   static const bool debug = getenv("HDIT_GEMM_DEBUG") != nullptr;
   if (debug) {
     fprintf(stderr, "hdit_gemm_bf16 plan:");
     for (int i = 0; i < nlive; i++) fprintf(stderr, " [%dx%dx%d epi%d own%d]", live[i].m, live[i].n, live[i].k, live[i].epilogue, own[i]);
-    fprintf(stderr, " single cfg%d %.1f us, two-shape(big cfg%d) %.1f us\n", single, single_cost, big_cfg, two_cost);
+    fprintf(stderr, " single cfg%d %.1f us, two-shape(big cfg%d, small cfg%d) %.1f us\n", single, single_cost, big_cfg,
+            small_cfg, two_cost);
   }
   if (two_cost < single_cost) {
-    if (big_cfg == 0) return launch2<Cfg256x192, Cfg128x128>(big, nb, small, ns, s);
-    return launch2<Cfg256x256, Cfg128x128>(big, nb, small, ns, s);
+    if (big_cfg == 0 && small_cfg == 2) return launch2<Cfg256x192, Cfg128x128>(big, nb, small, ns, s);
+    if (big_cfg == 0) return launch2<Cfg256x192, Cfg128x256>(big, nb, small, ns, s);
+    if (small_cfg == 2) return launch2<Cfg256x256, Cfg128x128>(big, nb, small, ns, s);
+    return launch2<Cfg256x256, Cfg128x256>(big, nb, small, ns, s);
   }
   return launch_cfg(single, live, nlive, s);
 }
