@@ -260,9 +260,8 @@ def main():
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
     clk1 = ops.clock_sample()
     torch.cuda.synchronize()
-    d_clk = (clk1 - clk0).tolist()
-    # average shader clock over the timed passes: shader-clock ticks per tick of the constant 100 MHz counter
-    shader_clock_ghz = d_clk[0] / d_clk[1] * 0.1 if d_clk[1] > 0 else None
+    # average shader clock over the timed passes (counter pairs per CU, median)
+    shader_clock_ghz = ops.shader_clock_ghz(clk0, clk1)
 
     # one plain device copy of known size (256 MiB read + 256 MiB written): the scale reference for the
     # FETCH_SIZE / WRITE_SIZE hardware counters when this command runs under `rocprofv3 --pmc`

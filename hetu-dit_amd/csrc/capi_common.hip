@@ -27,17 +27,21 @@ extern "C" __attribute__((visibility("default"))) int hdit_abi_version(void) { r
 extern "C" __attribute__((visibility("default"))) const char* hdit_last_error(void) { return g_err; }
 
 namespace {
-// one lane stores the shader-clock counter and the constant 100 MHz counter
+// Lane 0 of every workgroup stores {shader-clock counter, constant 100 MHz counter, XCD id, hardware id}.
+// Every CU counts its own shader clock, so samples can only be paired within one CU.
 __global__ void clock_sample_kernel(unsigned long long* out) {
   if (threadIdx.x == 0) {
-    out[0] = __builtin_amdgcn_s_memtime();
-    out[1] = __builtin_amdgcn_s_memrealtime();
+    unsigned long long* o = out + 4 * blockIdx.x;
+    o[0] = __builtin_amdgcn_s_memtime();
+    o[1] = __builtin_amdgcn_s_memrealtime();
+    o[2] = __builtin_amdgcn_s_getreg((3 << 11) | 20);   // HW_REG_XCC_ID, bits 3:0
+    o[3] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_REG_HW_ID
   }
 }
 }  // namespace
 
-extern "C" __attribute__((visibility("default"))) int hdit_clock_sample(void* out, void* stream) {
-  if (!out || (((uintptr_t)out) & 7)) return HDIT_EINVAL;
-  hipLaunchKernelGGL(clock_sample_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)out);
+extern "C" __attribute__((visibility("default"))) int hdit_clock_sample(void* out, int slots, void* stream) {
+  if (!out || (((uintptr_t)out) & 7) || slots <= 0 || slots > 1024) return HDIT_EINVAL;
+  hipLaunchKernelGGL(clock_sample_kernel, dim3(slots), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)out);
   return hdit_host::check_launch("hdit_clock_sample");
 }

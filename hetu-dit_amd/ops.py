@@ -458,8 +458,33 @@ def rope_table(positions: torch.Tensor, axes_dim, theta: float = 10000.0) -> Tup
     return cos, sin
 
 
-def clock_sample() -> torch.Tensor:
-    """int64 [2] on the device, filled on the current stream with (shader-clock counter, 100 MHz counter)."""
-    out = torch.zeros(2, dtype=torch.int64, device="cuda")
-    check(_lib.lib().hdit_clock_sample(out.data_ptr(), _stream()), "hdit_clock_sample")
+def clock_sample(slots: int = 1024) -> torch.Tensor:
+    """int64 [slots, 4] on the device, filled on the current stream with (shader-clock counter, 100 MHz counter,
+    XCD id, hardware id) of `slots` one-wave workgroups (enough of them to land on every CU)."""
+    out = torch.zeros(slots, 4, dtype=torch.int64, device="cuda")
+    check(_lib.lib().hdit_clock_sample(out.data_ptr(), slots, _stream()), "hdit_clock_sample")
     return out
+
+
+def shader_clock_ghz(before: torch.Tensor, after: torch.Tensor) -> Optional[float]:
+    """Average shader clock between two ``clock_sample`` results.  Every CU counts its own shader clock, so a
+    sample is paired with the later sample of the same CU (XCD id + shader-engine / shader-array / CU fields of the
+    hardware id); the median over the CUs is returned (None if no pair is usable)."""
+    def cu_key(row):
+        return (row[2], (row[3] >> 8) & 0xFF)
+
+    first = {}
+    for row in before.cpu().tolist():
+        first.setdefault(cu_key(row), row)
+    rates, seen = [], set()
+    for row in after.cpu().tolist():
+        k = cu_key(row)
+        if k in first and k not in seen:
+            seen.add(k)
+            d_ticks, d_real = row[0] - first[k][0], row[1] - first[k][1]
+            if d_ticks > 0 and d_real > 0:
+                rates.append(d_ticks / d_real * 0.1)
+    if not rates:
+        return None
+    rates.sort()
+    return rates[len(rates) // 2]

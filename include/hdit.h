@@ -30,12 +30,15 @@ extern "C" {
 int hdit_abi_version(void);
 /* Static string describing the last HDIT_ELAUNCH on this thread ("" if none). */
 const char* hdit_last_error(void);
-/* Measurement aid without a counterpart in the reference: enqueues a one-wave
- * kernel that stores two 64-bit counters to out[0..1] (device memory, 8-byte
- * aligned): the shader-clock counter and the constant 100 MHz counter.  Two
- * samples on one stream, around the work being timed, give the average shader
- * clock the work ran at: (d out[0]) / (d out[1]) x 100 MHz. */
-int hdit_clock_sample(void* out, void* stream);
+/* Measurement aid without a counterpart in the reference: enqueues `slots`
+ * one-wave workgroups (<= 1024; they spread over the CUs); workgroup i stores
+ * four 64-bit values to out[4i..4i+3] (device memory, 8-byte aligned): the
+ * shader-clock counter, the constant 100 MHz counter, the id of the XCD it ran
+ * on, and the hardware id register (shader engine / array / CU in bits 8-15).
+ * Every CU counts its own shader clock: two samples taken on the same CU around
+ * the work being timed give the average shader clock the work ran at,
+ * (d out[0]) / (d out[1]) x 100 MHz. */
+int hdit_clock_sample(void* out, int slots, void* stream);
 
 /* ------------------------------------------------------------------------
  * Grouped bf16 GEMM with fused epilogue:  C = epilogue(A . B^T + bias)
