@@ -249,3 +249,43 @@ def test_clock_sample_counts_forward(hdit):
     assert bool((b[:, 1] > a[:, 1]).all())  # the 100 MHz counter is global
     ghz = hdit.ops.shader_clock_ghz(a, b)
     assert ghz is not None and 0.05 < ghz < 3.5, ghz  # a plausible shader clock
+
+
+def test_unpatchify_channel_major_exact(hdit):
+    torch.manual_seed(1)
+    B, Fr, C, H, W, p = 1, 3, 16, 12, 20, 2
+    x = torch.randn(B, Fr * (H // p) * (W // p), C * p * p).bfloat16()
+    got = hdit.ops.unpatchify(x.view(B * Fr, -1, C * p * p).to(DEV), C, H, W, p, channel_major=True)
+    assert torch.equal(got.cpu().view(B, Fr, C, H, W), S.unpatchify_channel_major(x, Fr, C, H, W, p))
+
+
+def test_cogvideox_transformer_video_to_noise(hdit):
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.layers.embeddings import hetuDiTCogVideoXPatchEmbedWrapper
+    from hetu_dit_amd.layers.modules import CogVideoXPatchEmbed
+    from hetu_dit_amd.registry import hetuDiTLayerWrappersRegister
+    from hetu_dit_amd.transformer_cogvideox import CogVideoXTransformer3DModel
+    from oracle import ops as O
+
+    heads, L, Fr, H, W, Nt = 4, 2, 3, 12, 20, 34
+    model = CogVideoXTransformer3DModel(num_attention_heads=heads, attention_head_dim=64, num_layers=L, text_embed_dim=128,
+                                        time_embed_dim=64)
+    synthetic.init_module_(model, 31)
+    assert hetuDiTLayerWrappersRegister.get_wrapper(model.patch_embed.module) is hetuDiTCogVideoXPatchEmbedWrapper
+    assert isinstance(model.patch_embed.module, CogVideoXPatchEmbed)
+    params = step_params(model)
+    model = model.to(DEV)
+    B = 1
+    video = synthetic.randn_bf16((B, Fr, 16, H, W), 32)
+    text = synthetic.randn_bf16((B, Nt, 128), 33)
+    t = torch.tensor([731.0])
+    pos = synthetic.cogvideox_positions(Fr, H // 2, W // 2)
+    cos, sin = hdit.ops.rope_table(pos.float().to(DEV), (16, 24, 24))
+    got = model(video.to(DEV), text.to(DEV), t.to(DEV), (cos, sin))
+    torch.cuda.synchronize()
+    rope = O.cogvideox_rope_table(Fr, H // 2, W // 2, 64)
+    want = S.cogvideox_transformer(params, video.float(), text.float(), t, rope, heads, L, 2)
+    assert got.shape == video.shape
+    assert_parity(got, want, what="cogvideox transformer")
+    joint = model.patch_embed(text.to(DEV), video.to(DEV))
+    assert_parity(joint, S.cogvideox_patch_embed(params, "patch_embed.", text.float(), video.float()), what="cogvideox patch embed")
