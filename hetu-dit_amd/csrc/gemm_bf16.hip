@@ -67,10 +67,22 @@ struct Cfg {
   static constexpr int B_LOADS = BN / 8 / NW;
   static constexpr int LOADS = A_LOADS + B_LOADS;
   static constexpr int A_BYTES = BM * ROW_BYTES;
+  static constexpr int B_BYTES = BN * ROW_BYTES;
   static constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
-  static constexpr int BIAS_OFF = 2 * STAGE_BYTES;  // one 1 KiB bias slot per wave
-  static constexpr int LDS_BYTES = BIAS_OFF + NW * 1024;
-  static_assert(NW * EPI_WAVE_BYTES <= STAGE_BYTES, "the epilogue windows live inside one stage");
+  // DMA: the 256-row shapes take their operand slabs straight from global memory into LDS
+  // (global_load_lds_dwordx4: no staging registers, no ds_write).  A has three slots (requested two slabs
+  // ahead), B two (requested one slab ahead, first in the queue); the epilogue windows alias the A slot the
+  // tile's last slab vacated, which is exactly as large.  The bias slots exist when they still fit.
+  static constexpr bool DMA = TM == 4;
+  static constexpr int A_SLOTS = 3, B_SLOTS = 2;
+  static constexpr int B_OFF = A_SLOTS * A_BYTES;
+  static constexpr int DMA_BYTES = A_SLOTS * A_BYTES + B_SLOTS * B_BYTES;
+  static constexpr bool BIAS_IN_LDS = !DMA || DMA_BYTES + NW * 1024 <= 160 * 1024;
+  static constexpr int BIAS_OFF = DMA ? DMA_BYTES : 2 * STAGE_BYTES;  // one 1 KiB bias slot per wave
+  static constexpr int LDS_BYTES = BIAS_OFF + (BIAS_IN_LDS ? NW * 1024 : 0);
+  static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
+  static_assert(DMA ? NW * EPI_WAVE_BYTES <= A_BYTES : NW * EPI_WAVE_BYTES <= STAGE_BYTES,
+                "the epilogue windows live inside one stage (one A slot)");
   static_assert(TN <= 4, "epilogue staging window is 128 columns wide");
 };
 
@@ -113,6 +125,9 @@ __device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
 
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// s_waitcnt immediate that waits for all but the newest n vector-memory operations (and for nothing else)
+constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0f70; }
+
 // All tiles of one shape that this workgroup owns.
 template <class C>
 __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles, int tiles_per_xcd, int wgs_per_xcd,
@@ -141,13 +156,17 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
   const int ld_chunk = lane & 7;
   const int st_row = wave * 8 + ld_row;
   const int st_off = st_row * ROW_BYTES + ((ld_chunk ^ ((st_row >> 1) & 7)) << 4);
+  // A direct-to-LDS request lands lane l at byte 16*l of the wave's 1 KiB (row l/8, position l%8), so the
+  // swizzle is applied on the source side: position c' of row r receives chunk c' ^ ((r>>1)&7).
+  const int src_chunk = C::DMA ? (ld_chunk ^ ((st_row >> 1) & 7)) : ld_chunk;
+  const unsigned lds_base_addr = __builtin_amdgcn_readfirstlane(lds_address(lds));
   int p_lid = lid;
   bool p_valid = true;
   int p_kt = 0, p_KT = 0;
   const unsigned char* p_abase = nullptr;
   const unsigned char* p_bbase = nullptr;
   unsigned p_off[C::LOADS];
-  i32x4 G[C::LOADS];  // the slab in flight between global memory and LDS
+  i32x4 G[C::DMA ? 1 : C::LOADS];  // the slab in flight between global memory and LDS (register-staged shapes)
   auto p_setup = [&]() {
     const TileCoord tc = locate<C>(tab, p_lid);
     const hdit_gemm_problem& pr = tab.p[tc.pi];
@@ -158,12 +177,12 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
 #pragma unroll
     for (int i = 0; i < C::A_LOADS; i++) {
       const int gr = min(tc.m0 + (wave + i * NW) * 8 + ld_row, pr.m - 1);
-      p_off[i] = (unsigned)(((int64_t)gr * pr.lda + ld_chunk * 8) * 2);
+      p_off[i] = (unsigned)(((int64_t)gr * pr.lda + src_chunk * 8) * 2);
     }
 #pragma unroll
     for (int i = 0; i < C::B_LOADS; i++) {
       const int gr = min(tc.n0 + (wave + i * NW) * 8 + ld_row, pr.n - 1);
-      p_off[C::A_LOADS + i] = (unsigned)(((int64_t)gr * pr.ldb + ld_chunk * 8) * 2);
+      p_off[C::A_LOADS + i] = (unsigned)(((int64_t)gr * pr.ldb + src_chunk * 8) * 2);
     }
   };
   // Once the stream is exhausted the last slab is simply loaded again and written to a stage nobody
@@ -171,6 +190,15 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
   auto g_load = [&](int i) {
     const unsigned char* base = (i < C::A_LOADS ? p_abase : p_bbase) + (size_t)p_kt * ROW_BYTES;
     G[i] = *(const i32x4*)(base + p_off[i]);
+  };
+  // direct-to-LDS request i of the slab at the cursor: A rows into A slot `slot`, B rows into B slot `slot`
+  auto dma_a = [&](int slot, int i) {
+    lds_dma16(p_abase + (size_t)p_kt * ROW_BYTES, p_off[i],
+              lds_base_addr + slot * C::A_BYTES + i * (NW * 8 * ROW_BYTES) + wave * 8 * ROW_BYTES);
+  };
+  auto dma_b = [&](int slot, int i) {
+    lds_dma16(p_bbase + (size_t)p_kt * ROW_BYTES, p_off[C::A_LOADS + i],
+              lds_base_addr + C::B_OFF + slot * C::B_BYTES + i * (NW * 8 * ROW_BYTES) + wave * 8 * ROW_BYTES);
   };
   auto l_store = [&](int stage, int i) {
     const int tile_off = i < C::A_LOADS ? i * (NW * 8 * ROW_BYTES) : C::A_BYTES + (i - C::A_LOADS) * (NW * 8 * ROW_BYTES);
@@ -191,15 +219,16 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
   // l32 plus a multiple of 32, so (r>>1)&7 == (l32>>1)&7.  k-step ks uses chunk 2*ks + lh.
   const int swz = (l32 >> 1) & 7;
   const int a_row = (wm0 + l32) * ROW_BYTES;
-  const int b_row = C::A_BYTES + (wn0 + l32) * ROW_BYTES;
+  const int b_row = (wn0 + l32) * ROW_BYTES;
   bf16x8 fa[2][TM], fb[2][TN];
-  auto read_frags = [&](const unsigned char* sbase, int ks, int buf) {
+  auto read_frags2 = [&](const unsigned char* abase, const unsigned char* bbase, int ks, int buf) {
     const int ch = ((ks * 2 + lh) ^ swz) << 4;
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[buf][i] = *(const bf16x8*)(sbase + a_row + ch + i * 32 * ROW_BYTES);
+    for (int i = 0; i < TM; i++) fa[buf][i] = *(const bf16x8*)(abase + a_row + ch + i * 32 * ROW_BYTES);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb[buf][j] = *(const bf16x8*)(sbase + b_row + ch + j * 32 * ROW_BYTES);
+    for (int j = 0; j < TN; j++) fb[buf][j] = *(const bf16x8*)(bbase + b_row + ch + j * 32 * ROW_BYTES);
   };
+  auto read_frags = [&](const unsigned char* sbase, int ks, int buf) { read_frags2(sbase, sbase + C::A_BYTES, ks, buf); };
 
   // Bias of a tile: every wave copies the 32*TN bias values of its own columns (8 per lane, lanes past the
   // end clamped) into a private LDS slot when it starts the tile; the copy is older than the loads of the
@@ -210,23 +239,41 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
   auto issue_bias = [&](const TileCoord& tc) {
     const hdit_gemm_problem& pr = tab.p[tc.pi];
     const unsigned char* src = pr.bias ? (const unsigned char*)pr.bias : (const unsigned char*)pr.b;
-    lds_dma16(src, (unsigned)(min(tc.n0 + wn0 + lane * 8, pr.n - 8) * 2), bias_lds);
+    if constexpr (C::BIAS_IN_LDS) lds_dma16(src, (unsigned)(min(tc.n0 + wn0 + lane * 8, pr.n - 8) * 2), bias_lds);
   };
   issue_bias(locate<C>(tab, lid));
 
   // prologue: slab 0 into stage 0, slab 1 into the registers
   p_setup();
-#pragma unroll
-  for (int i = 0; i < C::LOADS; i++) g_load(i);
-  p_advance();
-#pragma unroll
-  for (int i = 0; i < C::LOADS; i++) l_store(0, i);
-#pragma unroll
-  for (int i = 0; i < C::LOADS; i++) g_load(i);
-  p_advance();
-  __syncthreads();
   int stage = 0;
-  read_frags(lds, 0, 0);
+  int sa = 0, sb = 0;  // DMA: the A and B slots of the slab being multiplied
+  if constexpr (C::DMA) {
+    // slab 0 into slots (0, 0), slab 1 into slots (1, 1); slab 0 has landed before the first fragment read
+#pragma unroll
+    for (int i = 0; i < C::A_LOADS; i++) dma_a(0, i);
+#pragma unroll
+    for (int i = 0; i < C::B_LOADS; i++) dma_b(0, i);
+    p_advance();
+#pragma unroll
+    for (int i = 0; i < C::A_LOADS; i++) dma_a(1, i);
+#pragma unroll
+    for (int i = 0; i < C::B_LOADS; i++) dma_b(1, i);
+    p_advance();
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(C::LOADS));
+    __syncthreads();
+    read_frags2(lds, lds + C::B_OFF, 0, 0);
+  } else {
+#pragma unroll
+    for (int i = 0; i < C::LOADS; i++) g_load(i);
+    p_advance();
+#pragma unroll
+    for (int i = 0; i < C::LOADS; i++) l_store(0, i);
+#pragma unroll
+    for (int i = 0; i < C::LOADS; i++) g_load(i);
+    p_advance();
+    __syncthreads();
+    read_frags(lds, 0, 0);
+  }
 
   constexpr int NMMA = TM * TN;
   constexpr int NRD = TM + TN;            // fragment reads per k-step
@@ -286,6 +333,58 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
       }
     };
 
+    // The same k-step for the direct-to-LDS shapes: under the MFMAs that carry no fragment reads, requests
+    // [first, last) of the slab at the cursor -- A rows (kind 0) or B rows (kind 1) -- into slot `slot`.
+    auto k_step_dma = [&](int buf, const unsigned char* rd_a, const unsigned char* rd_b, int rd_ks, int kind, int first,
+                          int last, int slot) {
+      read_frags2(rd_a, rd_b, rd_ks, buf ^ 1);
+#pragma unroll
+      for (int t = 0; t < NMMA; t++) {
+        acc[t / TN][t % TN] =
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][t % TN], fa[buf][t / TN], acc[t / TN][t % TN], 0, 0, 0);
+        if (t == RD_MFMA - 1) {
+#pragma unroll
+          for (int u = 0; u < RD_MFMA; u++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // MFMA
+            if (2 * u + 2 <= NRD) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // DS reads
+            else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          SCHED_FENCE();
+        }
+        if (t >= RD_MFMA) {
+          const int n = last - first;
+#pragma unroll
+          for (int j = 0; j < C::LOADS; j++)
+            if (j < n && RD_MFMA + (j * SLOTS) / (n > 0 ? n : 1) == t) {
+              if (kind == 0) dma_a(slot, first + j);
+              else dma_b(slot, first + j);
+            }
+          SCHED_FENCE();
+        }
+      }
+    };
+    constexpr int CPA = (C::A_LOADS + 2) / 3;  // A requests per k-step (k-steps 0..2 of a slab)
+
+    if constexpr (C::DMA) {
+      for (int kt = 0; kt < KT; kt++) {
+        const unsigned char* ab = lds + sa * C::A_BYTES;
+        const unsigned char* bb = lds + C::B_OFF + sb * C::B_BYTES;
+        // A rows of the slab after next go to the slot the previous slab vacated
+        const int sa_req = sa == 0 ? C::A_SLOTS - 1 : sa - 1;
+        k_step_dma(0, ab, bb, 1, 0, 0, CPA, sa_req);
+        k_step_dma(1, ab, bb, 2, 0, CPA, 2 * CPA, sa_req);
+        k_step_dma(0, ab, bb, 3, 0, 2 * CPA, C::A_LOADS, sa_req);
+        // ---- turn over: everything but the A requests just issued has landed (the next slab is complete),
+        // and the fragments of the last k-step are in registers
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(C::A_LOADS) & 0xf0ff);  // and lgkmcnt(0)
+        __syncthreads();
+        const int sb_req = sb;  // the B slot this slab vacates takes the B rows of the slab after next
+        sa = sa == C::A_SLOTS - 1 ? 0 : sa + 1;
+        sb ^= 1;
+        k_step_dma(1, lds + sa * C::A_BYTES, lds + C::B_OFF + sb * C::B_BYTES, 0, 1, 0, C::B_LOADS, sb_req);
+        p_advance();
+      }
+    } else
     for (int kt = 0; kt < KT; kt++) {
       const unsigned char* sbase = lds + stage * C::STAGE_BYTES;
       const int wstage = stage ^ 1;  // held slab h-1; every wave passed the barrier of that slab
@@ -299,10 +398,14 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
       stage ^= 1;
       k_step(1, lds + stage * C::STAGE_BYTES, 0, wstage, 0, 0);
     }
-    unsigned char* epi = lds + (stage ^ 1) * C::STAGE_BYTES + wave * EPI_WAVE_BYTES;  // the stage just vacated
+    // staging window of this wave: inside the stage (the A slot) the tile's last slab vacated
+    unsigned char* epi = lds + wave * EPI_WAVE_BYTES +
+                         (C::DMA ? (sa == 0 ? C::A_SLOTS - 1 : sa - 1) * C::A_BYTES : (stage ^ 1) * C::STAGE_BYTES);
 
     // ---- epilogue ---------------------------------------------------------
-    if (KT < 2) __builtin_amdgcn_s_waitcnt(0x0f70);  // the bias copy is only known to have landed after the second slab's loads
+    // register-staged shapes: the bias copy is only known to have landed after the second slab's loads
+    // (direct-to-LDS shapes: the wait before every slab's barrier covers it)
+    if (!C::DMA && KT < 2) __builtin_amdgcn_s_waitcnt(0x0f70);
     auto epilogue = [&](auto mode_tag) {
       constexpr int MODE = decltype(mode_tag)::value;
       constexpr bool GATED = MODE == HDIT_EPI_GATE_RESIDUAL;
@@ -343,6 +446,15 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
         gte0 = *(const f32x4*)g;
         gte1 = *(const f32x4*)(g + 4);
       };
+      i32x4 breg[C::BIAS_IN_LDS ? 1 : 2 * TN];  // the bias of this lane's columns when it has no LDS slot
+      if constexpr (!C::BIAS_IN_LDS) {
+#pragma unroll
+        for (int c = 0; c < 2 * TN; c++) {
+          const int col = min(ncol0 + ((c >> 1) * 4 + 2 * (c & 1) + lh) * 8, N - 8);
+          breg[c] = i32x4{0, 0, 0, 0};
+          if (pr.bias) breg[c] = *(const i32x4*)((const unsigned char*)pr.bias + (unsigned)(col * 2));
+        }
+      }
       if (GATED) {
         prefetch_rows(0, 0);
         prefetch_rows(0, 1);
@@ -367,7 +479,8 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
               v[4 + e] = __int_as_float(sw[1]);
             }
             const int chunk = j * 4 + 2 * gp + lh;  // 16-byte chunk inside the wave's 256-byte row
-            hdit::unpack8(*(const i32x4*)(bias_slot + (chunk << 4)) & bias_mask, bf);
+            if constexpr (C::BIAS_IN_LDS) hdit::unpack8(*(const i32x4*)(bias_slot + (chunk << 4)) & bias_mask, bf);
+            else hdit::unpack8(breg[j * 2 + gp], bf);
 #pragma unroll
             for (int e = 0; e < 8; e++) v[e] += bf[e];
             if (MODE == HDIT_EPI_BIAS_GELU) {
@@ -425,9 +538,14 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     else if (pr.epilogue == HDIT_EPI_BIAS_GELU) epilogue(std::integral_constant<int, HDIT_EPI_BIAS_GELU>{});
     else epilogue(std::integral_constant<int, HDIT_EPI_GATE_RESIDUAL>{});
 
+    // Direct-to-LDS shapes: the compiler does not see the requests in flight, so a wait it placed inside the
+    // main loop for a load of the epilogue would drain them; leave nothing of the epilogue in flight.
+    if constexpr (C::DMA) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     lid += wgs_per_xcd;
     if (lid >= xcd_end) break;
   }
+  // requests past the end of the stream are still in flight: nothing may land in LDS after this returns
+  if constexpr (C::DMA) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 }
 
 template <class C>

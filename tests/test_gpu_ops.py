@@ -21,7 +21,7 @@ def rnd(*shape, scale=1.0, seed=None):
     return bf16_round(torch.randn(*shape, generator=gen) * scale)
 
 
-@pytest.mark.parametrize("cfg", [-1, 0, 1, 2])
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 64), (300, 384, 128), (666, 1536, 1536), (1, 128, 64), (1024, 512, 256)])
 def test_gemm_bias(hdit, m, n, k, cfg):
     print(f"gemm_bias m={m} n={n} k={k} cfg={cfg}", flush=True)
@@ -63,6 +63,37 @@ def test_gemm_gelu_and_gate_residual_grouped(hdit):
     torch.cuda.synchronize()
     want = x1 + gate[:, None, D:2 * D] * O.linear(hh, w3, b3)
     assert_parity(res, want, what="gate residual")
+
+
+@pytest.mark.parametrize("cfg", [0, 3])
+@pytest.mark.parametrize("m,n,k", [(4096, 4608, 64), (2500, 3000, 192), (5000, 2056, 320)])
+@pytest.mark.parametrize("epi", ["bias", "nobias", "gate"])
+def test_gemm_many_short_tiles_per_workgroup(hdit, m, n, k, cfg, epi):
+    """More tiles than workgroups with one, three and five slabs per tile: the operand stream of the 256-row
+    shapes runs two slabs ahead of the MFMAs across tile boundaries, through three A slots and two B slots, so
+    the slot a tile ends on (and the one its epilogue stages through) differs from tile to tile."""
+    print(f"gemm short tiles m={m} n={n} k={k} cfg={cfg} epi={epi}", flush=True)
+    ops = hdit.ops
+    a, w, b = rnd(m, k, seed=31), rnd(n, k, scale=0.05, seed=32), rnd(n, seed=33)
+    hdit._lib.lib().hdit_gemm_force_config(cfg)
+    try:
+        if epi == "gate":
+            r = rnd(m, n, seed=34)
+            gate = torch.randn(2, n, generator=torch.Generator().manual_seed(35))
+            rows = (m + 1) // 2
+            out = g(r).clone()
+            ops.gemm_launch([ops.gemm_problem(g(a), g(w), out, g(b), ops.EPI_GATE_RESIDUAL, resid=out, gate=gate.to(DEV),
+                                              rows_per_batch=rows)])
+            lin = O.linear(a, w, b)
+            want = r + gate.repeat_interleave(rows, dim=0)[:m] * lin
+        else:
+            out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+            ops.gemm_launch([ops.gemm_problem(g(a), g(w), out, g(b) if epi == "bias" else None, ops.EPI_BIAS)])
+            want = O.linear(a, w, b if epi == "bias" else None)
+        torch.cuda.synchronize()
+        assert_parity(out, want, what=f"gemm short tiles {epi}")
+    finally:
+        hdit._lib.lib().hdit_gemm_force_config(-1)
 
 
 @pytest.mark.parametrize("epi", ["bias", "gelu", "gate"])
