@@ -92,8 +92,15 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
-  const int qt = blockIdx.x % q_tiles;
-  const int bh = blockIdx.x / q_tiles;
+  // Workgroups go to the 8 XCDs round-robin by id, and each XCD has its own L2: all query tiles of one
+  // (batch, head) run on one XCD, so that its K and V are fetched into one L2 instead of eight.
+  int qt = blockIdx.x % q_tiles;
+  int bh = blockIdx.x / q_tiles;
+  if ((P.batch * P.heads) % 8 == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    qt = slot % q_tiles;
+    bh = (slot / q_tiles) * 8 + xcd;
+  }
   const int b = bh / P.heads, h = bh % P.heads;
   const int q0 = qt * BQ + wave * WQ;
 
