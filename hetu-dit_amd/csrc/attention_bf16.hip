@@ -60,7 +60,15 @@ struct Lds {
   static constexpr int K_BYTES = BKV * K_ROW;
   static constexpr int V_BYTES = BKV * V_ROW;
   static constexpr int STAGE = K_BYTES + V_BYTES;
-  static constexpr int TOTAL = 2 * STAGE;
+  // d = 128: the Q fragments (64 registers) live in LDS instead, one private region per wave, rows strided like
+  // the K rows, and are read per k-step next to the K fragments: the registers they would occupy are what the
+  // loop otherwise spills (and reloads from scratch on every tile, with one wave per SIMD to hide nothing).
+  static constexpr bool Q_IN_LDS = HD == 128;
+  static constexpr int Q_ROW = K_ROW;
+  static constexpr int Q_OFF = 2 * STAGE;
+  static constexpr int Q_WAVE_BYTES = WQ * Q_ROW;
+  static constexpr int TOTAL = 2 * STAGE + (Q_IN_LDS ? 4 * Q_WAVE_BYTES : 0);
+  static_assert(TOTAL <= 160 * 1024, "attention tiles do not fit the LDS");
 };
 
 // The running row maximum is only raised when some row's maximum grew by more than this many powers of
@@ -96,7 +104,20 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   const int q0 = qt * BQ + wave * WQ;
 
   // ---- Q fragments: lane holds q row (qb*32 + l32), d = 16*ks + 8*lh .. +7
-  bf16x8 qf[2][KS];
+  bf16x8 qf[2][L::Q_IN_LDS ? 1 : KS];
+  unsigned char* qlds = lds + L::Q_OFF + wave * L::Q_WAVE_BYTES;
+  if constexpr (L::Q_IN_LDS) {
+    // the wave's 64 query rows, 16 lanes per row (coalesced 256-byte rows), into its private LDS region;
+    // only this wave reads them back, so its own wait for the writes is all the synchronisation needed
+    constexpr int RPI = 64 / CPR;  // rows per wave-wide load
+#pragma unroll
+    for (int i = 0; i < WQ / RPI; i++) {
+      const int row = i * RPI + lane / CPR, cc = lane % CPR;
+      const int r = min(q0 + row, P.sq - 1);
+      const i32x4 raw = *(const i32x4*)(row_ptr(P.q, b, h, r) + cc * 8);
+      *(i32x4*)(qlds + row * L::Q_ROW + cc * 16) = raw;
+    }
+  } else
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
     int r = min(q0 + qb * 32 + l32, P.sq - 1);
@@ -204,6 +225,21 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     // ---- S^T[kb][qb] = K_tile . Q^T (first k-step starts from a zero accumulator operand)
     f32x16 sacc[2][2];
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if constexpr (L::Q_IN_LDS) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        bf16x8 qk[2], kf[2];
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) qk[qb] = *(const bf16x8*)(qlds + (qb * 32 + l32) * L::Q_ROW + lh * 16 + ks * 32);
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) kf[kb] = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + ks * 32);
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+          for (int qb = 0; qb < 2; qb++)
+            sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qk[qb], ks == 0 ? zero16 : sacc[kb][qb], 0, 0, 0);
+      }
+    } else
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
