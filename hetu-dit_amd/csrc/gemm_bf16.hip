@@ -663,6 +663,7 @@ using Cfg256x256 = Cfg<4, 4>;
 using Cfg256x192 = Cfg<4, 3>;
 using Cfg128x256 = Cfg<2, 4>;
 using Cfg128x128 = Cfg<2, 2>;
+using Cfg128x192 = Cfg<2, 3>;
 
 std::atomic<int> g_force_cfg{-1};
 
@@ -672,12 +673,12 @@ std::atomic<int> g_force_cfg{-1};
 // block) are badly served by one tile shape: the small problem's few large tiles add a nearly empty
 // round.  The planner therefore gives every problem the shape that is cheapest for it alone, launches
 // one kernel per shape, and falls back to a single shape when that is cheaper.
-constexpr int NCFG = 4;
-constexpr int kBM[NCFG] = {256, 128, 128, 256};
-constexpr int kBN[NCFG] = {192, 256, 128, 256};
+constexpr int NCFG = 5;
+constexpr int kBM[NCFG] = {256, 128, 128, 256, 128};
+constexpr int kBN[NCFG] = {192, 256, 128, 256, 192};
 // measured on MI355X: microseconds per 64-wide slab and per epilogue of one tile
-constexpr double kSlabUs[NCFG] = {1.21, 0.72, 0.44, 1.40};
-constexpr double kEpiUs[NCFG] = {13.0, 12.4, 8.0, 16.0};  // epilogue plus the pipeline fill of a tile
+constexpr double kSlabUs[NCFG] = {1.21, 0.72, 0.44, 1.40, 0.68};
+constexpr double kEpiUs[NCFG] = {13.0, 12.4, 8.0, 16.0, 7.1};  // epilogue plus the pipeline fill of a tile
 constexpr double kLaunchUs = 3.0;
 constexpr int kSlots = 256;
 
@@ -705,6 +706,7 @@ int launch_cfg(int cfg, const hdit_gemm_problem* problems, int count, hipStream_
   switch (cfg) {
     case 0: return build_and_launch<Cfg256x192>(problems, count, s);
     case 1: return build_and_launch<Cfg128x256>(problems, count, s);
+    case 4: return build_and_launch<Cfg128x192>(problems, count, s);
     case 3: return build_and_launch<Cfg256x256>(problems, count, s);
     default: return build_and_launch<Cfg128x128>(problems, count, s);
   }

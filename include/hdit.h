@@ -82,7 +82,7 @@ int hdit_gemm_bf16(const hdit_gemm_problem* problems, int count, void* stream);
 
 /* Test hook without a counterpart in the reference: pins the tile shape of
  * every later hdit_gemm_bf16 call of the process (0: 256x192, 1: 128x256,
- * 2: 128x128, 3: 256x256; -1: back to the planner). */
+ * 2: 128x128, 3: 256x256, 4: 128x192; -1: back to the planner). */
 void hdit_gemm_force_config(int cfg);
 
 /* ------------------------------------------------------------------------
