@@ -21,7 +21,7 @@ def rnd(*shape, scale=1.0, seed=None):
     return bf16_round(torch.randn(*shape, generator=gen) * scale)
 
 
-@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 64), (300, 384, 128), (666, 1536, 1536), (1, 128, 64), (1024, 512, 256)])
 def test_gemm_bias(hdit, m, n, k, cfg):
     print(f"gemm_bias m={m} n={n} k={k} cfg={cfg}", flush=True)
