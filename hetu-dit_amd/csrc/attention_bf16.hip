@@ -92,16 +92,30 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
   // Workgroups go to the 8 XCDs round-robin by id, and each XCD has its own L2: all query tiles of one
-  // (batch, head) run on one XCD, so that its K and V are fetched into one L2 instead of eight.
-  int qt = blockIdx.x % q_tiles;
-  int bh = blockIdx.x / q_tiles;
-  if ((gridDim.x / q_tiles) % 8 == 0) {
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    qt = slot % q_tiles;
-    bh = (slot / q_tiles) * 8 + xcd;
+  // (batch, head) run on one XCD, so that its K and V are fetched into one L2 instead of eight.  Within that,
+  // the partly filled last query tiles (some of their waves have no rows and skip the arithmetic) come after
+  // all full ones: workgroups are placed in id order, one per CU first, so when a launch has a few more
+  // workgroups than CUs it is the light ones that share a CU with a full one.
+  const int nbh = gridDim.x / q_tiles;
+  const bool by_xcd = nbh % 8 == 0;
+  const int slot = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int nbh_loc = by_xcd ? nbh / 8 : nbh;
+  int qt = slot % q_tiles, bhl = slot / q_tiles;
+  if (q_tiles > 1 && P.sq % BQ != 0) {
+    const int heavy = nbh_loc * (q_tiles - 1);
+    if (slot < heavy) {
+      qt = slot % (q_tiles - 1);
+      bhl = slot / (q_tiles - 1);
+    } else {
+      qt = q_tiles - 1;
+      bhl = slot - heavy;
+    }
   }
+  const int bh = by_xcd ? bhl * 8 + (int)(blockIdx.x & 7) : bhl;
   const int b = bh / P.heads, h = bh % P.heads;
   const int q0 = qt * BQ + wave * WQ;
+  // a wave past the last query row still stages K/V tiles and meets the barriers, but does no arithmetic
+  const bool active = __builtin_amdgcn_readfirstlane(q0 < P.sq);
 
   // ---- Q fragments: lane holds q row (qb*32 + l32), d = 16*ks + 8*lh .. +7
   bf16x8 qf[2][L::Q_IN_LDS ? 1 : KS];
@@ -376,6 +390,15 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   __syncthreads();
   if (NT > 1) load_tile(1);
 
+  if (!active) {
+    // no query rows: stage this wave's share of every K/V tile and meet the same barriers, nothing else
+    for (int t = 0; t < NT - 1; t++) {
+      store_tile((t + 1) & 1);
+      __syncthreads();
+      if (t + 2 < NT) load_tile(t + 2);
+    }
+    return;
+  }
   for (int t = 0; t < NT - 1; t++) {
     tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
     store_tile((t + 1) & 1);
