@@ -25,8 +25,8 @@ PEAK_FP8_TFLOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes summarised in
 # profiles/sd3_1024_step_hbm_traffic.txt (hardware counters cannot be read from inside this process)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 351.2e6
-ATTN_TRAFFIC_BYTES_PER_LAUNCH = 516.7e6
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 344.7e6
+ATTN_TRAFFIC_BYTES_PER_LAUNCH = 189.6e6
 
 
 def build_stack(cfg, device, seed=0):
