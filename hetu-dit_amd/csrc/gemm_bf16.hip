@@ -538,9 +538,11 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     else if (pr.epilogue == HDIT_EPI_BIAS_GELU) epilogue(std::integral_constant<int, HDIT_EPI_BIAS_GELU>{});
     else epilogue(std::integral_constant<int, HDIT_EPI_GATE_RESIDUAL>{});
 
-    // Direct-to-LDS shapes: the compiler does not see the requests in flight, so a wait it placed inside the
-    // main loop for a load of the epilogue would drain them; leave nothing of the epilogue in flight.
-    if constexpr (C::DMA) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    // Leave nothing of the epilogue in flight.  The compiler's bookkeeping of pending loads is path-insensitive:
+    // one epilogue load it believes may still be pending makes it place a small vmcnt wait where the main loop
+    // first reuses that register, and that wait drains the operand stream on every slab (the direct-to-LDS
+    // requests are invisible to it, and the register-staged loads of the slab after next are younger).
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     lid += wgs_per_xcd;
     if (lid >= xcd_end) break;
   }
