@@ -253,29 +253,36 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
           for (int qb = 0; qb < 2; qb++)
             sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qk[qb], ks == 0 ? zero16 : sacc[kb][qb], 0, 0, 0);
       }
-    } else
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-      for (int ks = 0; ks < KS; ks++) {
-        bf16x8 kf = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + ks * 32);
-#pragma unroll
-        for (int qb = 0; qb < 2; qb++)
-          sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], ks == 0 ? (FOLD ? negm[qb] : zero16) : sacc[kb][qb], 0, 0, 0);
-      }
     }
-    if (MASK) {
+    auto mask_scores = [&]() {
+      if (MASK) {
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++)
+        for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          int key = kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-          if (key >= valid) {
-            sacc[kb][0][v] = -INFINITY;
-            sacc[kb][1][v] = -INFINITY;
+          for (int v = 0; v < 16; v++) {
+            int key = kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (key >= valid) {
+              sacc[kb][0][v] = -INFINITY;
+              sacc[kb][1][v] = -INFINITY;
+            }
           }
+      }
+    };
+    auto scores_from_registers = [&]() {
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          bf16x8 kf = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + ks * 32);
+#pragma unroll
+          for (int qb = 0; qb < 2; qb++)
+            sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][L::Q_IN_LDS ? 0 : ks], ks == 0 ? (FOLD ? negm[qb] : zero16) : sacc[kb][qb], 0, 0, 0);
         }
-    }
+      }
+      mask_scores();
+    };
+    if constexpr (L::Q_IN_LDS) mask_scores();
+    else scores_from_registers();
 
     // ---- online softmax in the log2 domain.  A lane owns one query column per qb and 32 of its 64 keys;
     // the other 32 live in lane^32.
