@@ -5,31 +5,35 @@
 // (32*TM) x (32*TN) sub-tile in accumulators (v_mfma_f32_32x32x16_bf16).
 //
 // Staging.  Both operands are k-contiguous, so A and B tiles are staged the
-// same way, in slabs of 64 k (128 bytes per row).  A wave-wide global load
-// fetches 8 rows x 128 bytes, eight lanes per row: every request covers whole
-// 128-byte cache lines (64-byte row pieces were measured at half the L2->CU
-// rate, 29 B/clk/CU against 58).  The data waits in registers for one slab time
-// and is then written to LDS with ds_write_b128 into rows of 128 bytes whose
-// 16-byte chunks are XOR-swizzled with (row>>1)&7: the 16 lanes of a
-// ds_read_b128 pass (16 rows, one chunk) and of a ds_write_b128 pass (2 rows,
-// 8 chunks) then land on 16 distinct 16-byte slots of the 256-byte bank window.
+// same way, in slabs of 64 k (128 bytes per row).  A wave-wide request fetches
+// 8 rows x 128 bytes, eight lanes per row: every request covers whole 128-byte
+// cache lines (64-byte row pieces were measured at half the L2->CU rate,
+// 29 B/clk/CU against 58).  LDS rows are 128 bytes whose 16-byte chunks are
+// XOR-swizzled with (row>>1)&7: the 16 lanes of a ds_read_b128 pass (16 rows,
+// one chunk) land on 16 distinct 16-byte slots of the 256-byte bank window.
 //
-// Pipeline.  The k slabs of all tiles of a workgroup form one flat stream over
-// two LDS stages.  While slab h is multiplied out of stage h&1, the registers
-// holding slab h+1 are written to the other stage and immediately refilled
-// with the global loads of slab h+2, one write+load pair every few MFMAs (the
-// loads have a whole slab time to arrive).  Fragments are double-buffered in
-// registers one k-step ahead; the workgroup barrier sits before the last
-// k-step of a slab, whose fragments are already in registers, so that the
-// first fragments of slab h+1 are read under that k-step's MFMAs.  Tile
-// boundaries are invisible to the stream, so a tile's first slabs arrive
-// during the previous tile's last slab and epilogue.
+// Pipeline.  The k slabs of all tiles of a workgroup form one flat stream; tile
+// boundaries are invisible to it, so a tile's first slabs arrive during the
+// previous tile's last slab and epilogue.  Fragments are double-buffered in
+// registers one k-step ahead; the workgroup barrier sits before the last k-step
+// of a slab, whose fragments are already in registers, so that the first
+// fragments of the next slab are read under that k-step's MFMAs.
+//  * 256-row shapes: direct to LDS (global_load_lds_dwordx4, swizzle applied on
+//    the source side), three A slots and two B slots.  During slab g the A rows
+//    of slab g+2 are requested (k-steps 0..2) into the slot slab g-1 vacated;
+//    behind the barrier that ends slab g, the B rows of slab g+2 go into the B
+//    slot just vacated.  Requests retire in order, so the wait in front of the
+//    barrier leaves exactly the newest A requests in flight.
+//  * 128-row shapes: two LDS stages, register-staged.  While slab h is
+//    multiplied out of stage h&1, the registers holding slab h+1 are written
+//    to the other stage and immediately refilled with the global loads of slab
+//    h+2, one write+load pair every few MFMAs.
 //
 // Epilogue.  A lane's accumulator holds one output row m and runs of 4
 // consecutive n; lanes l and l^32 swap halves (v_permlane32_swap) to own 8
 // consecutive n.  bias / GELU-tanh are applied there, the bf16 result is staged
-// through a wave-private 8 KiB window inside the LDS stage the last slab just
-// vacated and written back with 16 lanes covering 256 contiguous bytes of a row
+// through a wave-private 8 KiB window inside the LDS stage (the A slot) the last
+// slab just vacated and written back with 16 lanes covering 256 contiguous bytes of a row
 // (gate and residual are applied in that coalesced layout, in fp32).
 //
 // One launch covers up to HDIT_GEMM_MAX_PROBLEMS problems.  Tiles are dealt to
