@@ -54,7 +54,7 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
       int c = lane + i * 64;
-      if (c < nchunks) raw[buf][i] = __builtin_nontemporal_load((const i32x4*)(xr + c * 8));
+      if (c < nchunks) raw[buf][i] = *(const i32x4*)(xr + c * 8);
     }
   };
   load(0, row0);
@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
             o[e + 4] += s1[e];
           }
         }
-        __builtin_nontemporal_store(pack8(o), (i32x4*)(yr + c * 8));
+        *(i32x4*)(yr + c * 8) = pack8(o);
       }
     }
   }
