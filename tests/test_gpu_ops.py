@@ -358,3 +358,71 @@ def test_gemm_more_problems_than_one_call_takes(hdit):
     torch.cuda.synchronize()
     for x, w, o in zip(xs, ws, outs):
         assert_parity(o, O.linear(x, w), what="one of 20 problems")
+
+
+def test_gemm_random_shapes_and_epilogues(hdit):
+    """Seeded sweep over ragged m / n, short and long k, every tile shape and epilogue, one to three problems
+    per call."""
+    import random
+
+    rng = random.Random(7)
+    ops = hdit.ops
+    lib = hdit._lib.lib()
+    try:
+        for it in range(40):
+            cfg = rng.choice([-1, 0, 1, 2, 3, 4, 0, 3])
+            k = 64 * rng.randint(1, 7)
+            probs, checks = [], []
+            for j in range(rng.choice([1, 1, 2, 3])):
+                m = rng.choice([1, 7, 130, 255, 257, 600, 1000])
+                n = 8 * rng.randint(1, 90)
+                epi = rng.choice(["bias", "nobias", "gelu", "gate"])
+                a, w, b = rnd(m, k, seed=100 * it + j), rnd(n, k, scale=0.05, seed=100 * it + j + 10), rnd(n, seed=100 * it + j + 20)
+                lin = O.linear(a, w, None if epi == "nobias" else b)
+                if epi == "gate":
+                    r = rnd(m, n, seed=100 * it + j + 30)
+                    gate = torch.randn(2, n, generator=torch.Generator().manual_seed(100 * it + j + 40))
+                    rows = (m + 1) // 2
+                    out = g(r).clone()
+                    probs.append(ops.gemm_problem(g(a), g(w), out, g(b), ops.EPI_GATE_RESIDUAL, resid=out, gate=gate.to(DEV),
+                                                  rows_per_batch=rows))
+                    want = r + gate.repeat_interleave(rows, dim=0)[:m] * lin
+                else:
+                    out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+                    probs.append(ops.gemm_problem(g(a), g(w), out, None if epi == "nobias" else g(b),
+                                                  ops.EPI_BIAS_GELU if epi == "gelu" else ops.EPI_BIAS))
+                    want = O.gelu_tanh(lin) if epi == "gelu" else lin
+                checks.append((out, want, f"case {it} cfg {cfg} m={m} n={n} k={k} {epi}"))
+            print(f"gemm random case {it}: cfg={cfg} k={k} problems={len(probs)}", flush=True)
+            lib.hdit_gemm_force_config(cfg)
+            ops.gemm_launch(probs)
+            torch.cuda.synchronize()
+            for out, want, what in checks:
+                assert_parity(out, want, what=what)
+    finally:
+        lib.hdit_gemm_force_config(-1)
+
+
+def test_attention_random_shapes(hdit):
+    """Seeded sweep over head sizes, batch x heads that are and are not a multiple of 8 (the two workgroup
+    mappings), partly filled last query tiles, ragged key counts and K/V split into two segments."""
+    import random
+
+    rng = random.Random(11)
+    for it in range(30):
+        hd = rng.choice([64, 128])
+        B, H = rng.choice([1, 2]), rng.choice([1, 3, 4, 8])
+        sq = rng.choice([1, 31, 64, 77, 200, 256, 257, 300, 511, 600])
+        skv = rng.choice([1, 5, 64, 65, 130, 333, 512, 777])
+        print(f"attention random case {it}: hd={hd} B={B} H={H} sq={sq} skv={skv}", flush=True)
+        q, k, v = rnd(B, sq, H, hd, seed=3 * it), rnd(B, skv, H, hd, seed=3 * it + 1), rnd(B, skv, H, hd, seed=3 * it + 2)
+        kd, vd = g(k), g(v)
+        if rng.random() < 0.5 and skv > 1:
+            c = rng.randint(1, skv - 1)
+            ks, vs = [kd[:, :c], kd[:, c:]], [vd[:, :c], vd[:, c:]]
+        else:
+            ks, vs = [kd], [vd]
+        (o,) = hdit.ops.attention([g(q)], ks, vs)
+        torch.cuda.synchronize()
+        want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
+        assert_parity(o, want, what=f"attention random case {it}")
