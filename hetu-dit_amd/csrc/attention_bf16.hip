@@ -55,8 +55,14 @@ struct Lds {
   // Row strides chosen for the 64-bank (256-byte) LDS window: a ds_read_b128 pass covers 16 consecutive K
   // rows, which must land on 16 distinct 16-byte slots (stride = 16 mod 256 works); a transpose-read pass
   // covers 4 consecutive V rows x 64 bytes, which must land on 4 distinct 64-byte slots (stride = 64 mod 256).
-  static constexpr int K_ROW = HD * 2 + 16;
-  static constexpr int V_ROW = HD * 2 + 64;
+  // d = 64: K and V tiles come straight from global memory (global_load_lds_dwordx4: no staging registers, no
+  // ds_write), which lands a wave's 64 x 16 bytes contiguously -- eight unpadded 128-byte rows.  The bank spread
+  // then comes from XOR swizzles applied on the source side: slot p of K row r holds chunk p ^ ((r>>1)&7) (16
+  // rows of a fragment read pass on 16 distinct slots), slot p of V row r holds chunk p ^ 4*((r>>1)&1) (the four
+  // rows of a transpose-read pass on four distinct 64-byte slots).
+  static constexpr bool KV_DMA = HD == 64;
+  static constexpr int K_ROW = KV_DMA ? HD * 2 : HD * 2 + 16;
+  static constexpr int V_ROW = KV_DMA ? HD * 2 : HD * 2 + 64;
   static constexpr int K_BYTES = BKV * K_ROW;
   static constexpr int V_BYTES = BKV * V_ROW;
   static constexpr int STAGE = K_BYTES + V_BYTES;
@@ -70,6 +76,24 @@ struct Lds {
   static constexpr int TOTAL = 2 * STAGE + (Q_IN_LDS ? 4 * Q_WAVE_BYTES : 0);
   static_assert(TOTAL <= 160 * 1024, "attention tiles do not fit the LDS");
 };
+
+// One wave-wide direct-to-LDS copy: lane l's 16 bytes land at LDS byte address lds_addr + 16*l.  Inline
+// assembly, so the compiler's wait-count bookkeeping does not see it; the tile loop waits for it explicitly.
+__device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr_uniform), "v"(voff), "s"(base_uniform)
+               : "m0", "memory");
+}
+__device__ __forceinline__ void lds_dma16_ptr(const unsigned char* ptr_per_lane, unsigned lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_addr_uniform), "v"(ptr_per_lane)
+               : "m0", "memory");
+}
+__device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
+  return (unsigned)(uintptr_t)((const __attribute__((address_space(3))) unsigned char*)p);
+}
 
 // The running row maximum is only raised when some row's maximum grew by more than this many powers of
 // two; until then exp2(s - m) may reach 2^8, harmless for the bf16 P operand and the fp32 row sums, and the
@@ -154,15 +178,23 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   // ---- K/V tile staging: global -> registers -> LDS.  A tile that lies inside one segment is addressed as
   // (wave-uniform base) + (loop-invariant per-thread offset); the tile that straddles the segment boundary
   // and the last, clamped tile take the per-row path.
-  i32x4 kreg[NCH], vreg[NCH];
+  i32x4 kreg[L::KV_DMA ? 1 : NCH], vreg[L::KV_DMA ? 1 : NCH];
   unsigned koff[2][NCH], voff[2][NCH];
+  // direct-to-LDS (d = 64): request i of a wave covers rows 8*(wave + 4*i) .. +7, lane -> (row, slot lane%8);
+  // the chunk fetched for a slot is the slot index XORed with the row's swizzle (the same for every i)
+  const int dma_row = wave * 8 + (lane >> 3);
+  const int dma_kc = (lane & 7) ^ ((dma_row >> 1) & 7);
+  const int dma_vc = (lane & 7) ^ (4 * ((dma_row >> 1) & 1));
+  const unsigned lds_base_addr = __builtin_amdgcn_readfirstlane(lds_address(lds));
 #pragma unroll
   for (int i = 0; i < NCH; i++) {
-    const int c = tid + i * 256, row = c / CPR, cc = c % CPR;
-    koff[0][i] = (unsigned)((row * P.k.ss0 + cc * 8) * 2);
-    koff[1][i] = (unsigned)((row * P.k.ss1 + cc * 8) * 2);
-    voff[0][i] = (unsigned)((row * P.v.ss0 + cc * 8) * 2);
-    voff[1][i] = (unsigned)((row * P.v.ss1 + cc * 8) * 2);
+    const int c = tid + i * 256;
+    const int row = L::KV_DMA ? dma_row + 32 * i : c / CPR;
+    const int kc = L::KV_DMA ? dma_kc : c % CPR, vc = L::KV_DMA ? dma_vc : c % CPR;
+    koff[0][i] = (unsigned)((row * P.k.ss0 + kc * 8) * 2);
+    koff[1][i] = (unsigned)((row * P.k.ss1 + kc * 8) * 2);
+    voff[0][i] = (unsigned)((row * P.v.ss0 + vc * 8) * 2);
+    voff[1][i] = (unsigned)((row * P.v.ss1 + vc * 8) * 2);
   }
   const unsigned char* kb0 = (const unsigned char*)(P.k.p0 + b * P.k.sb0 + h * P.k.sh0);
   const unsigned char* kb1 = (const unsigned char*)(P.k.p1 + b * P.k.sb1 + h * P.k.sh1);
@@ -197,6 +229,36 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
       }
     }
   };
+  // the same tile straight into LDS stage `stage`
+  auto dma_tile = [&](int t, int stage) {
+    const int r0 = t * BKV;
+    const unsigned kdst = lds_base_addr + stage * L::STAGE + __builtin_amdgcn_readfirstlane(wave) * 1024;
+    const unsigned vdst = kdst + L::K_BYTES;
+    if (r0 + BKV <= len0) {
+      const unsigned char* kb = kb0 + (int64_t)r0 * P.k.ss0 * 2;
+      const unsigned char* vb = vb0 + (int64_t)r0 * P.v.ss0 * 2;
+#pragma unroll
+      for (int i = 0; i < NCH; i++) {
+        lds_dma16(kb, koff[0][i], kdst + i * 4096);
+        lds_dma16(vb, voff[0][i], vdst + i * 4096);
+      }
+    } else if (r0 >= len0 && r0 + BKV <= P.skv) {
+      const unsigned char* kb = kb1 + (int64_t)(r0 - len0) * P.k.ss1 * 2;
+      const unsigned char* vb = vb1 + (int64_t)(r0 - len0) * P.v.ss1 * 2;
+#pragma unroll
+      for (int i = 0; i < NCH; i++) {
+        lds_dma16(kb, koff[1][i], kdst + i * 4096);
+        lds_dma16(vb, voff[1][i], vdst + i * 4096);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NCH; i++) {
+        const int r = min(r0 + dma_row + 32 * i, P.skv - 1);
+        lds_dma16_ptr((const unsigned char*)(row_ptr(P.k, b, h, r) + dma_kc * 8), kdst + i * 4096);
+        lds_dma16_ptr((const unsigned char*)(row_ptr(P.v, b, h, r) + dma_vc * 8), vdst + i * 4096);
+      }
+    }
+  };
   auto store_tile = [&](int stage) {
     unsigned char* base = lds + stage * L::STAGE;
 #pragma unroll
@@ -228,8 +290,11 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
 
   // lane-constant part of the V^T transpose-read address:
   // 16-lane group G = lane/16, x = lane%16: key row 4*(G/2) + x/4, column 16*(G%2) + 4*(x%4)
-  const int vt_off = (4 * (lane >> 5) + ((lane & 15) >> 2)) * L::V_ROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-  const int k_off = l32 * L::K_ROW + lh * 16;
+  const int vt_row = 4 * (lane >> 5) + ((lane & 15) >> 2);
+  const int vt_off = vt_row * L::V_ROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  const int vt_swz = L::KV_DMA ? ((vt_row >> 1) & 1) : 0;  // 64-byte half of a V row is XORed with this
+  const int k_off = L::KV_DMA ? l32 * L::K_ROW : l32 * L::K_ROW + lh * 16;
+  const int k_swz = (l32 >> 1) & 7;  // direct-to-LDS layout: chunk c of K row r sits in slot c ^ ((r>>1)&7)
   const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
   // one K/V tile: scores, online softmax, PV.  MASK: keys >= valid do not exist (last tile only).
@@ -273,7 +338,8 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
       for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-          bf16x8 kf = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + ks * 32);
+          bf16x8 kf = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW +
+                                       (L::KV_DMA ? (((ks * 2 + lh) ^ k_swz) << 4) : ks * 32));
 #pragma unroll
           for (int qb = 0; qb < 2; qb++)
             sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][L::Q_IN_LDS ? 0 : ks], ks == 0 ? (FOLD ? negm[qb] : zero16) : sacc[kb][qb], 0, 0, 0);
@@ -377,7 +443,7 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     for (int u = 0; u < 4; u++) {
 #pragma unroll
       for (int db = 0; db < DB; db++) {
-        const unsigned char* va = sv + vt_off + (u * 16) * L::V_ROW + db * 64;
+        const unsigned char* va = sv + vt_off + (u * 16) * L::V_ROW + ((db ^ vt_swz) << 6);
         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(va));
         s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (s16x4 __attribute__((address_space(3)))*)(va + 8 * L::V_ROW));
@@ -392,25 +458,41 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   };
 
   const int NT = (P.skv + BKV - 1) / BKV;
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-  if (NT > 1) load_tile(1);
-
-  if (!active) {
-    // no query rows: stage this wave's share of every K/V tile and meet the same barriers, nothing else
-    for (int t = 0; t < NT - 1; t++) {
+  // Tile t+1 is fetched while tile t is worked on.  Register path: its loads are issued behind the barrier
+  // that published tile t and written to LDS after tile t's arithmetic.  Direct path: its requests are issued at
+  // the same point into the stage tile t-1 vacated; every wave waits for its own requests before the barrier.
+  if constexpr (L::KV_DMA) {
+    dma_tile(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    __syncthreads();
+    if (NT > 1) dma_tile(1, 1);
+  } else {
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+    if (NT > 1) load_tile(1);
+  }
+  auto next_tile = [&](int t) {  // end of iteration t: publish tile t+1, start fetching tile t+2
+    if constexpr (L::KV_DMA) {
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile t+1 has landed
+      __syncthreads();
+      if (t + 2 < NT) dma_tile(t + 2, t & 1);
+    } else {
       store_tile((t + 1) & 1);
       __syncthreads();
       if (t + 2 < NT) load_tile(t + 2);
     }
+  };
+
+  if (!active) {
+    // no query rows: stage this wave's share of every K/V tile and meet the same barriers, nothing else
+    for (int t = 0; t < NT - 1; t++) next_tile(t);
+    if constexpr (L::KV_DMA) __builtin_amdgcn_s_waitcnt(0x0f70);
     return;
   }
   for (int t = 0; t < NT - 1; t++) {
     tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
-    store_tile((t + 1) & 1);
-    __syncthreads();
-    if (t + 2 < NT) load_tile(t + 2);
+    next_tile(t);
   }
   {
     const int t = NT - 1;
