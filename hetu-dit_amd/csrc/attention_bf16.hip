@@ -55,12 +55,13 @@ struct Lds {
   // Row strides chosen for the 64-bank (256-byte) LDS window: a ds_read_b128 pass covers 16 consecutive K
   // rows, which must land on 16 distinct 16-byte slots (stride = 16 mod 256 works); a transpose-read pass
   // covers 4 consecutive V rows x 64 bytes, which must land on 4 distinct 64-byte slots (stride = 64 mod 256).
-  // d = 64: K and V tiles come straight from global memory (global_load_lds_dwordx4: no staging registers, no
-  // ds_write), which lands a wave's 64 x 16 bytes contiguously -- eight unpadded 128-byte rows.  The bank spread
-  // then comes from XOR swizzles applied on the source side: slot p of K row r holds chunk p ^ ((r>>1)&7) (16
-  // rows of a fragment read pass on 16 distinct slots), slot p of V row r holds chunk p ^ 4*((r>>1)&1) (the four
-  // rows of a transpose-read pass on four distinct 64-byte slots).
-  static constexpr bool KV_DMA = HD == 64;
+  // K and V tiles come straight from global memory (global_load_lds_dwordx4: no staging registers, no
+  // ds_write), which lands a wave's 64 x 16 bytes contiguously -- eight (d = 64) or four (d = 128) unpadded
+  // rows.  The bank spread then comes from XOR swizzles applied on the source side.  d = 64: slot p of K row r
+  // holds chunk p ^ ((r>>1)&7) (16 rows of a fragment read pass on 16 distinct slots), slot p of V row r holds
+  // chunk p ^ 4*((r>>1)&1) (the four rows of a transpose-read pass on four distinct 64-byte slots).  d = 128
+  // (rows of 256 bytes, a whole bank window): K chunk p ^ (r&15), V chunk p ^ 4*(r&3).
+  static constexpr bool KV_DMA = true;
   static constexpr int K_ROW = KV_DMA ? HD * 2 : HD * 2 + 16;
   static constexpr int V_ROW = KV_DMA ? HD * 2 : HD * 2 + 64;
   static constexpr int K_BYTES = BKV * K_ROW;
@@ -70,7 +71,7 @@ struct Lds {
   // the K rows, and are read per k-step next to the K fragments: the registers they would occupy are what the
   // loop otherwise spills (and reloads from scratch on every tile, with one wave per SIMD to hide nothing).
   static constexpr bool Q_IN_LDS = HD == 128;
-  static constexpr int Q_ROW = K_ROW;
+  static constexpr int Q_ROW = HD * 2 + 16;
   static constexpr int Q_OFF = 2 * STAGE;
   static constexpr int Q_WAVE_BYTES = WQ * Q_ROW;
   static constexpr int TOTAL = 2 * STAGE + (Q_IN_LDS ? 4 * Q_WAVE_BYTES : 0);
@@ -182,14 +183,15 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   unsigned koff[2][NCH], voff[2][NCH];
   // direct-to-LDS (d = 64): request i of a wave covers rows 8*(wave + 4*i) .. +7, lane -> (row, slot lane%8);
   // the chunk fetched for a slot is the slot index XORed with the row's swizzle (the same for every i)
-  const int dma_row = wave * 8 + (lane >> 3);
-  const int dma_kc = (lane & 7) ^ ((dma_row >> 1) & 7);
-  const int dma_vc = (lane & 7) ^ (4 * ((dma_row >> 1) & 1));
+  constexpr int RPI = 64 / CPR;  // rows per request
+  const int dma_row = wave * RPI + lane / CPR;
+  const int dma_kc = (lane % CPR) ^ (HD == 64 ? ((dma_row >> 1) & 7) : (dma_row & 15));
+  const int dma_vc = (lane % CPR) ^ (4 * (HD == 64 ? ((dma_row >> 1) & 1) : (dma_row & 3)));
   const unsigned lds_base_addr = __builtin_amdgcn_readfirstlane(lds_address(lds));
 #pragma unroll
   for (int i = 0; i < NCH; i++) {
     const int c = tid + i * 256;
-    const int row = L::KV_DMA ? dma_row + 32 * i : c / CPR;
+    const int row = L::KV_DMA ? dma_row + 4 * RPI * i : c / CPR;
     const int kc = L::KV_DMA ? dma_kc : c % CPR, vc = L::KV_DMA ? dma_vc : c % CPR;
     koff[0][i] = (unsigned)((row * P.k.ss0 + kc * 8) * 2);
     koff[1][i] = (unsigned)((row * P.k.ss1 + kc * 8) * 2);
@@ -253,7 +255,7 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     } else {
 #pragma unroll
       for (int i = 0; i < NCH; i++) {
-        const int r = min(r0 + dma_row + 32 * i, P.skv - 1);
+        const int r = min(r0 + dma_row + 4 * RPI * i, P.skv - 1);
         lds_dma16_ptr((const unsigned char*)(row_ptr(P.k, b, h, r) + dma_kc * 8), kdst + i * 4096);
         lds_dma16_ptr((const unsigned char*)(row_ptr(P.v, b, h, r) + dma_vc * 8), vdst + i * 4096);
       }
@@ -292,9 +294,9 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   // 16-lane group G = lane/16, x = lane%16: key row 4*(G/2) + x/4, column 16*(G%2) + 4*(x%4)
   const int vt_row = 4 * (lane >> 5) + ((lane & 15) >> 2);
   const int vt_off = vt_row * L::V_ROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-  const int vt_swz = L::KV_DMA ? ((vt_row >> 1) & 1) : 0;  // 64-byte half of a V row is XORed with this
+  const int vt_swz = !L::KV_DMA ? 0 : HD == 64 ? ((vt_row >> 1) & 1) : (vt_row & 3);  // XORed into the 64-byte piece index
   const int k_off = L::KV_DMA ? l32 * L::K_ROW : l32 * L::K_ROW + lh * 16;
-  const int k_swz = (l32 >> 1) & 7;  // direct-to-LDS layout: chunk c of K row r sits in slot c ^ ((r>>1)&7)
+  const int k_swz = HD == 64 ? ((l32 >> 1) & 7) : (l32 & 15);  // direct-to-LDS layout: chunk c of K row r sits in slot c ^ this
   const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
   // one K/V tile: scores, online softmax, PV.  MASK: keys >= valid do not exist (last tile only).
@@ -311,7 +313,8 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) qk[qb] = *(const bf16x8*)(qlds + (qb * 32 + l32) * L::Q_ROW + lh * 16 + ks * 32);
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) kf[kb] = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + ks * 32);
+        for (int kb = 0; kb < 2; kb++)
+          kf[kb] = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + (L::KV_DMA ? (((ks * 2 + lh) ^ k_swz) << 4) : ks * 32));
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
