@@ -2,8 +2,8 @@
 //
 // Work split: one workgroup = 4 waves = 256 query rows of one (batch, head);
 // each wave owns 64 query rows (two 32-row MFMA column blocks) and walks the
-// keys in tiles of 64.  K and V tiles are staged global -> registers -> LDS in
-// two buffers (one barrier per tile).
+// keys in tiles of 64.  K and V tiles go straight from global memory into two
+// LDS buffers (direct-to-LDS loads, one barrier per tile).
 //
 // The scores are produced transposed, S^T = K . Q^T, with K rows as the MFMA
 // "A" operand and the wave's Q rows (held in registers for the whole kernel)
@@ -52,18 +52,16 @@ struct AttnParams {
 
 template <int HD>
 struct Lds {
-  // Row strides chosen for the 64-bank (256-byte) LDS window: a ds_read_b128 pass covers 16 consecutive K
-  // rows, which must land on 16 distinct 16-byte slots (stride = 16 mod 256 works); a transpose-read pass
-  // covers 4 consecutive V rows x 64 bytes, which must land on 4 distinct 64-byte slots (stride = 64 mod 256).
   // K and V tiles come straight from global memory (global_load_lds_dwordx4: no staging registers, no
   // ds_write), which lands a wave's 64 x 16 bytes contiguously -- eight (d = 64) or four (d = 128) unpadded
-  // rows.  The bank spread then comes from XOR swizzles applied on the source side.  d = 64: slot p of K row r
-  // holds chunk p ^ ((r>>1)&7) (16 rows of a fragment read pass on 16 distinct slots), slot p of V row r holds
-  // chunk p ^ 4*((r>>1)&1) (the four rows of a transpose-read pass on four distinct 64-byte slots).  d = 128
-  // (rows of 256 bytes, a whole bank window): K chunk p ^ (r&15), V chunk p ^ 4*(r&3).
-  static constexpr bool KV_DMA = true;
-  static constexpr int K_ROW = KV_DMA ? HD * 2 : HD * 2 + 16;
-  static constexpr int V_ROW = KV_DMA ? HD * 2 : HD * 2 + 64;
+  // rows.  The spread over the 64-bank (256-byte) LDS window therefore comes from XOR swizzles applied on the
+  // source side.  A ds_read_b128 pass covers 16 consecutive K rows, which must land on 16 distinct 16-byte
+  // slots; a transpose-read pass covers 4 consecutive V rows x 64 bytes, which must land on 4 distinct 64-byte
+  // slots.  d = 64 (rows of 128 bytes): slot p of K row r holds chunk p ^ ((r>>1)&7), slot p of V row r holds
+  // chunk p ^ 4*((r>>1)&1).  d = 128 (rows of 256 bytes, a whole bank window): K chunk p ^ (r&15), V chunk
+  // p ^ 4*(r&3).
+  static constexpr int K_ROW = HD * 2;
+  static constexpr int V_ROW = HD * 2;
   static constexpr int K_BYTES = BKV * K_ROW;
   static constexpr int V_BYTES = BKV * V_ROW;
   static constexpr int STAGE = K_BYTES + V_BYTES;
@@ -179,7 +177,6 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   // ---- K/V tile staging: global -> registers -> LDS.  A tile that lies inside one segment is addressed as
   // (wave-uniform base) + (loop-invariant per-thread offset); the tile that straddles the segment boundary
   // and the last, clamped tile take the per-row path.
-  i32x4 kreg[L::KV_DMA ? 1 : NCH], vreg[L::KV_DMA ? 1 : NCH];
   unsigned koff[2][NCH], voff[2][NCH];
   // direct-to-LDS (d = 64): request i of a wave covers rows 8*(wave + 4*i) .. +7, lane -> (row, slot lane%8);
   // the chunk fetched for a slot is the slot index XORed with the row's swizzle (the same for every i)
@@ -190,48 +187,18 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   const unsigned lds_base_addr = __builtin_amdgcn_readfirstlane(lds_address(lds));
 #pragma unroll
   for (int i = 0; i < NCH; i++) {
-    const int c = tid + i * 256;
-    const int row = L::KV_DMA ? dma_row + 4 * RPI * i : c / CPR;
-    const int kc = L::KV_DMA ? dma_kc : c % CPR, vc = L::KV_DMA ? dma_vc : c % CPR;
-    koff[0][i] = (unsigned)((row * P.k.ss0 + kc * 8) * 2);
-    koff[1][i] = (unsigned)((row * P.k.ss1 + kc * 8) * 2);
-    voff[0][i] = (unsigned)((row * P.v.ss0 + vc * 8) * 2);
-    voff[1][i] = (unsigned)((row * P.v.ss1 + vc * 8) * 2);
+    const int row = dma_row + 4 * RPI * i;
+    koff[0][i] = (unsigned)((row * P.k.ss0 + dma_kc * 8) * 2);
+    koff[1][i] = (unsigned)((row * P.k.ss1 + dma_kc * 8) * 2);
+    voff[0][i] = (unsigned)((row * P.v.ss0 + dma_vc * 8) * 2);
+    voff[1][i] = (unsigned)((row * P.v.ss1 + dma_vc * 8) * 2);
   }
   const unsigned char* kb0 = (const unsigned char*)(P.k.p0 + b * P.k.sb0 + h * P.k.sh0);
   const unsigned char* kb1 = (const unsigned char*)(P.k.p1 + b * P.k.sb1 + h * P.k.sh1);
   const unsigned char* vb0 = (const unsigned char*)(P.v.p0 + b * P.v.sb0 + h * P.v.sh0);
   const unsigned char* vb1 = (const unsigned char*)(P.v.p1 + b * P.v.sb1 + h * P.v.sh1);
   const int len0 = P.k.len0;
-  auto load_tile = [&](int t) {
-    const int r0 = t * BKV;
-    if (r0 + BKV <= len0) {
-      const unsigned char* kb = kb0 + (int64_t)r0 * P.k.ss0 * 2;
-      const unsigned char* vb = vb0 + (int64_t)r0 * P.v.ss0 * 2;
-#pragma unroll
-      for (int i = 0; i < NCH; i++) {
-        kreg[i] = *(const i32x4*)(kb + koff[0][i]);
-        vreg[i] = *(const i32x4*)(vb + voff[0][i]);
-      }
-    } else if (r0 >= len0 && r0 + BKV <= P.skv) {
-      const unsigned char* kb = kb1 + (int64_t)(r0 - len0) * P.k.ss1 * 2;
-      const unsigned char* vb = vb1 + (int64_t)(r0 - len0) * P.v.ss1 * 2;
-#pragma unroll
-      for (int i = 0; i < NCH; i++) {
-        kreg[i] = *(const i32x4*)(kb + koff[1][i]);
-        vreg[i] = *(const i32x4*)(vb + voff[1][i]);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < NCH; i++) {
-        int c = tid + i * 256, row = c / CPR, cc = c % CPR;
-        int r = min(r0 + row, P.skv - 1);
-        kreg[i] = *(const i32x4*)(row_ptr(P.k, b, h, r) + cc * 8);
-        vreg[i] = *(const i32x4*)(row_ptr(P.v, b, h, r) + cc * 8);
-      }
-    }
-  };
-  // the same tile straight into LDS stage `stage`
+  // tile t straight into LDS stage `stage`
   auto dma_tile = [&](int t, int stage) {
     const int r0 = t * BKV;
     const unsigned kdst = lds_base_addr + stage * L::STAGE + __builtin_amdgcn_readfirstlane(wave) * 1024;
@@ -261,16 +228,6 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
       }
     }
   };
-  auto store_tile = [&](int stage) {
-    unsigned char* base = lds + stage * L::STAGE;
-#pragma unroll
-    for (int i = 0; i < NCH; i++) {
-      int c = tid + i * 256, row = c / CPR, cc = c % CPR;
-      *(i32x4*)(base + row * L::K_ROW + cc * 16) = kreg[i];
-      *(i32x4*)(base + L::K_BYTES + row * L::V_ROW + cc * 16) = vreg[i];
-    }
-  };
-
   f32x16 oacc[DB][2];
 #pragma unroll
   for (int i = 0; i < DB; i++)
@@ -294,8 +251,8 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   // 16-lane group G = lane/16, x = lane%16: key row 4*(G/2) + x/4, column 16*(G%2) + 4*(x%4)
   const int vt_row = 4 * (lane >> 5) + ((lane & 15) >> 2);
   const int vt_off = vt_row * L::V_ROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-  const int vt_swz = !L::KV_DMA ? 0 : HD == 64 ? ((vt_row >> 1) & 1) : (vt_row & 3);  // XORed into the 64-byte piece index
-  const int k_off = L::KV_DMA ? l32 * L::K_ROW : l32 * L::K_ROW + lh * 16;
+  const int vt_swz = HD == 64 ? ((vt_row >> 1) & 1) : (vt_row & 3);  // XORed into the 64-byte piece index
+  const int k_off = l32 * L::K_ROW;
   const int k_swz = HD == 64 ? ((l32 >> 1) & 7) : (l32 & 15);  // direct-to-LDS layout: chunk c of K row r sits in slot c ^ this
   const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
@@ -314,7 +271,7 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
         for (int qb = 0; qb < 2; qb++) qk[qb] = *(const bf16x8*)(qlds + (qb * 32 + l32) * L::Q_ROW + lh * 16 + ks * 32);
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
-          kf[kb] = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + (L::KV_DMA ? (((ks * 2 + lh) ^ k_swz) << 4) : ks * 32));
+          kf[kb] = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW + (((ks * 2 + lh) ^ k_swz) << 4));
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
@@ -342,7 +299,7 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
           bf16x8 kf = *(const bf16x8*)(sk + k_off + kb * 32 * L::K_ROW +
-                                       (L::KV_DMA ? (((ks * 2 + lh) ^ k_swz) << 4) : ks * 32));
+                                       (((ks * 2 + lh) ^ k_swz) << 4));
 #pragma unroll
           for (int qb = 0; qb < 2; qb++)
             sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][L::Q_IN_LDS ? 0 : ks], ks == 0 ? (FOLD ? negm[qb] : zero16) : sacc[kb][qb], 0, 0, 0);
@@ -461,36 +418,22 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
   };
 
   const int NT = (P.skv + BKV - 1) / BKV;
-  // Tile t+1 is fetched while tile t is worked on.  Register path: its loads are issued behind the barrier
-  // that published tile t and written to LDS after tile t's arithmetic.  Direct path: its requests are issued at
-  // the same point into the stage tile t-1 vacated; every wave waits for its own requests before the barrier.
-  if constexpr (L::KV_DMA) {
-    dma_tile(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-    __syncthreads();
-    if (NT > 1) dma_tile(1, 1);
-  } else {
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-    if (NT > 1) load_tile(1);
-  }
+  // Tile t+1 is fetched while tile t is worked on: its requests are issued behind the barrier that published
+  // tile t, into the stage tile t-1 vacated; every wave waits for its own requests before the next barrier.
+  dma_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  if (NT > 1) dma_tile(1, 1);
   auto next_tile = [&](int t) {  // end of iteration t: publish tile t+1, start fetching tile t+2
-    if constexpr (L::KV_DMA) {
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile t+1 has landed
-      __syncthreads();
-      if (t + 2 < NT) dma_tile(t + 2, t & 1);
-    } else {
-      store_tile((t + 1) & 1);
-      __syncthreads();
-      if (t + 2 < NT) load_tile(t + 2);
-    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile t+1 has landed
+    __syncthreads();
+    if (t + 2 < NT) dma_tile(t + 2, t & 1);
   };
 
   if (!active) {
     // no query rows: stage this wave's share of every K/V tile and meet the same barriers, nothing else
     for (int t = 0; t < NT - 1; t++) next_tile(t);
-    if constexpr (L::KV_DMA) __builtin_amdgcn_s_waitcnt(0x0f70);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
     return;
   }
   for (int t = 0; t < NT - 1; t++) {
