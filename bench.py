@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes summarised in
 # profiles/sd3_1024_step_hbm_traffic.txt (hardware counters cannot be read from inside this process)
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 344.7e6
-ATTN_TRAFFIC_BYTES_PER_LAUNCH = 189.6e6
+ATTN_TRAFFIC_BYTES_PER_LAUNCH = 185.6e6
 
 
 def build_stack(cfg, device, seed=0):
