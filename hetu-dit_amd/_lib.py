@@ -12,6 +12,8 @@ LIB_PATH = os.environ.get("HDIT_LIBRARY") or os.path.join(HERE, "libhdit.so")
 
 HDIT_GEMM_MAX_PROBLEMS = 16
 EPI_BIAS, EPI_BIAS_GELU, EPI_GATE_RESIDUAL = 0, 1, 2
+EPI_RESID_F32, EPI_OUT_F32 = 0x10, 0x20
+ABI_VERSION = 2
 
 
 class GemmProblem(C.Structure):
@@ -89,6 +91,8 @@ class LnJob(C.Structure):
         ("mod_stride", C.c_int64),
         ("batch", C.c_int32),
         ("tokens", C.c_int32),
+        ("x_f32", C.c_int32),
+        ("pad_", C.c_int32),
     ]
 
 
@@ -160,6 +164,9 @@ def lib():
                 fn = getattr(handle, name)  # AttributeError if the library lacks a declared symbol
                 fn.restype = res
                 fn.argtypes = args
+            if handle.hdit_abi_version() != ABI_VERSION:
+                raise RuntimeError(f"{LIB_PATH} has ABI version {handle.hdit_abi_version()}, this binding needs "
+                                   f"{ABI_VERSION}: rebuild the library")
             _lib = handle
     return _lib
 

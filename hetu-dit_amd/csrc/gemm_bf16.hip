@@ -431,7 +431,11 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
       const int wr_n = ncol0 + rchunk * 8;
       const int wr_nc = min(wr_n, N - 8);
       const bool wr_ok = rchunk < 4 * TN && wr_n < N;
-      i32x4 rres[8];
+      // The residual stream may be carried in fp32 (HDIT_EPI_RESID_F32 / HDIT_EPI_OUT_F32): a lane's 8 columns
+      // are then 32 bytes, moved as two 16-byte accesses.
+      const bool rf32 = GATED && (pr.epilogue & HDIT_EPI_RESID_F32) != 0;
+      const bool of32 = GATED && (pr.epilogue & HDIT_EPI_OUT_F32) != 0;
+      i32x4 rres[8], rres_hi[GATED ? 8 : 1];
       f32x4 gte0, gte1;
       bool straddle = false;
       auto prefetch_rows = [&](int i, int half) {
@@ -439,7 +443,13 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
 #pragma unroll
         for (int it = half * 4; it < half * 4 + 4; it++) {
           const int mm = min(mrow0 + it * 4 + wr_row, M - 1);
-          rres[it] = *(const i32x4*)(Rb + (unsigned)((mm * ldr + wr_nc) * 2));
+          if (rf32) {
+            const unsigned char* rp = Rb + (unsigned)((mm * ldr + wr_nc) * 4);
+            rres[it] = *(const i32x4*)rp;
+            rres_hi[GATED ? it : 0] = *(const i32x4*)(rp + 16);
+          } else {
+            rres[it] = *(const i32x4*)(Rb + (unsigned)((mm * ldr + wr_nc) * 2));
+          }
         }
       };
       auto prefetch_gate = [&](int i) {
@@ -498,7 +508,7 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
         // coalesced write-back of this 32 x (32*TN) block
 #pragma unroll
         for (int half = 0; half < 2; half++) {
-          i32x4 outv[4];
+          i32x4 outv[4], outv_hi[GATED ? 4 : 1];
 #pragma unroll
           for (int q = 0; q < 4; q++) {
             const int it = half * 4 + q;
@@ -514,13 +524,29 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
               }
               float u[8], rf[8];
               hdit::unpack8(val, u);
-              hdit::unpack8(rres[it], rf);
+              if (rf32) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                  rf[e] = __int_as_float(rres[it][e]);
+                  rf[4 + e] = __int_as_float(rres_hi[GATED ? it : 0][e]);
+                }
+              } else {
+                hdit::unpack8(rres[it], rf);
+              }
 #pragma unroll
               for (int e = 0; e < 4; e++) {
                 u[e] = __builtin_fmaf(g0[e], u[e], rf[e]);
                 u[4 + e] = __builtin_fmaf(g1[e], u[4 + e], rf[4 + e]);
               }
-              val = hdit::pack8(u);
+              if (of32) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                  val[e] = __float_as_int(u[e]);
+                  outv_hi[GATED ? q : 0][e] = __float_as_int(u[4 + e]);
+                }
+              } else {
+                val = hdit::pack8(u);
+              }
             }
             outv[q] = val;
           }
@@ -532,14 +558,22 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
 #pragma unroll
           for (int q = 0; q < 4; q++) {
             const int mm = mrow0 + (half * 4 + q) * 4 + wr_row;
-            if (wr_ok && mm < M) *(i32x4*)(Cb + (unsigned)((mm * ldc + wr_n) * 2)) = outv[q];
+            if (wr_ok && mm < M) {
+              if (of32) {
+                unsigned char* cp = Cb + (unsigned)((mm * ldc + wr_n) * 4);
+                *(i32x4*)cp = outv[q];
+                *(i32x4*)(cp + 16) = outv_hi[GATED ? q : 0];
+              } else {
+                *(i32x4*)(Cb + (unsigned)((mm * ldc + wr_n) * 2)) = outv[q];
+              }
+            }
           }
           SCHED_FENCE();
         }
       }
     };
-    if (pr.epilogue == HDIT_EPI_BIAS) epilogue(std::integral_constant<int, HDIT_EPI_BIAS>{});
-    else if (pr.epilogue == HDIT_EPI_BIAS_GELU) epilogue(std::integral_constant<int, HDIT_EPI_BIAS_GELU>{});
+    if ((pr.epilogue & HDIT_EPI_MODE_MASK) == HDIT_EPI_BIAS) epilogue(std::integral_constant<int, HDIT_EPI_BIAS>{});
+    else if ((pr.epilogue & HDIT_EPI_MODE_MASK) == HDIT_EPI_BIAS_GELU) epilogue(std::integral_constant<int, HDIT_EPI_BIAS_GELU>{});
     else epilogue(std::integral_constant<int, HDIT_EPI_GATE_RESIDUAL>{});
 
     // Leave nothing of the epilogue in flight.  The compiler's bookkeeping of pending loads is path-insensitive:
@@ -736,11 +770,16 @@ extern "C" __attribute__((visibility("default"))) int hdit_gemm_bf16(const hdit_
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uintptr_t)p.c | (uintptr_t)p.bias) & 15) return HDIT_EINVAL;
     // rows are addressed with 32-bit byte offsets from the operand base
     if ((int64_t)p.m * p.lda * 2 >= (1ll << 32) || (int64_t)p.n * p.ldb * 2 >= (1ll << 32)) return HDIT_EUNSUPPORTED;
-    if ((int64_t)p.m * p.ldc * 2 >= (1ll << 31)) return HDIT_EUNSUPPORTED;
-    if (p.epilogue < HDIT_EPI_BIAS || p.epilogue > HDIT_EPI_GATE_RESIDUAL) return HDIT_EINVAL;
-    if (p.epilogue == HDIT_EPI_GATE_RESIDUAL) {
+    const int mode = p.epilogue & HDIT_EPI_MODE_MASK;
+    const int c_bytes = (p.epilogue & HDIT_EPI_OUT_F32) ? 4 : 2, r_bytes = (p.epilogue & HDIT_EPI_RESID_F32) ? 4 : 2;
+    if (p.epilogue & ~(HDIT_EPI_MODE_MASK | HDIT_EPI_RESID_F32 | HDIT_EPI_OUT_F32)) return HDIT_EINVAL;
+    if (mode > HDIT_EPI_GATE_RESIDUAL) return HDIT_EINVAL;
+    // the fp32 residual stream only exists in the gated-residual epilogue
+    if (mode != HDIT_EPI_GATE_RESIDUAL && (p.epilogue & (HDIT_EPI_RESID_F32 | HDIT_EPI_OUT_F32))) return HDIT_EINVAL;
+    if ((int64_t)p.m * p.ldc * c_bytes >= (1ll << 31)) return HDIT_EUNSUPPORTED;
+    if (mode == HDIT_EPI_GATE_RESIDUAL) {
       if (!p.resid || !p.gate || p.rows_per_batch <= 0 || p.ldr % 8) return HDIT_EINVAL;
-      if ((int64_t)p.m * p.ldr * 2 >= (1ll << 31)) return HDIT_EUNSUPPORTED;
+      if ((int64_t)p.m * p.ldr * r_bytes >= (1ll << 31)) return HDIT_EUNSUPPORTED;
       if (((uintptr_t)p.resid & 15) || ((uintptr_t)p.gate & 15) || p.gate_stride % 4) return HDIT_EINVAL;
     }
     live[nlive++] = p;

@@ -19,7 +19,10 @@ struct LnJobs {
   hdit_ln_job j[HDIT_LN_MAX_JOBS];
 };
 
-template <int NCH>  // 16-byte chunks per lane (row has dim/8 chunks, NCH = ceil(dim/512))
+// NCH = 16-byte input chunks per lane.  A chunk is 8 elements of a bf16 row or (XF32: the fp32 residual stream of
+// a block stack) 4 elements of an f32 row; the output is bf16 either way, so a lane stores 16 or 8 bytes per
+// chunk and a wave-wide access is contiguous in both cases.
+template <int NCH, bool XF32>
 __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, const __bf16* __restrict__ lw,
                                                           const __bf16* __restrict__ lb, int dim, float eps) {
   // which job this workgroup belongs to (a launch normalises up to HDIT_LN_MAX_JOBS tensors, e.g. the
@@ -28,7 +31,9 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
 #pragma unroll 1
   while (ji + 1 < jobs.count && (int)blockIdx.x >= jobs.block_start[ji + 1]) ji++;
   const hdit_ln_job& job = jobs.j[ji];
-  const __bf16* __restrict__ x = (const __bf16*)job.x;
+  constexpr int EPC = XF32 ? 4 : 8;  // elements per chunk
+  constexpr int XB = XF32 ? 4 : 2;   // bytes per input element
+  const unsigned char* __restrict__ x = (const unsigned char*)job.x;
   __bf16* __restrict__ y = (__bf16*)job.y;
   const float* __restrict__ shift = job.shift;
   const float* __restrict__ scale = job.scale;
@@ -42,19 +47,45 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
   const int lane = threadIdx.x & 63;
   const int64_t row0 = ((int64_t)(blockIdx.x - jobs.block_start[ji]) * 4 + (threadIdx.x >> 6)) * RPW;
   if (row0 >= rows) return;
-  const int nchunks = dim >> 3;
+  const int nchunks = dim / EPC;
   const float inv_d = 1.0f / (float)dim;
   i32x4 raw[RPW][NCH];
-  auto row_x = [&](int64_t row) {
-    const int64_t b = row / tokens;
-    return x + b * x_sb + (row - b * tokens) * x_st;
-  };
   auto load = [&](int buf, int64_t row) {
-    const __bf16* xr = row_x(row);
+    const int64_t b = row / tokens;
+    const unsigned char* xr = x + (b * x_sb + (row - b * tokens) * x_st) * XB;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
       int c = lane + i * 64;
-      if (c < nchunks) raw[buf][i] = *(const i32x4*)(xr + c * 8);
+      if (c < nchunks) raw[buf][i] = *(const i32x4*)(xr + c * 16);
+    }
+  };
+  auto unpack = [&](const i32x4& r, float (&f)[EPC]) {
+    if constexpr (XF32) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) f[e] = __int_as_float(r[e]);
+    } else {
+      unpack8(r, f);
+    }
+  };
+  // EPC bf16 values (an affine weight or bias) at element offset c * EPC
+  auto load_bf16 = [&](const __bf16* p, int c, float (&w)[EPC]) {
+    if constexpr (XF32) {
+      const i32x2 r = *(const i32x2*)(p + c * 4);
+#pragma unroll
+      for (int e = 0; e < 2; e++) {
+        w[2 * e] = __uint_as_float((uint32_t)r[e] << 16);
+        w[2 * e + 1] = __uint_as_float((uint32_t)r[e] & 0xffff0000u);
+      }
+    } else {
+      unpack8(*(const i32x4*)(p + c * 8), w);
+    }
+  };
+  auto load_f32 = [&](const float* p, int c, float (&w)[EPC]) {
+#pragma unroll
+    for (int h = 0; h < EPC / 4; h++) {
+      const f32x4 v = *(const f32x4*)(p + c * EPC + h * 4);
+#pragma unroll
+      for (int e = 0; e < 4; e++) w[h * 4 + e] = v[e];
     }
   };
   load(0, row0);
@@ -64,14 +95,14 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
     if (row >= rows) break;
     if (r + 1 < RPW && row + 1 < rows) load(r + 1, row + 1);
     float s = 0.f;
-    float f[NCH][8];
+    float f[NCH][EPC];
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
       int c = lane + i * 64;
       if (c < nchunks) {
-        unpack8(raw[r][i], f[i]);
+        unpack(raw[r][i], f[i]);
 #pragma unroll
-        for (int e = 0; e < 8; e++) s += f[i][e];
+        for (int e = 0; e < EPC; e++) s += f[i][e];
       }
     }
     const float mean = wave_sum(s) * inv_d;
@@ -81,7 +112,7 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
       int c = lane + i * 64;
       if (c < nchunks) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
+        for (int e = 0; e < EPC; e++) {
           f[i][e] -= mean;
           q += f[i][e] * f[i][e];
         }
@@ -96,38 +127,35 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
     for (int i = 0; i < NCH; i++) {
       int c = lane + i * 64;
       if (c < nchunks) {
-        float o[8];
+        float o[EPC], w[EPC];
 #pragma unroll
-        for (int e = 0; e < 8; e++) o[e] = f[i][e] * rstd;
+        for (int e = 0; e < EPC; e++) o[e] = f[i][e] * rstd;
         if (lw) {
-          float w[8];
-          unpack8(*(const i32x4*)(lw + c * 8), w);
+          load_bf16(lw, c, w);
 #pragma unroll
-          for (int e = 0; e < 8; e++) o[e] *= w[e];
+          for (int e = 0; e < EPC; e++) o[e] *= w[e];
         }
         if (lb) {
-          float w[8];
-          unpack8(*(const i32x4*)(lb + c * 8), w);
+          load_bf16(lb, c, w);
 #pragma unroll
-          for (int e = 0; e < 8; e++) o[e] += w[e];
+          for (int e = 0; e < EPC; e++) o[e] += w[e];
         }
         if (sc) {
-          f32x4 s0 = *(const f32x4*)(sc + c * 8), s1 = *(const f32x4*)(sc + c * 8 + 4);
+          load_f32(sc, c, w);
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
-            o[e] *= 1.0f + s0[e];
-            o[e + 4] *= 1.0f + s1[e];
-          }
+          for (int e = 0; e < EPC; e++) o[e] *= 1.0f + w[e];
         }
         if (sh) {
-          f32x4 s0 = *(const f32x4*)(sh + c * 8), s1 = *(const f32x4*)(sh + c * 8 + 4);
+          load_f32(sh, c, w);
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
-            o[e] += s0[e];
-            o[e + 4] += s1[e];
-          }
+          for (int e = 0; e < EPC; e++) o[e] += w[e];
         }
-        *(i32x4*)(yr + c * 8) = pack8(o);
+        if constexpr (XF32) {
+          i32x2 pk = {(int)hdit::pack2(o[0], o[1]), (int)hdit::pack2(o[2], o[3])};
+          *(i32x2*)(yr + c * 4) = pk;
+        } else {
+          *(i32x4*)(yr + c * 8) = pack8(o);
+        }
       }
     }
   }
@@ -358,39 +386,53 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate_jo
   if (dim % 8) return HDIT_EINVAL;
   if (dim > 8192) return HDIT_EUNSUPPORTED;
   if (!aligned16(ln_weight) || !aligned16(ln_bias)) return HDIT_EINVAL;
-  LnJobs tab;
-  tab.count = 0;
-  int64_t blocks = 0;
-  for (int i = 0; i < count; i++) {
-    const hdit_ln_job& j = jobs[i];
-    if (j.batch < 0 || j.tokens < 0) return HDIT_EINVAL;
-    const int64_t rows = (int64_t)j.batch * j.tokens;
-    if (rows == 0) continue;  // an empty tensor may come with a null pointer
-    if (!j.x || !j.y) return HDIT_EINVAL;
-    if (j.x_sb % 8 || j.x_st % 8 || j.y_sb % 8 || j.y_st % 8 || j.mod_stride % 4) return HDIT_EINVAL;
-    if (!aligned16(j.x) || !aligned16(j.y) || !aligned16(j.shift) || !aligned16(j.scale)) return HDIT_EINVAL;
-    tab.block_start[tab.count] = (int)blocks;
-    tab.j[tab.count++] = j;
-    blocks += (rows + 7) / 8;  // 4 waves x 2 rows
-    if (blocks > 0x7fffffff) return HDIT_EUNSUPPORTED;
-  }
-  if (tab.count == 0) return HDIT_OK;
-  for (int i = tab.count; i <= HDIT_LN_MAX_JOBS; i++) tab.block_start[i] = (int)blocks;
-  dim3 grid((unsigned)blocks), block(256);
   hipStream_t s = (hipStream_t)stream;
-  int nch = (dim / 8 + 63) / 64;
-#define LN_LAUNCH(N) \
-  hipLaunchKernelGGL(ln_modulate_kernel<N>, grid, block, 0, s, tab, (const __bf16*)ln_weight, (const __bf16*)ln_bias, dim, eps)
-  if (nch <= 1) LN_LAUNCH(1);
-  else if (nch <= 2) LN_LAUNCH(2);
-  else if (nch <= 3) LN_LAUNCH(3);
-  else if (nch <= 4) LN_LAUNCH(4);
-  else if (nch <= 6) LN_LAUNCH(6);
-  else if (nch <= 8) LN_LAUNCH(8);
-  else if (nch <= 12) LN_LAUNCH(12);
-  else LN_LAUNCH(16);
+  // jobs that read a bf16 tensor and jobs that read the fp32 residual stream run as separate launches
+  for (int f32 = 0; f32 < 2; f32++) {
+    LnJobs tab;
+    tab.count = 0;
+    int64_t blocks = 0;
+    for (int i = 0; i < count; i++) {
+      const hdit_ln_job& j = jobs[i];
+      if (j.batch < 0 || j.tokens < 0) return HDIT_EINVAL;
+      if ((j.x_f32 != 0) != (f32 != 0)) continue;
+      const int64_t rows = (int64_t)j.batch * j.tokens;
+      if (rows == 0) continue;  // an empty tensor may come with a null pointer
+      if (!j.x || !j.y) return HDIT_EINVAL;
+      if (j.x_sb % 8 || j.x_st % 8 || j.y_sb % 8 || j.y_st % 8 || j.mod_stride % 4) return HDIT_EINVAL;
+      if (!aligned16(j.x) || !aligned16(j.y) || !aligned16(j.shift) || !aligned16(j.scale)) return HDIT_EINVAL;
+      tab.block_start[tab.count] = (int)blocks;
+      tab.j[tab.count++] = j;
+      blocks += (rows + 7) / 8;  // 4 waves x 2 rows
+      if (blocks > 0x7fffffff) return HDIT_EUNSUPPORTED;
+    }
+    if (tab.count == 0) continue;
+    for (int i = tab.count; i <= HDIT_LN_MAX_JOBS; i++) tab.block_start[i] = (int)blocks;
+    dim3 grid((unsigned)blocks), block(256);
+    if (f32 && dim > 4096) return HDIT_EUNSUPPORTED;  // a row of the fp32 stream is held in registers: 16 chunks per lane
+    const int nch = (dim / (f32 ? 4 : 8) + 63) / 64;
+#define LN_LAUNCH(N)                                                                                                  \
+  do {                                                                                                                \
+    if (f32)                                                                                                          \
+      hipLaunchKernelGGL((ln_modulate_kernel<N, true>), grid, block, 0, s, tab, (const __bf16*)ln_weight,             \
+                         (const __bf16*)ln_bias, dim, eps);                                                           \
+    else                                                                                                              \
+      hipLaunchKernelGGL((ln_modulate_kernel<N, false>), grid, block, 0, s, tab, (const __bf16*)ln_weight,            \
+                         (const __bf16*)ln_bias, dim, eps);                                                           \
+  } while (0)
+    if (nch <= 1) LN_LAUNCH(1);
+    else if (nch <= 2) LN_LAUNCH(2);
+    else if (nch <= 3) LN_LAUNCH(3);
+    else if (nch <= 4) LN_LAUNCH(4);
+    else if (nch <= 6) LN_LAUNCH(6);
+    else if (nch <= 8) LN_LAUNCH(8);
+    else if (nch <= 12) LN_LAUNCH(12);
+    else LN_LAUNCH(16);
 #undef LN_LAUNCH
-  return hdit_host::check_launch("hdit_layernorm_modulate");
+    const int rc = hdit_host::check_launch("hdit_layernorm_modulate");
+    if (rc != HDIT_OK) return rc;
+  }
+  return HDIT_OK;
 }
 
 extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate(const void* x, void* y, const float* shift, const float* scale,
@@ -400,6 +442,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate(co
   hdit_ln_job j;
   j.x = x, j.y = y, j.shift = shift, j.scale = scale;
   j.batch = batch, j.tokens = tokens;
+  j.x_f32 = 0, j.pad_ = 0;
   j.x_sb = x_sb, j.x_st = x_st, j.y_sb = y_sb, j.y_st = y_st, j.mod_stride = mod_stride;
   return hdit_layernorm_modulate_jobs(&j, 1, dim, ln_weight, ln_bias, eps, stream);
 }

@@ -186,13 +186,15 @@ class hetuDiTAttentionWrapper(hetuDiTAttentionBaseWrapper):
     def out_proj_problems(self, o_img, o_txt, resid_img=None, gate_img=None, resid_txt=None, gate_txt=None):
         """Problems for ``to_out[0]`` (+ ``output_bias``) and ``to_add_out``
         (+ ``encoder_output_bias`` unless ``encoder_bias`` is off for this
-        family).  With ``resid``/``gate`` the epilogue is the gated residual."""
+        family).  With ``resid``/``gate`` the epilogue is the gated residual and
+        the result is f32: the residual stream inside a block is carried in fp32."""
         m = self.module
         problems, outs = [], []
 
         def one(o, weight, bias, resid, gate):
             B, T, _ = o.shape
-            out = torch.empty(B, T, weight.shape[0], dtype=torch.bfloat16, device=o.device)
+            out = torch.empty(B, T, weight.shape[0], dtype=torch.bfloat16 if resid is None else torch.float32,
+                              device=o.device)
             if resid is None:
                 problems.append(ops.gemm_problem(_rows2d(o), weight, out.view(-1, out.shape[-1]), bias))
             else:
@@ -274,8 +276,8 @@ class hetuDiTJointAttnProcessor2_0(JointAttnProcessor2_0):
     def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, *args, **kwargs):
         H = attn.heads_per_device
         inner = attn.module.to_k.weight.shape[0]
-        p_img, q_img, kv_img = _qkv_problems(hidden_states, attn._qkv, attn.module, inner, use_cache=True)
-        p_txt, q_txt, kv_txt = _qkv_problems(encoder_hidden_states, attn._add_qkv, attn.module, inner, use_cache=False)
+        p_img, q_img, kv_img = _qkv_problems(hidden_states, attn._qkv, attn, inner, use_cache=True)
+        p_txt, q_txt, kv_txt = _qkv_problems(encoder_hidden_states, attn._add_qkv, attn, inner, use_cache=False)
         ops.gemm_launch(p_img + p_txt)
         B, N, _ = hidden_states.shape
         Nt = encoder_hidden_states.shape[1]
@@ -346,8 +348,8 @@ class hetuDiTFluxAttnProcessor2_0(FluxAttnProcessor2_0):
         if encoder_hidden_states is not None:
             n_txt = encoder_hidden_states.shape[1]
             N = hidden_states.shape[1]
-            p_img, q_img, kv_img = _qkv_problems(hidden_states, attn._qkv, m, inner, use_cache=True)
-            p_txt, q_txt, kv_txt = _qkv_problems(encoder_hidden_states, attn._add_qkv, m, inner, use_cache=False)
+            p_img, q_img, kv_img = _qkv_problems(hidden_states, attn._qkv, attn, inner, use_cache=True)
+            p_txt, q_txt, kv_txt = _qkv_problems(encoder_hidden_states, attn._add_qkv, attn, inner, use_cache=False)
             ops.gemm_launch(p_img + p_txt)
             waq, _ = _norm_wb(m.norm_added_q)
             wak, _ = _norm_wb(m.norm_added_k)
@@ -382,7 +384,7 @@ class hetuDiTFluxAttnProcessor2_0(FluxAttnProcessor2_0):
             qkv = torch.empty(B, S, 3 * inner, dtype=torch.bfloat16, device=dev)
             ops.gemm_launch([ops.gemm_problem(x2, w, qkv.view(-1, 3 * inner), b)] + extra_problems)
             q = qkv[:, :, :inner]
-            get_cache_manager()._entry(m, "attn").tensors[0] = qkv[:, n_txt:, inner:]
+            get_cache_manager()._entry(attn, "attn").tensors[0] = qkv[:, n_txt:, inner:]
             k_segs = [_heads(qkv[:, :, inner:2 * inner], H)]
             v_segs = [_heads(qkv[:, :, 2 * inner:], H)]
             jobs = [
@@ -391,7 +393,7 @@ class hetuDiTFluxAttnProcessor2_0(FluxAttnProcessor2_0):
             ]
         else:
             # patch mode: text rows and the image patch rows form this call's joint input
-            buf, start, end = get_cache_manager().kv_buffer(m, B, N, inner, dev)
+            buf, start, end = get_cache_manager().kv_buffer(attn, B, N, inner, dev)
             qkv = torch.empty(B, S, 3 * inner, dtype=torch.bfloat16, device=dev)
             ops.gemm_launch([ops.gemm_problem(x2, w, qkv.view(-1, 3 * inner), b)] + extra_problems)
             ops.copy_rows(qkv[:, n_txt:, inner:], buf[:, start:end])

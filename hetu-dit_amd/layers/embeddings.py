@@ -51,9 +51,10 @@ class hetuDiTPatchEmbedWrapper(hetuDiTDiffusionLayerBaseWrapper):
             return out
         if rs.patch_mode:
             # the latent holds the rows of the current pipeline patch; the table is that of the whole image
-            if not rs.latents_height:
-                raise ValueError("patch mode needs the latent height of the whole image (runtime state set_patches)")
-            height = rs.latents_height
+            height = rs.whole_image_latent_rows()
+            if not height:
+                raise ValueError("patch mode needs the height of the whole image: input_config.height and "
+                                 "vae_scale_factor on the runtime state (set_input_parameters), or set_patches")
             start, end = rs.pp_patches_token_start_end_idx_global[rs.pipeline_patch_idx]
         else:
             height, start, end = H, 0, T

@@ -87,8 +87,15 @@ def gemm_problem(
     """Describe out[m, n] = epilogue(a[m, k] @ w[n, k]^T + bias).
 
     a, out (and resid) are 2-D views with unit inner stride (row stride free);
-    gate is an f32 [batch, n] view with unit inner stride."""
-    _need(a, bf16, "a"), _need(w, bf16, "w"), _need(out, bf16, "out")
+    gate is an f32 [batch, n] view with unit inner stride.  In the gated-residual
+    epilogue ``resid`` and ``out`` may each be f32 instead of bf16 (the residual
+    stream of a block stack carried in fp32)."""
+    _need(a, bf16, "a"), _need(w, bf16, "w")
+    if epilogue == EPI_GATE_RESIDUAL and out.dtype == torch.float32:
+        _need(out, torch.float32, "out")
+        epilogue |= _lib.EPI_OUT_F32
+    else:
+        _need(out, bf16, "out")
     m, k = a.shape
     n, k2 = w.shape
     if k2 != k or tuple(out.shape) != (m, n):
@@ -105,8 +112,11 @@ def gemm_problem(
         if bias.numel() != n or not bias.is_contiguous():
             raise ValueError("bias must be a contiguous [n] vector")
         p.bias = bias.data_ptr()
-    if epilogue == EPI_GATE_RESIDUAL:
-        _need(resid, bf16, "resid"), _need(gate, torch.float32, "gate")
+    if epilogue & 0xF == EPI_GATE_RESIDUAL:
+        if resid is not None and resid.dtype == torch.float32:
+            epilogue |= _lib.EPI_RESID_F32
+        _need(resid, torch.float32 if epilogue & _lib.EPI_RESID_F32 else bf16, "resid"), _need(gate, torch.float32, "gate")
+        p.epilogue = epilogue
         if tuple(resid.shape) != (m, n) or resid.stride(1) != 1:
             raise ValueError("resid must be [m, n] with unit inner stride")
         if gate.dim() != 2 or gate.shape[1] != n or gate.stride(1) != 1:
@@ -206,9 +216,9 @@ def attention(q: Sequence[torch.Tensor], k: Sequence[torch.Tensor], v: Sequence[
 # glue
 # ---------------------------------------------------------------------------
 
-def _as3d(x: torch.Tensor, name: str) -> Tuple[int, int, int, int, int]:
+def _as3d(x: torch.Tensor, name: str, dtype=bf16) -> Tuple[int, int, int, int, int]:
     """[B, T, D] view with unit inner stride; returns (B, T, D, batch stride, token stride)."""
-    _need(x, bf16, name)
+    _need(x, dtype, name)
     if x.dim() != 3 or x.stride(2) != 1:
         raise ValueError(f"{name} must be [batch, tokens, dim] with unit inner stride")
     B, T, D = x.shape
@@ -227,6 +237,10 @@ def _mod(v: Optional[torch.Tensor], B: int, D: int, name: str):
 
 
 def layernorm_modulate(x, shift=None, scale=None, eps: float = 1e-6, ln_weight=None, ln_bias=None, out=None):
+    """bf16 out = LayerNorm(x) * (1 + scale) + shift; x bf16, or f32 (the fp32 residual stream)."""
+    if x.dtype == torch.float32:
+        return layernorm_modulate_many([(x, shift, scale, out) if out is not None else (x, shift, scale)], eps, ln_weight,
+                                       ln_bias)[0]
     B, T, D, xsb, xst = _as3d(x, "x")
     if out is None:
         out = torch.empty(B, T, D, dtype=bf16, device=x.device)
@@ -260,7 +274,8 @@ def layernorm_modulate_many(items, eps: float = 1e-6, ln_weight=None, ln_bias=No
     for i, it in enumerate(items):
         x, shift, scale = it[0], it[1], it[2]
         out = it[3] if len(it) > 3 else None
-        B, T, D, xsb, xst = _as3d(x, "x")
+        x_f32 = x.dtype == torch.float32
+        B, T, D, xsb, xst = _as3d(x, "x", torch.float32 if x_f32 else bf16)
         if D0 is None:
             D0 = D
         elif D != D0:
@@ -277,10 +292,10 @@ def layernorm_modulate_many(items, eps: float = 1e-6, ln_weight=None, ln_bias=No
         j = jobs[i]
         j.x, j.y, j.shift, j.scale = x.data_ptr(), out.data_ptr(), sh, sc
         j.x_sb, j.x_st, j.y_sb, j.y_st, j.mod_stride = xsb, xst, ysb, yst, (st1 or st2 or 0)
-        j.batch, j.tokens = B, T
+        j.batch, j.tokens, j.x_f32 = B, T, int(x_f32)
         outs.append(out)
         keep.append((x, shift, scale, out))
-        nbytes += 4.0 * B * T * D
+        nbytes += (6.0 if x_f32 else 4.0) * B * T * D
     for w in (ln_weight, ln_bias):
         if w is not None:
             _need(w, bf16, "ln affine")

@@ -6,8 +6,23 @@ with the same names, plus the patch-metadata arithmetic of
 from typing import List, Optional
 
 
+class InputConfig:
+    """The request geometry the reference keeps on its runtime state
+    (``runtime_state.py:50-58,:305-321``): image height / width in pixels (0 = not set)."""
+
+    def __init__(self):
+        self.height: int = 0
+        self.width: int = 0
+        self.batch_size: int = 1
+        self.num_frames: int = 0
+
+
 class DiTRuntimeState:
     def __init__(self):
+        # pixels; latent rows of the whole image = input_config.height // vae_scale_factor
+        # (runtime_state.py:340-342, read by the patch-embedding wrapper at layers/embeddings.py:33-36)
+        self.input_config = InputConfig()
+        self.vae_scale_factor: int = 8
         self.patch_mode: bool = False
         self.pipeline_patch_idx: int = 0
         self.num_pipeline_patch: int = 1
@@ -18,11 +33,27 @@ class DiTRuntimeState:
         # [start, end) token range of every pipeline patch within the whole image (runtime_state.py:106); with one
         # sequence-parallel rank the global ranges are the local ones
         self.pp_patches_token_start_end_idx_global: List[List[int]] = []
-        # latent rows of the whole image (the reference's input_config.height // vae_scale_factor); 0 = unknown
+        # latent rows of the whole image when no pixel geometry was given (set_patches / set_token_patches); 0 = unknown
         self.latents_height: int = 0
         self.max_condition_sequence_length: int = 0
         # forced False by the reference (runtime_state.py:188,:225)
         self.split_text_embed_in_sp: bool = False
+
+    def set_input_parameters(self, height: Optional[int] = None, width: Optional[int] = None,
+                             batch_size: Optional[int] = None, vae_scale_factor: Optional[int] = None):
+        """Pixel geometry of the request (``runtime_state.py:296-309``)."""
+        self.input_config.height = height or self.input_config.height
+        self.input_config.width = width or self.input_config.width
+        self.input_config.batch_size = batch_size or self.input_config.batch_size
+        if vae_scale_factor:
+            self.vae_scale_factor = vae_scale_factor
+
+    def whole_image_latent_rows(self) -> int:
+        """Latent rows of the whole image: ``input_config.height // vae_scale_factor`` as the reference's
+        patch-embedding wrapper computes it, else what ``set_patches`` recorded; 0 if neither is known."""
+        if self.input_config.height:
+            return self.input_config.height // self.vae_scale_factor
+        return self.latents_height
 
     # -- runtime_state.py:254-264 -------------------------------------------
     def set_patched_mode(self, patch_mode: bool):

@@ -15,7 +15,7 @@ import torch
 from torch import nn
 
 from .blocks import (CogVideoXBlock, FluxSingleTransformerBlock, FluxTransformerBlock, JointTransformerBlock,
-                     StackModulation)
+                     StackModulation, use_fp32_residual_stream)
 from .runtime_state import get_runtime_state
 
 
@@ -32,6 +32,7 @@ class SD3TransformerBlocks(nn.Module):
         )
         self.encoder_hidden_states_cache: List[Optional[torch.Tensor]] = [None] * num_layers
         self.modulation = StackModulation(self.transformer_blocks)
+        use_fp32_residual_stream(self.transformer_blocks)
 
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb):
@@ -65,6 +66,7 @@ class FluxTransformerBlocks(nn.Module):
             [FluxSingleTransformerBlock(dim, num_attention_heads, attention_head_dim) for _ in range(num_single_layers)]
         )
         self.modulation = StackModulation(list(self.transformer_blocks) + list(self.single_transformer_blocks))
+        use_fp32_residual_stream(list(self.transformer_blocks) + list(self.single_transformer_blocks))
 
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb):
@@ -91,6 +93,7 @@ class CogVideoXTransformerBlocks(nn.Module):
             [CogVideoXBlock(dim, num_attention_heads, attention_head_dim, time_embed_dim) for _ in range(num_layers)]
         )
         self.modulation = StackModulation(self.transformer_blocks)
+        use_fp32_residual_stream(self.transformer_blocks)
 
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None) -> Tuple[torch.Tensor, torch.Tensor]:

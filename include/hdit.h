@@ -63,13 +63,22 @@ int hdit_clock_sample(void* out, int slots, void* stream);
 #define HDIT_EPI_BIAS 0          /* C = acc + bias */
 #define HDIT_EPI_BIAS_GELU 1     /* C = gelu_tanh(acc + bias) */
 #define HDIT_EPI_GATE_RESIDUAL 2 /* C = resid + gate[row / rows_per_batch] * (acc + bias) */
+#define HDIT_EPI_MODE_MASK 0xf
+/* Flags ORed into `epilogue` with HDIT_EPI_GATE_RESIDUAL: the residual stream of a
+ * block stack carried in fp32 between the gated residuals, so that its rounding
+ * does not accumulate over 24+ blocks.  With HDIT_EPI_RESID_F32 `resid` is f32
+ * [m, n] (ldr in f32 elements), with HDIT_EPI_OUT_F32 `c` is f32 [m, n] (ldc in
+ * f32 elements); the sum resid + gate * (.) is formed in fp32 either way. */
+#define HDIT_EPI_RESID_F32 0x10
+#define HDIT_EPI_OUT_F32 0x20
 
 typedef struct hdit_gemm_problem {
   const void* a;     /* bf16 [m, k] */
   const void* b;     /* bf16 [n, k] */
-  void* c;           /* bf16 [m, n] */
+  void* c;           /* bf16 [m, n] (f32 with HDIT_EPI_OUT_F32) */
   const void* bias;  /* bf16 [n] or NULL */
-  const void* resid; /* bf16 [m, n] (ldr), HDIT_EPI_GATE_RESIDUAL only; may alias c */
+  const void* resid; /* bf16 [m, n] (ldr; f32 with HDIT_EPI_RESID_F32), HDIT_EPI_GATE_RESIDUAL only; may alias c
+                        when both have one element type */
   const float* gate; /* f32, element (batch, col) at gate[batch * gate_stride + col] */
   int64_t lda, ldb, ldc, ldr;
   int32_t m, n, k;
@@ -151,12 +160,14 @@ int hdit_layernorm_modulate(const void* x, void* y, const float* shift, const fl
  * norm2 + norm2_context, of the blocks cited above). */
 #define HDIT_LN_MAX_JOBS 4
 typedef struct hdit_ln_job {
-  const void* x;      /* bf16 [batch, tokens, dim] */
+  const void* x;      /* bf16 [batch, tokens, dim], or f32 with x_f32 */
   void* y;            /* bf16 [batch, tokens, dim] */
   const float* shift; /* f32, batch stride mod_stride, or NULL */
   const float* scale;
   int64_t x_sb, x_st, y_sb, y_st, mod_stride;
   int32_t batch, tokens;
+  int32_t x_f32; /* != 0: x is f32 [batch, tokens, dim] (strides in f32 elements): the fp32 residual stream */
+  int32_t pad_;
 } hdit_ln_job;
 
 int hdit_layernorm_modulate_jobs(const hdit_ln_job* jobs, int count, int dim, const void* ln_weight,

@@ -426,3 +426,92 @@ def test_attention_random_shapes(hdit):
         torch.cuda.synchronize()
         want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
         assert_parity(o, want, what=f"attention random case {it}")
+
+
+# ---------------------------------------------------------------------------
+# fp32 residual stream: gated-residual epilogue with f32 residual and / or f32 output, LayerNorm on f32 rows
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4])
+@pytest.mark.parametrize("resid_f32,out_f32", [(True, True), (False, True), (True, False)])
+@pytest.mark.parametrize("m,n,k", [(666, 1536, 128), (1000, 520, 64), (4100, 1536, 192)])
+def test_gemm_gate_residual_fp32_stream(hdit, m, n, k, resid_f32, out_f32, cfg):
+    """out = resid + gate * (a w^T + b) with the residual and / or the result in fp32; rows straddle the batch
+    boundary inside a tile, n is not a multiple of the tile width, and (f32 -> f32) is also run in place."""
+    print(f"gemm fp32 stream m={m} n={n} k={k} resid_f32={resid_f32} out_f32={out_f32} cfg={cfg}", flush=True)
+    ops = hdit.ops
+    a, w, b = rnd(m, k, seed=61), rnd(n, k, scale=0.05, seed=62), rnd(n, seed=63)
+    gen = torch.Generator().manual_seed(64)
+    r32 = torch.randn(m, n, generator=gen)
+    r = r32 if resid_f32 else bf16_round(r32)
+    gate = torch.randn(2, n, generator=gen)
+    rows = (m + 1) // 2
+    lin = O.linear(a, w, b)
+    want = r + gate.repeat_interleave(rows, dim=0)[:m] * lin
+    hdit._lib.lib().hdit_gemm_force_config(cfg)
+    try:
+        resid = r.to(DEV) if resid_f32 else g(r)
+        out = torch.empty(m, n, dtype=torch.float32 if out_f32 else torch.bfloat16, device=DEV)
+        ops.gemm_launch([ops.gemm_problem(g(a), g(w), out, g(b), ops.EPI_GATE_RESIDUAL, resid=resid, gate=gate.to(DEV),
+                                          rows_per_batch=rows)])
+        torch.cuda.synchronize()
+        assert out.dtype == (torch.float32 if out_f32 else torch.bfloat16)
+        # the update gate * (acc + bias) is rounded to bf16 once; the sum itself is exact in fp32
+        assert_parity(out, want, rel=3e-3, what="gate residual, fp32 stream")
+        if out_f32:
+            # an f32 result keeps the bits a bf16 stream would drop
+            assert (out != out.to(torch.bfloat16).float()).float().mean() > 0.9
+        if resid_f32 and out_f32:
+            inplace = resid.clone()
+            ops.gemm_launch([ops.gemm_problem(g(a), g(w), inplace, g(b), ops.EPI_GATE_RESIDUAL, resid=inplace,
+                                              gate=gate.to(DEV), rows_per_batch=rows)])
+            torch.cuda.synchronize()
+            assert torch.equal(inplace, out)
+    finally:
+        hdit._lib.lib().hdit_gemm_force_config(-1)
+
+
+def test_gemm_fp32_flags_only_with_gate_residual(hdit):
+    from hetu_dit_amd import _lib
+
+    ops = hdit.ops
+    a, w = g(rnd(64, 64)), g(rnd(64, 64))
+    out = torch.empty(64, 64, dtype=torch.bfloat16, device=DEV)
+    p = ops.gemm_problem(a, w, out)
+    p.epilogue = _lib.EPI_BIAS | _lib.EPI_OUT_F32
+    arr = (_lib.GemmProblem * 1)(p)
+    assert _lib.lib().hdit_gemm_bf16(arr, 1, None) == -1
+    with pytest.raises(TypeError):
+        ops.gemm_problem(a, w, torch.empty(64, 64, dtype=torch.float32, device=DEV))
+
+
+@pytest.mark.parametrize("D", [256, 1536, 3072, 4096, 264])
+@pytest.mark.parametrize("affine", [False, True])
+def test_layernorm_modulate_fp32_rows(hdit, D, affine):
+    """LayerNorm + modulate reading the fp32 residual stream, alone and in one call with a bf16 tensor."""
+    print(f"ln fp32 D={D} affine={affine}", flush=True)
+    ops = hdit.ops
+    B, T, T2 = 2, 37, 9
+    gen = torch.Generator().manual_seed(71)
+    x = torch.randn(B, T, D, generator=gen) * 3 + 0.5
+    x2 = rnd(B, T2, D, seed=72)
+    sh, sc = torch.randn(B, D, generator=gen), torch.randn(B, D, generator=gen) * 0.1
+    lw = rnd(D, seed=73) if affine else None
+    lb = rnd(D, seed=74) if affine else None
+    want = O.modulate(O.layer_norm(x, 1e-5, lw, lb), sh, sc)
+    want2 = O.modulate(O.layer_norm(x2, 1e-5, lw, lb), sh, sc)
+    args = dict(eps=1e-5, ln_weight=g(lw) if affine else None, ln_bias=g(lb) if affine else None)
+    got = ops.layernorm_modulate(x.to(DEV), sh.to(DEV), sc.to(DEV), **args)
+    y1, y2 = ops.layernorm_modulate_many([(x.to(DEV), sh.to(DEV), sc.to(DEV)), (g(x2), sh.to(DEV), sc.to(DEV))], **args)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16
+    assert_parity(got, want, rel=4e-3, what="ln fp32 rows")
+    assert torch.equal(got, y1)
+    assert_parity(y2, want2, rel=4e-3, what="ln bf16 rows in the same call")
+    # strided fp32 rows (a slice of a wider stream) into a slice of a joint buffer
+    wide = torch.zeros(B, T, 2 * D, device=DEV)
+    wide[:, :, D:] = x.to(DEV)
+    joint = torch.zeros(B, T + 3, D, dtype=torch.bfloat16, device=DEV)
+    ops.layernorm_modulate_many([(wide[:, :, D:], sh.to(DEV), sc.to(DEV), joint[:, 3:])], **args)
+    torch.cuda.synchronize()
+    assert torch.equal(joint[:, 3:], got) and not joint[:, :3].any()
