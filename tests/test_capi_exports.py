@@ -47,7 +47,7 @@ def test_binding_covers_every_declared_symbol():
 
     assert sorted(_lib.SIGNATURES) == declared_symbols()
     lib = _lib.lib()
-    assert lib.hdit_abi_version() == 1
+    assert lib.hdit_abi_version() == _lib.ABI_VERSION == 2
     assert lib.hdit_last_error() == b""
 
 
@@ -59,6 +59,7 @@ def test_struct_layouts_match_the_header(library):
     assert ctypes.sizeof(_lib.SeqSegment) == 8 + 3 * 8 + 2 * 4
     assert ctypes.sizeof(_lib.AttnArgs) == 8 * ctypes.sizeof(_lib.SeqSegment) + 4 * 4
     assert ctypes.sizeof(_lib.QkNormJob) == 8 + 3 * 8 + 4 * 8 + 4 * 4
+    assert ctypes.sizeof(_lib.LnJob) == 4 * 8 + 5 * 8 + 4 * 4
 
 
 def test_entry_points_reject_bad_arguments_without_a_gpu(library):
@@ -80,6 +81,10 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(library):
     a = _lib.AttnArgs()
     a.batch, a.heads, a.head_dim = 1, 1, 96
     assert lib.hdit_attn_fwd_bf16(ctypes.byref(a), None) == -2
+    p.a = 4096
+    p.epilogue = _lib.EPI_BIAS | _lib.EPI_OUT_F32  # the fp32 stream flags belong to the gated-residual epilogue only
+    arr = (_lib.GemmProblem * 1)(p)
+    assert lib.hdit_gemm_bf16(arr, 1, None) == -1
     assert lib.hdit_layernorm_modulate(None, None, None, None, None, None, 1, 1, 64, 64, 64, 64, 64, 0, 1e-6, None) == -1
     assert lib.hdit_layernorm_modulate_jobs(None, 1, 64, None, None, 1e-6, None) == -1
     assert lib.hdit_adaln_gemv(4096, 4096, None, 4096, 9, 16, 64, None) == -2
