@@ -105,6 +105,7 @@ SIGNATURES = {
     "hdit_attn_absmax": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p]),
     "hdit_attn_fp8_workspace_bytes": (C.c_int64, [C.POINTER(AttnArgs)]),
     "hdit_attn_fwd_fp8": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p, C.c_void_p]),
+    "hdit_attn_fwd_fp8_static": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p]),
     "hdit_layernorm_modulate": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
@@ -175,12 +176,12 @@ class HditError(RuntimeError):
     pass
 
 
-_CODES = {-1: "HDIT_EINVAL", -2: "HDIT_EUNSUPPORTED", -3: "HDIT_ELAUNCH"}
+_CODES = {-1: "HDIT_EINVAL", -2: "HDIT_EUNSUPPORTED", -3: "HDIT_ELAUNCH", -4: "HDIT_ETOOLARGE"}
 
 
 def check(rc: int, what: str):
     if rc != 0:
         detail = ""
-        if rc == -3:
+        if rc in (-3, -4):
             detail = ": " + lib().hdit_last_error().decode()
         raise HditError(f"{what} failed with {_CODES.get(rc, rc)}{detail}")

@@ -18,6 +18,7 @@
 // In the 32x32 accumulator layout a lane's 32 score registers are exactly its
 // 32 bytes of the P^T "B" operand; the matching V^T "A" bytes are gathered from
 // the row-major fp8 V tile with the byte transpose read (ds_read_b64_tr_b8).
+#include <atomic>
 #include <type_traits>
 
 #include "hdit_common.h"
@@ -423,14 +424,11 @@ extern "C" __attribute__((visibility("default"))) int64_t hdit_attn_fp8_workspac
   return (int64_t)(2 * kv8_bytes(a));
 }
 
-extern "C" __attribute__((visibility("default"))) int hdit_attn_fwd_fp8(const hdit_attn_args* a, const float* absmax, void* workspace,
-                                                                         void* stream) {
-  int rc = hdit_host::attn_validate(a);
-  if (rc != HDIT_OK) return rc;
-  if (!absmax || !workspace || (((uintptr_t)workspace) & 15)) return HDIT_EINVAL;
+namespace {
+
+int fwd_fp8_launch(const hdit_attn_args* a, const float* absmax, void* workspace, hipStream_t s, const char* what) {
   AttnParams P = make_params(a, absmax, workspace);
   if (P.sq == 0) return HDIT_OK;
-  hipStream_t s = (hipStream_t)stream;
   const int cpr = a->head_dim / 8;
   dim3 qgrid((unsigned)((P.skv_pad * cpr + 255) / 256), (unsigned)(a->batch * a->heads));
   if (a->head_dim == 64)
@@ -443,5 +441,63 @@ extern "C" __attribute__((visibility("default"))) int hdit_attn_fwd_fp8(const hd
     hipLaunchKernelGGL(attn_fp8_kernel<64>, grid, block, Lds8<64>::TOTAL, s, P, q_tiles);
   else
     hipLaunchKernelGGL(attn_fp8_kernel<128>, grid, block, Lds8<128>::TOTAL, s, P, q_tiles);
-  return hdit_host::check_launch("hdit_attn_fwd_fp8");
+  return hdit_host::check_launch(what);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------------
+// The quantised K / V copy of hdit_attn_fwd_fp8_static lives in this array instead of a caller workspace.
+// Every GPU the library runs on holds its own copy at its own address until the process ends; in host
+// code the name below is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t STATIC_SCRATCH_BYTES = HDIT_ATTN_FP8_STATIC_MAX_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> g_scratch_ptr[MAX_DEVICES];
+
+// Device address of `scratch` on the current device, looked up once per device (the first call on it).
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    hdit_host::set_error(hipGetErrorString(e));
+    return HDIT_ELAUNCH;
+  }
+  if (dev < 0 || dev >= MAX_DEVICES) return HDIT_EUNSUPPORTED;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // the same address for every thread asking on this device
+    if (e != hipSuccess || !p) {
+      hdit_host::set_error(e != hipSuccess ? hipGetErrorString(e) : "hipGetSymbolAddress returned a null address");
+      return HDIT_ELAUNCH;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return HDIT_OK;
+}
+
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int hdit_attn_fwd_fp8(const hdit_attn_args* a, const float* absmax, void* workspace,
+                                                                         void* stream) {
+  int rc = hdit_host::attn_validate(a);
+  if (rc != HDIT_OK) return rc;
+  if (!absmax || !workspace || (((uintptr_t)workspace) & 15)) return HDIT_EINVAL;
+  return fwd_fp8_launch(a, absmax, workspace, (hipStream_t)stream, "hdit_attn_fwd_fp8");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_attn_fwd_fp8_static(const hdit_attn_args* a, const float* absmax,
+                                                                                void* stream) {
+  int rc = hdit_host::attn_validate(a);
+  if (rc != HDIT_OK) return rc;
+  if (!absmax) return HDIT_EINVAL;
+  if (2 * kv8_bytes(a) > STATIC_SCRATCH_BYTES) {
+    hdit_host::set_error("hdit_attn_fwd_fp8_static: batch * heads * keys (padded to 64) * head_dim * 2 exceeds "
+                         "HDIT_ATTN_FP8_STATIC_MAX_BYTES; use hdit_attn_fwd_fp8 with a caller workspace");
+    return HDIT_ETOOLARGE;
+  }
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != HDIT_OK) return rc;
+  return fwd_fp8_launch(a, absmax, ws, (hipStream_t)stream, "hdit_attn_fwd_fp8_static");
 }

@@ -212,6 +212,24 @@ def attention(q: Sequence[torch.Tensor], k: Sequence[torch.Tensor], v: Sequence[
     return list(out)
 
 
+def attention_fp8_absmax(args: AttnArgs) -> torch.Tensor:
+    """f32 [3, batch, heads] absmax of q, k, v per (batch, head): the scales of the fp8 path."""
+    dev = args._keep[0][0].device
+    absmax = torch.empty(3, args.batch, args.heads, dtype=torch.float32, device=dev)
+    check(_lib.lib().hdit_attn_absmax(C.byref(args), absmax.data_ptr(), _stream()), "hdit_attn_absmax")
+    return absmax
+
+
+def attention_fp8_static(args: AttnArgs, absmax: torch.Tensor):
+    """fp8 attention through the entry point that allocates nothing: the quantised K / V copy lives in a
+    fixed array inside the library (``HDIT_ATTN_FP8_STATIC_MAX_BYTES`` per GPU) instead of a workspace.
+    Calls on one GPU share that array and must not overlap."""
+    _need(absmax, torch.float32, "absmax")
+    if tuple(absmax.shape) != (3, args.batch, args.heads) or not absmax.is_contiguous():
+        raise ValueError("absmax must be a contiguous f32 [3, batch, heads] tensor")
+    check(_lib.lib().hdit_attn_fwd_fp8_static(C.byref(args), absmax.data_ptr(), _stream()), "hdit_attn_fwd_fp8_static")
+
+
 # ---------------------------------------------------------------------------
 # glue
 # ---------------------------------------------------------------------------

@@ -25,6 +25,7 @@ extern "C" {
 #define HDIT_EINVAL (-1)      /* bad shape / stride / alignment / null pointer */
 #define HDIT_EUNSUPPORTED (-2) /* shape outside what the kernels are built for */
 #define HDIT_ELAUNCH (-3)     /* the HIP runtime refused the launch */
+#define HDIT_ETOOLARGE (-4)   /* the problem needs more than a fixed-size internal buffer holds */
 
 /* Version of this ABI; bumped when a struct below changes. */
 int hdit_abi_version(void);
@@ -136,6 +137,21 @@ int hdit_attn_fwd_bf16(const hdit_attn_args* args, void* stream);
 int hdit_attn_absmax(const hdit_attn_args* args, float* absmax, void* stream);
 int64_t hdit_attn_fp8_workspace_bytes(const hdit_attn_args* args);
 int hdit_attn_fwd_fp8(const hdit_attn_args* args, const float* absmax, void* workspace, void* stream);
+
+/* hdit_attn_fwd_fp8 without a workspace argument, for callers that cannot
+ * allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * The quantised K / V copy goes into a fixed array inside the library's device
+ * image (HDIT_ATTN_FP8_STATIC_MAX_BYTES per GPU, held until the process ends)
+ * instead; the call allocates and frees nothing.  Results are bit-identical to
+ * hdit_attn_fwd_fp8 on the same arguments.  A problem whose workspace
+ * (hdit_attn_fp8_workspace_bytes) exceeds the array is refused with
+ * HDIT_ETOOLARGE and a message in hdit_last_error.  All calls on one GPU share
+ * that GPU's array: calls that overlap there (two streams, two threads) race;
+ * serialise them.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress): make that call outside graph capture. */
+#define HDIT_ATTN_FP8_STATIC_MAX_BYTES (32u << 20)
+int hdit_attn_fwd_fp8_static(const hdit_attn_args* args, const float* absmax, void* stream);
 
 /* ------------------------------------------------------------------------
  * Bandwidth-bound glue, one coalesced pass each.
