@@ -35,17 +35,29 @@ therefore pinned by what mathematics and PyTorch's own library routines fix
                            position-0 identity, relative-position property
 * ``flux_rope_table`` / ``cogvideox_rope_table`` -- closed-form angle checks
 * stale KV buffer       -- brute-force concatenation of fresh and stale slices
-* block wiring (``sd3_joint_block``, ``flux_double_block``, ``flux_single_block``,
-  ``cogvideox_block``): the composition order, chunk orders, eps values and
-  which LayerNorm carries affine weights follow the published diffusers
-  modules (``JointTransformerBlock``, ``FluxTransformerBlock``,
+* block wiring (``sd3_joint_block`` with and without ``context_pre_only``,
+  ``flux_double_block``, ``flux_single_block``, ``cogvideox_block``, and the
+  attention functions inside them): every block is assembled a second time in
+  ``tests/test_oracle_wiring.py`` from PyTorch's library modules
+  (``nn.LayerNorm``, ``nn.Linear``, ``F.silu``, ``F.gelu(approximate="tanh")``,
+  ``F.rms_norm``, ``F.scaled_dot_product_attention``, complex multiplication for
+  the rotary embedding) in the order of the published diffusers ``forward`` of
+  ``JointTransformerBlock``, ``FluxTransformerBlock``,
   ``FluxSingleTransformerBlock``, ``CogVideoXBlock``, ``AdaLayerNormZero``,
   ``AdaLayerNormZeroSingle``, ``AdaLayerNormContinuous``,
-  ``CogVideoXLayerNormZero``).  diffusers cannot be imported here, so this
-  wiring is **parity unpinned** beyond the constraints the reference's call
-  sites fix (joint ordering, return order, split points, argument names) and
-  the adaLN-"Zero" identity property (zero modulation weights => block is the
-  identity on the residual stream).
+  ``CogVideoXLayerNormZero`` and of the reference's processors; the two agree
+  to fp32 round-off, and each of some thirty plausible wiring mistakes (shift
+  and scale swapped, gate chunks swapped, eps 1e-5 <-> 1e-6, scale-first <->
+  shift-first, affine dropped, joint order flipped, text bias kept, wrong norm
+  weights, rotation missing or on the wrong rows) breaks the agreement.  Also
+  pinned: the adaLN-"Zero" identity (zero modulation weights => block is the
+  identity on the residual stream), return orders and split points fixed by
+  the reference's call sites, patch mode with a fresh buffer = rows of the full
+  pass (``tests/test_oracle_blocks.py``).  What no test here can confirm is
+  that the published diffusers modules are what the package a deployment
+  installs really computes: diffusers (``setup.py:27``, ``>=0.31``, no upper
+  pin) is neither under ``/root/reference`` nor installed, and the reference
+  holds no golden vectors.
 * head and tail of a step (``oracle/step.py``): patch embedding -- ``F.conv2d``;
   unpatchify -- ``F.fold`` and index checks; timestep projection and the 2-D
   sin-cos table -- closed forms; conditioning embedders and ``norm_out`` +
