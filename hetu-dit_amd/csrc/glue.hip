@@ -514,6 +514,8 @@ extern "C" __attribute__((visibility("default"))) int hdit_qk_norm_rope(const hd
     if (!aligned16(j.weight) || !aligned16(j.bias) || !aligned16(j.cos_table) || !aligned16(j.sin_table))
       return HDIT_EINVAL;
     if (j.cos_table && !j.sin_table) return HDIT_EINVAL;
+    // the table must cover every row from rope_row0 on: a short table would leave rows silently unrotated
+    if (j.cos_table && (j.rope_row0 < 0 || j.seq - j.rope_row0 > j.rope_rows)) return HDIT_EINVAL;
     tab.j[i] = j;
     int64_t nv = (int64_t)batch * j.seq * heads;
     if (nv > max_vec) max_vec = nv;

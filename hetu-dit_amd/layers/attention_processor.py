@@ -52,17 +52,24 @@ class _PackedProjection:
     tensor; if someone re-assigns ``.data`` the pack is rebuilt on next use."""
 
     def __init__(self, layers: List[nn.Linear]):
+        if len({l.bias is None for l in layers}) != 1:
+            raise ValueError("the layers of one packed projection must all have a bias or all have none")
         self.layers = layers
         self.weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
         self.splits = [l.weight.shape[0] for l in layers]
 
     def _stale(self) -> bool:
+        """True when a weight or a bias no longer is the row slice of the pack it was made (a hot-swap
+        re-assigned its ``.data``)."""
         if self.weight is None:
             return True
         off = 0
         for l, n in zip(self.layers, self.splits):
             if l.weight.data_ptr() != self.weight.data_ptr() + off * self.weight.shape[1] * self.weight.element_size():
+                return True
+            if l.bias is not None and (self.bias is None or
+                                       l.bias.data_ptr() != self.bias.data_ptr() + off * self.bias.element_size()):
                 return True
             off += n
         return False
@@ -348,6 +355,9 @@ class hetuDiTFluxAttnProcessor2_0(FluxAttnProcessor2_0):
         if encoder_hidden_states is not None:
             n_txt = encoder_hidden_states.shape[1]
             N = hidden_states.shape[1]
+            if cos is not None and cos.shape[0] != n_txt + N:
+                raise ValueError(f"image_rotary_emb has {cos.shape[0]} rows, this call's joint [text, image] "
+                                 f"sequence has {n_txt + N}")
             p_img, q_img, kv_img = _qkv_problems(hidden_states, attn._qkv, attn, inner, use_cache=True)
             p_txt, q_txt, kv_txt = _qkv_problems(encoder_hidden_states, attn._add_qkv, attn, inner, use_cache=False)
             ops.gemm_launch(p_img + p_txt)
@@ -378,6 +388,8 @@ class hetuDiTFluxAttnProcessor2_0(FluxAttnProcessor2_0):
         n_txt = get_runtime_state().max_condition_sequence_length
         S = hidden_states.shape[1]
         N = S - n_txt
+        if cos is not None and cos.shape[0] != S:
+            raise ValueError(f"image_rotary_emb has {cos.shape[0]} rows, this call's joint sequence has {S}")
         x2 = _rows2d(hidden_states)
         w, b = attn._qkv.get()
         if rng is None:

@@ -395,6 +395,10 @@ def qk_norm_rope_job(x: torch.Tensor, norm_kind: int = 0, weight=None, bias=None
         _need(cos, torch.float32, "cos"), _need(sin, torch.float32, "sin")
         if cos.shape != sin.shape or cos.shape[1] != x.shape[3] or not (cos.is_contiguous() and sin.is_contiguous()):
             raise ValueError("cos/sin must be contiguous f32 [rows, head_dim]")
+        if cos.shape[0] != x.shape[1] - rope_row0:
+            # the reference's `x * cos` would fail to broadcast; a silent partial rotation must not happen
+            raise ValueError(f"rotary table has {cos.shape[0]} rows for {x.shape[1] - rope_row0} rotated tokens "
+                             f"(sequence {x.shape[1]}, first rotated row {rope_row0})")
         j.cos_table, j.sin_table = cos.data_ptr(), sin.data_ptr()
         j.rope_row0, j.rope_rows = rope_row0, cos.shape[0]
     j._keep = (x, weight, bias, cos, sin)

@@ -212,7 +212,8 @@ int hdit_gelu_tanh(const void* x, const void* bias, void* y, int64_t rows, int d
  *   norm_kind 0: none; 1: RMSNorm(eps, weight); 2: LayerNorm(eps, weight, bias)
  *   then, for rows s in [rope_row0, rope_row0 + rope_rows):
  *   out = x*cos[s - rope_row0] + rotate_pairs(x)*sin[s - rope_row0]  (fp32 math)
- * cos/sin f32 [rope_rows, head_dim] (NULL => no rotation).  Up to 4 jobs per
+ * cos/sin f32 [rope_rows, head_dim] (NULL => no rotation); rope_rows must cover
+ * seq - rope_row0 rows (HDIT_EINVAL otherwise).  Up to 4 jobs per
  * launch.  Replaces attn.norm_q/norm_k/norm_added_q/norm_added_k and
  * apply_rotary_emb at attention_processor.py:68-120,:859-905,:1069-1082. */
 typedef struct hdit_qknorm_job {

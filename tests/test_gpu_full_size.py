@@ -160,3 +160,34 @@ def test_sd3_stack_full_size_properties(hdit):
     out = stack(x, e, t)
     torch.cuda.synchronize()
     assert torch.equal(out, x)
+
+
+def test_attention_fp8_full_size_cogvideox(hdit):
+    """configs[4]'s fp8 leg at its real length: 48 heads, 226 text + 17550 video tokens (17776 keys).  Sampled
+    query rows against the fp32 oracle at the kernel-level fp8 bound (zero-mean random V: nothing averages the
+    e4m3 rounding of V and P away relative to the signal), and a V that is the same for every key and exactly
+    representable in e4m3: the output must then be V itself, which holds only if the row sum is taken over the
+    same rounded probabilities the P.V product consumes -- a mismatch between the two grows with the number of
+    keys."""
+    print("attention fp8 full size 1x48x17776 d64", flush=True)
+    ops = hdit.ops
+    B, H, n_txt, n_img, hd = 1, 48, 226, 17550, 64
+    S = n_txt + n_img
+    q, k, v = dev_randn((B, S, H, hd), 1), dev_randn((B, S, H, hd), 2), dev_randn((B, S, H, hd), 3)
+    (o,) = ops.attention([q], [k], [v], fp8=True)
+    torch.cuda.synchronize()
+    rows = sample_rows(S, 24, 7)
+    for h in (0, 17, H - 1):
+        want = O.attention(q[0, rows.to(DEV), h].float().cpu()[None, None], k[0, :, h].float().cpu()[None, None],
+                           v[0, :, h].float().cpu()[None, None])[0, 0]
+        assert_parity(o[0, rows.to(DEV), h], want, rel=6e-2, cos=0.998, what=f"fp8 attention rows, head {h}")
+    # constant, e4m3-representable V (absmax 1 maps to 448 = 1.75 * 2^8; +-1, +-0.5, +-0.25 stay exact)
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    vals = torch.tensor([1.0, -1.0, 0.5, -0.5, 0.25, -0.25], device=DEV)
+    const = vals[torch.randint(0, 6, (B, 1, H, hd), generator=gen, device=DEV)].to(torch.bfloat16)
+    const[..., 0] = 1.0  # every head's absmax is 1
+    (oc,) = ops.attention([q], [k], [const.expand(B, S, H, hd).contiguous()], fp8=True)
+    torch.cuda.synchronize()
+    err = (oc.float() - const.float()).abs().max().item()
+    print(f"constant V: max |out - V| = {err:.3e}", flush=True)
+    assert err <= 2.0 ** -8, f"softmax weights do not sum to one over {S} keys: max |out - V| = {err:.3e}"

@@ -135,6 +135,75 @@ def test_packed_projection_views_and_repack():
     assert w2.data_ptr() != w.data_ptr() and torch.all(w2[4:8] == 7.0)
     wq, bq = pk.rows(4, 4)
     assert torch.all(wq == 7.0) and bq.shape == (4,)
+    # a bias alone re-assigned: the packed bias must follow
+    c.bias.data = torch.full((6,), 3.0)
+    _, b3 = pk.get()
+    assert torch.all(b3[8:] == 3.0) and c.bias.data_ptr() == b3[8:].data_ptr()
+    with pytest.raises(ValueError, match="all have a bias"):
+        _PackedProjection([nn.Linear(8, 4), nn.Linear(8, 4, bias=False)])
+
+
+def test_wrap_layers_and_register_cache_follow_the_reference_rules():
+    """``_wrap_layers`` + ``_register_cache`` of the reference (models/base_model.py:59-112,:162-178) on the
+    stand-in classes: children are wrapped by *name* ("attn") or by *class* (FeedForward), constructed through
+    the registry, and the K/V cache entry is keyed by the attention *wrapper* -- the object the processors
+    later pass as ``layer=attn``."""
+    from hetu_dit_amd.base_model import register_cache, wrap_layers
+    from hetu_dit_amd.cache_manager import get_cache_manager, reset_cache_manager
+    from hetu_dit_amd.layers.attention_processor import hetuDiTAttentionWrapper, hetuDiTJointAttnProcessor2_0
+    from hetu_dit_amd.layers.feedforward import hetuDiTFeedForwardWrapper
+    from hetu_dit_amd.layers.modules import Attention, FeedForward, JointAttnProcessor2_0
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.attn = Attention(64, 2, 32, added_kv_proj_dim=64, context_pre_only=False, bias=True,
+                                  processor=JointAttnProcessor2_0())
+            self.ff = FeedForward(64)
+            self.other = nn.Linear(64, 64)
+
+    class Model(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.transformer_blocks = nn.ModuleList([Block(), Block()])
+
+    reset_cache_manager()
+    model = Model()
+    raw_attn = model.transformer_blocks[0].attn
+    wrapped = wrap_layers(model, submodule_classes_to_wrap=[FeedForward], submodule_name_to_wrap=["attn"])
+    assert len(wrapped) == 4
+    blk = model.transformer_blocks[0]
+    assert isinstance(blk.attn, hetuDiTAttentionWrapper) and blk.attn.module is raw_attn
+    assert isinstance(blk.ff, hetuDiTFeedForwardWrapper) and isinstance(blk.other, nn.Linear)
+    assert isinstance(blk.attn.processor, hetuDiTJointAttnProcessor2_0)
+    # parameter paths gain the .module hop; re-homed biases live on the wrapper
+    names = dict(model.named_parameters())
+    assert "transformer_blocks.0.attn.module.to_q.weight" in names
+    assert "transformer_blocks.0.attn.output_bias" in names and "transformer_blocks.1.ff.output_bias" in names
+    cm = get_cache_manager()
+    assert not cm.cache
+    register_cache(wrapped)
+    assert set(cm.cache) == {("attn", b.attn) for b in model.transformer_blocks}
+    cm._entry(blk.attn, "attn")  # the wrapper is the key
+    with pytest.raises(KeyError):
+        cm._entry(blk.attn.module, "attn")
+    # wrapping again leaves wrappers alone
+    assert wrap_layers(model, [FeedForward], ["attn"]) == []
+    reset_cache_manager()
+
+
+def test_patch_embed_height_from_input_config():
+    """The patch-embedding wrapper takes the whole image's latent rows from input_config.height //
+    vae_scale_factor like the reference (layers/embeddings.py:33-36), else from set_patches."""
+    from hetu_dit_amd.runtime_state import reset_runtime_state
+
+    rs = reset_runtime_state()
+    assert rs.whole_image_latent_rows() == 0
+    rs.set_patches(latents_height=128, latents_width=128, patch_size=2, num_pipeline_patch=4)
+    assert rs.whole_image_latent_rows() == 128
+    rs.set_input_parameters(height=512, width=512, vae_scale_factor=8)
+    assert rs.whole_image_latent_rows() == 64
+    reset_runtime_state()
 
 
 def test_ops_refuse_cpu_tensors():
