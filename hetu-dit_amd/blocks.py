@@ -145,7 +145,12 @@ class JointTransformerBlock(nn.Module):
             self.ff_context = None
 
     @torch.no_grad()
-    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor):
+    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
+                skip_text_output: bool = False):
+        """``skip_text_output``: the caller drops this block's text output (the SD3 block loop does for every
+        pipeline patch after the first, ``transformer_sd3.py:131-146``), so the text stream stops after its
+        q|k|v projection -- no out-projection, ``norm2_context`` or ``ff_context`` -- and ``None`` is returned
+        for it.  The image output is unchanged bit for bit."""
         eps = 1e-6
         sh_a, sc_a, g_a, sh_m, sc_m, g_m = _adaln(self.norm1, temb)
         if self.context_pre_only:
@@ -155,9 +160,10 @@ class JointTransformerBlock(nn.Module):
         else:
             c_sh_a, c_sc_a, c_g_a, c_sh_m, c_sc_m, c_g_m = _adaln(self.norm1_context, temb)
             n, nc = ops.layernorm_modulate_many([(hidden_states, sh_a, sc_a), (encoder_hidden_states, c_sh_a, c_sc_a)], eps)
-            hidden, encoder = self.attn.forward_gated(n, nc, hidden_states, g_a, encoder_hidden_states, c_g_a)
+            hidden, encoder = self.attn.forward_gated(n, nc, hidden_states, g_a, encoder_hidden_states, c_g_a,
+                                                      skip_txt=skip_text_output)
         # between the two residuals of a block the stream is always fp32
-        if self.context_pre_only:
+        if self.context_pre_only or skip_text_output:
             n2 = ops.layernorm_modulate(hidden, sh_m, sc_m, eps)
             hidden, _ = _mlp_both_streams(self.ff, _rows2d(n2), hidden, g_m, out_dtype=self.stream_dtype)
             return None, hidden

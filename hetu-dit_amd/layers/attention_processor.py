@@ -190,7 +190,8 @@ class hetuDiTAttentionWrapper(hetuDiTAttentionBaseWrapper):
         self._proc_params = set(inspect.signature(self.processor.__call__).parameters.keys())
 
     # -- out-projection as GEMM problems (optionally with the gated residual) ------
-    def out_proj_problems(self, o_img, o_txt, resid_img=None, gate_img=None, resid_txt=None, gate_txt=None):
+    def out_proj_problems(self, o_img, o_txt, resid_img=None, gate_img=None, resid_txt=None, gate_txt=None,
+                          skip_txt: bool = False):
         """Problems for ``to_out[0]`` (+ ``output_bias``) and ``to_add_out``
         (+ ``encoder_output_bias`` unless ``encoder_bias`` is off for this
         family).  With ``resid``/``gate`` the epilogue is the gated residual and
@@ -212,7 +213,7 @@ class hetuDiTAttentionWrapper(hetuDiTAttentionBaseWrapper):
             outs.append(out)
 
         one(o_img, m.to_out[0].weight.data, self.output_bias.data if self.has_output_bias else None, resid_img, gate_img)
-        if o_txt is not None and not m.context_pre_only and getattr(m, "to_add_out", None) is not None:
+        if o_txt is not None and not skip_txt and not m.context_pre_only and getattr(m, "to_add_out", None) is not None:
             bias = None
             if self.has_encoder_output_bias and self.processor.adds_encoder_output_bias:
                 bias = self.encoder_output_bias.data
@@ -253,14 +254,15 @@ class hetuDiTAttentionWrapper(hetuDiTAttentionBaseWrapper):
         return outs[0], o_txt  # context_pre_only: raw attention slice (attention_processor.py:420-421)
 
     def forward_gated(self, hidden_states, encoder_hidden_states, resid_img, gate_img, resid_txt=None, gate_txt=None,
-                      **kwargs):
+                      skip_txt: bool = False, **kwargs):
         """``resid + gate * attn(...)`` for both streams with the gated residual
         fused into the out-projection epilogue (what the diffusers block does
         with the wrapper's outputs right after the call).  Returns
-        ``(hidden_new, encoder_new_or_None)``."""
+        ``(hidden_new, encoder_new_or_None)``.  ``skip_txt`` leaves the text
+        stream's out-projection out (its result would be dropped by the caller)."""
         kwargs = {k: v for k, v in kwargs.items() if k in self._proc_params}
         o_img, o_txt = self.processor(self, hidden_states, encoder_hidden_states=encoder_hidden_states, **kwargs)
-        problems, outs = self.out_proj_problems(o_img, o_txt, resid_img, gate_img, resid_txt, gate_txt)
+        problems, outs = self.out_proj_problems(o_img, o_txt, resid_img, gate_img, resid_txt, gate_txt, skip_txt=skip_txt)
         ops.gemm_launch(problems)
         return outs[0], (outs[1] if len(outs) == 2 else None)
 

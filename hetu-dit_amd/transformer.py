@@ -45,8 +45,10 @@ class SD3TransformerBlocks(nn.Module):
                     hidden_states=hidden_states, encoder_hidden_states=encoder_hidden_states, temb=temb
                 )
             elif rs.patch_mode:
+                # the text output of these calls is dropped: the block does not compute it
                 _, hidden_states = block(
-                    hidden_states=hidden_states, encoder_hidden_states=self.encoder_hidden_states_cache[i], temb=temb
+                    hidden_states=hidden_states, encoder_hidden_states=self.encoder_hidden_states_cache[i], temb=temb,
+                    skip_text_output=True,
                 )
             else:
                 encoder_hidden_states, hidden_states = block(

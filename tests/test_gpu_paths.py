@@ -262,3 +262,59 @@ def test_block_called_alone_after_a_stack_run_uses_its_own_temb(hdit):
     o_enc, o_hid = oracle.sd3_joint_block(params, x.float(), e.float(), t2.float(), H)
     assert_parity(hid, o_hid, what=f"block alone with a new temb (address reused: {same_address})")
     assert_parity(enc, o_enc, what="block alone with a new temb, encoder")
+
+
+def test_sd3_patches_skip_the_dropped_text_stream_bit_exact(hdit):
+    """For pipeline patches after the first the block loop drops every block's text output
+    (transformer_sd3.py:131-146); the runner therefore asks the blocks not to compute it.  The image output of
+    every patch must equal, bit for bit, what the same blocks return when they do compute the text stream."""
+    from hetu_dit_amd import synthetic, transformer
+    from hetu_dit_amd.cache_manager import get_cache_manager
+    from hetu_dit_amd.runtime_state import get_runtime_state
+
+    B, N, Nt, D, H, L, P = 2, 1024, 333, 512, 8, 3, 4
+    starts = [N // P * i for i in range(P + 1)]
+    stack = transformer.SD3TransformerBlocks(L, D, H, 64)
+    synthetic.init_module_(stack, 101)
+    stack = stack.to(DEV)
+    x_prev, x_now = synthetic.randn_bf16((B, N, D), 102).to(DEV), synthetic.randn_bf16((B, N, D), 103).to(DEV)
+    e, t = synthetic.randn_bf16((B, Nt, D), 104).to(DEV), synthetic.randn_bf16((B, D), 105).to(DEV)
+    rs = get_runtime_state()
+    rs.set_token_patches(starts)
+    rs.set_patched_mode(False)
+    stack(x_prev, e, t)
+    torch.cuda.synchronize()
+    saved = {k: [None if b is None else b.clone() for b in v.tensors] for k, v in get_cache_manager().cache.items()}
+
+    def full_text_pass(p):
+        """the reference's loop: every block computes both streams, the text output is dropped for p > 0"""
+        hid, enc = x_now[:, starts[p]:starts[p + 1]].contiguous(), e
+        for i, blk in enumerate(stack.transformer_blocks):
+            if p == 0:
+                enc_cache[i] = enc
+                enc, hid = blk(hidden_states=hid, encoder_hidden_states=enc, temb=t)
+            else:
+                _, hid = blk(hidden_states=hid, encoder_hidden_states=enc_cache[i], temb=t)
+        return hid
+
+    rs.set_patched_mode(True)
+    enc_cache = [None] * L
+    want = []
+    for p in range(P):
+        want.append(full_text_pass(p).clone())
+        rs.next_patch()
+    torch.cuda.synchronize()
+    for k, v in get_cache_manager().cache.items():  # back to the buffers of the previous step
+        for dst, src in zip(v.tensors, saved[k]):
+            if dst is not None:
+                dst.copy_(src)
+    rs.set_patched_mode(True)
+    for p in range(P):
+        got = stack(x_now[:, starts[p]:starts[p + 1]].contiguous(), e, t)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want[p]), f"patch {p}: skipping the text stream changed the image output"
+        rs.next_patch()
+    # and a block asked to skip it returns None for the text stream
+    enc, hid = stack.transformer_blocks[0](hidden_states=x_now[:, :starts[1]].contiguous(), encoder_hidden_states=e, temb=t,
+                                           skip_text_output=True)
+    assert enc is None and hid.shape == (B, starts[1], D)
