@@ -119,9 +119,12 @@ def make_workload(name, dev):
             return out
 
         L = cfg["layers"]
-        Sq = Ni // P + Nt
-        gemm = (24.0 * Sq * D * D * B * L - 18.0 * Nt * D * D * B) * P
-        attn = 4.0 * Sq * S * D * B * L * P
+        Np = Ni // P
+        Sq = Np + Nt
+        # patch 0 runs both streams; the block loop drops the text output of patches 1..P-1, for which the text
+        # stream only supplies keys and values (k|v projection, no query rows, no out-projection, no MLP)
+        gemm = (24.0 * Sq * D * D * B * L - 18.0 * Nt * D * D * B) + (P - 1) * (24.0 * Np + 4.0 * Nt) * D * D * B * L
+        attn = 4.0 * Sq * S * D * B * L + (P - 1) * 4.0 * Np * S * D * B * L
         desc = ("configs[3]: SD3 PipeFusion shard, 24 joint blocks x 4 patches, B2, query 1024 image + 333 text tokens "
                 "against the 4096 + 333 stale K/V buffer")
         return step, desc, gemm, attn, L * P, "attn_fwd_kernel<64>"

@@ -261,6 +261,8 @@ class hetuDiTAttentionWrapper(hetuDiTAttentionBaseWrapper):
         ``(hidden_new, encoder_new_or_None)``.  ``skip_txt`` leaves the text
         stream's out-projection out (its result would be dropped by the caller)."""
         kwargs = {k: v for k, v in kwargs.items() if k in self._proc_params}
+        if skip_txt and "skip_text_queries" in self._proc_params:
+            kwargs["skip_text_queries"] = True
         o_img, o_txt = self.processor(self, hidden_states, encoder_hidden_states=encoder_hidden_states, **kwargs)
         problems, outs = self.out_proj_problems(o_img, o_txt, resid_img, gate_img, resid_txt, gate_txt, skip_txt=skip_txt)
         ops.gemm_launch(problems)
@@ -282,16 +284,33 @@ class hetuDiTJointAttnProcessor2_0(JointAttnProcessor2_0):
         super().__init__()
         self.use_long_ctx_attn_kvcache = HAS_LONG_CTX_ATTN and get_sequence_parallel_world_size() > 1
 
-    def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, *args, **kwargs):
+    def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, *args,
+                 skip_text_queries: bool = False, **kwargs):
+        """``skip_text_queries``: the caller drops the text rows of the attention output (the SD3 block loop
+        does for pipeline patches after the first), so the text stream only contributes keys and values: its
+        q projection and its query rows are left out and ``None`` is returned for them."""
         H = attn.heads_per_device
         inner = attn.module.to_k.weight.shape[0]
         p_img, q_img, kv_img = _qkv_problems(hidden_states, attn._qkv, attn, inner, use_cache=True)
-        p_txt, q_txt, kv_txt = _qkv_problems(encoder_hidden_states, attn._add_qkv, attn, inner, use_cache=False)
-        ops.gemm_launch(p_img + p_txt)
         B, N, _ = hidden_states.shape
         Nt = encoder_hidden_states.shape[1]
-        o_img = torch.empty(B, N, inner, dtype=torch.bfloat16, device=hidden_states.device)
-        o_txt = torch.empty(B, Nt, inner, dtype=torch.bfloat16, device=hidden_states.device)
+        dev = hidden_states.device
+        o_img = torch.empty(B, N, inner, dtype=torch.bfloat16, device=dev)
+        if skip_text_queries:
+            wkv, bkv = attn._add_qkv.rows(inner, 2 * inner)
+            kv_txt = torch.empty(B, Nt, 2 * inner, dtype=torch.bfloat16, device=dev)
+            ops.gemm_launch(p_img + [ops.gemm_problem(_rows2d(encoder_hidden_states), wkv, kv_txt.view(-1, 2 * inner), bkv)])
+            ops.attention(
+                [_heads(q_img, H)],
+                [_heads(kv_img[:, :, :inner], H), _heads(kv_txt[:, :, :inner], H)],
+                [_heads(kv_img[:, :, inner:], H), _heads(kv_txt[:, :, inner:], H)],
+                out=[_heads(o_img, H)],
+                fp8=getattr(attn, "fp8_attention", False),
+            )
+            return o_img, None
+        p_txt, q_txt, kv_txt = _qkv_problems(encoder_hidden_states, attn._add_qkv, attn, inner, use_cache=False)
+        ops.gemm_launch(p_img + p_txt)
+        o_txt = torch.empty(B, Nt, inner, dtype=torch.bfloat16, device=dev)
         ops.attention(
             [_heads(q_img, H), _heads(q_txt, H)],
             [_heads(kv_img[:, :, :inner], H), _heads(kv_txt[:, :, :inner], H)],
