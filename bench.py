@@ -57,7 +57,8 @@ def randomize_(module, device, seed=0):
     return module
 
 
-WORKLOADS = ("sd3_1024", "sd3_1024_transformer", "sd3_pipefusion", "flux_1024", "cogvideox_5b")
+WORKLOADS = ("sd3_1024", "sd3_1024_transformer", "sd3_pipefusion", "flux_1024", "cogvideox_5b", "sd3_1024_fp8",
+             "cogvideox_5b_fp8")
 
 
 def make_workload(name, dev):
@@ -72,6 +73,17 @@ def make_workload(name, dev):
     reset_runtime_state()
     gen = torch.Generator(device=dev).manual_seed(1)
     rnd = lambda *shape: torch.randn(*shape, generator=gen, device=dev).to(torch.bfloat16)
+    if name.endswith("_fp8"):
+        # the same blocks with the attention on the fp8-e4m3 path (per-(batch, head) absmax scales)
+        from hetu_dit_amd.layers.attention_processor import hetuDiTAttentionWrapper
+
+        step, desc, gemm, attn, blocks, kernel = make_workload(name[:-4], dev)
+        for obj in (c.cell_contents for c in step.__closure__):
+            if isinstance(obj, torch.nn.Module):
+                for m in obj.modules():
+                    if isinstance(m, hetuDiTAttentionWrapper):
+                        m.fp8_attention = True
+        return step, desc + "; attention on the fp8-e4m3 path", gemm, attn, blocks, kernel.replace("attn_fwd_kernel", "attn_fp8_kernel")
     if name == "sd3_1024_transformer":
         # the same 24 blocks inside the whole transformer: latent in, guided and Euler-updated latent out
         from hetu_dit_amd.transformer_sd3 import SD3Transformer2DModel
@@ -288,7 +300,11 @@ def main():
         return n, ms, work
 
     n_g, ms_g, fl_g = per_class("gemm")
-    n_a, ms_a, fl_a = per_class("attn_bf16")
+    fp8 = args.workload.endswith("_fp8")
+    n_a, ms_a, fl_a = per_class("attn_fp8" if fp8 else "attn_bf16")
+    attn_peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
+    if fp8:  # the fp8 path's own passes count as attention time: absmax of q, k, v and the K / V quantisation
+        ms_a += per_class("attn_absmax")[1]
     gemm_tflops = fl_g / ms_g / 1e9 if ms_g else 0.0
     attn_tflops = fl_a / ms_a / 1e9 if ms_a else 0.0
     glue = {}
@@ -335,7 +351,7 @@ def main():
         },
         "roofline_attention": {
             "kernel": attn_kernel + " (joint flash attention)", "bound": "mfma", "achieved": round(attn_tflops, 1),
-            "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
+            "peak": attn_peak, "unit": "TFLOP/s", "frac": round(attn_tflops / attn_peak, 4),
             "traffic": ATTN_TRAFFIC_BYTES_PER_LAUNCH if headline else None, "launches_per_step": n_a // 3, "avg_launch_us": round(ms_a / max(n_a, 1) * 1e3, 2),
             "flops_per_launch": round(fl_a / max(n_a, 1), 1),
         },

@@ -88,12 +88,28 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
       for (int e = 0; e < 4; e++) w[h * 4 + e] = v[e];
     }
   };
+  // modulation vectors of the batch element the current row belongs to, kept in registers across the wave's
+  // rows and requested before the row statistics are reduced, so that they arrive under the reductions
+  float msc[NCH][EPC], msh[NCH][EPC];
+  int64_t mod_b = -1;
   load(0, row0);
 #pragma unroll
   for (int r = 0; r < RPW; r++) {
     const int64_t row = row0 + r;
     if (row >= rows) break;
     if (r + 1 < RPW && row + 1 < rows) load(r + 1, row + 1);
+    const int64_t b = row / tokens;
+    if (b != mod_b) {
+      mod_b = b;
+#pragma unroll
+      for (int i = 0; i < NCH; i++) {
+        int c = lane + i * 64;
+        if (c < nchunks) {
+          if (scale) load_f32(scale + b * mod_stride, c, msc[i]);
+          if (shift) load_f32(shift + b * mod_stride, c, msh[i]);
+        }
+      }
+    }
     float s = 0.f;
     float f[NCH][EPC];
 #pragma unroll
@@ -119,9 +135,6 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
       }
     }
     const float rstd = rsqrtf(wave_sum(q) * inv_d + eps);
-    const int64_t b = row / tokens;
-    const float* sh = shift ? shift + b * mod_stride : nullptr;
-    const float* sc = scale ? scale + b * mod_stride : nullptr;
     __bf16* yr = y + b * y_sb + (row - b * tokens) * y_st;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
@@ -140,15 +153,13 @@ __global__ void __launch_bounds__(256) ln_modulate_kernel(const LnJobs jobs, con
 #pragma unroll
           for (int e = 0; e < EPC; e++) o[e] += w[e];
         }
-        if (sc) {
-          load_f32(sc, c, w);
+        if (scale) {
 #pragma unroll
-          for (int e = 0; e < EPC; e++) o[e] *= 1.0f + w[e];
+          for (int e = 0; e < EPC; e++) o[e] *= 1.0f + msc[i][e];
         }
-        if (sh) {
-          load_f32(sh, c, w);
+        if (shift) {
 #pragma unroll
-          for (int e = 0; e < EPC; e++) o[e] += w[e];
+          for (int e = 0; e < EPC; e++) o[e] += msh[i][e];
         }
         if constexpr (XF32) {
           i32x2 pk = {(int)hdit::pack2(o[0], o[1]), (int)hdit::pack2(o[2], o[3])};
