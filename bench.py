@@ -23,10 +23,26 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
-# HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes summarised in
-# profiles/sd3_1024_step_hbm_traffic.txt (hardware counters cannot be read from inside this process)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 344.7e6
-ATTN_TRAFFIC_BYTES_PER_LAUNCH = 185.6e6
+
+
+def profiled_traffic():
+    """HBM-side bytes per launch of the grouped GEMM and of the attention kernel in the headline workload, as
+    summarised in profiles/sd3_1024_step_hbm_traffic.txt from two `rocprofv3 --pmc` passes (FETCH_SIZE, WRITE_SIZE;
+    hardware counters cannot be read from inside this process).  (None, None) when the summary is absent."""
+    path = os.path.join(ROOT, "profiles", "sd3_1024_step_hbm_traffic.txt")
+    gemm = attn = None
+    try:
+        for line in open(path):
+            if line.startswith("# bench.py reads:"):
+                for item in line.split(":", 1)[1].split():
+                    key, _, val = item.partition("=")
+                    if key == "gemm_bytes_per_call":
+                        gemm = float(val)
+                    elif key == "attn_bytes_per_launch":
+                        attn = float(val)
+    except OSError:
+        pass
+    return gemm, attn
 
 
 def build_stack(cfg, device, seed=0):
@@ -299,6 +315,7 @@ def main():
         n, ms, work = summ.get(kind, (0, 0.0, 0.0))
         return n, ms, work
 
+    gemm_traffic, attn_traffic = profiled_traffic()
     n_g, ms_g, fl_g = per_class("gemm")
     fp8 = args.workload.endswith("_fp8")
     n_a, ms_a, fl_a = per_class("attn_fp8" if fp8 else "attn_bf16")
@@ -343,16 +360,17 @@ def main():
         "roofline": {
             "kernel": "gemm_kernel (grouped bf16 MFMA GEMM, all projection/MLP launches of the step)",
             "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if headline else None,
-            "traffic_note": "rocprofv3 FETCH_SIZE x2.0 + WRITE_SIZE x1.0 (factors from a 256 MiB copy), mean over the "
-                            "step's hdit_gemm_bf16 calls; algorithmic operand+result bytes average 86.6 MB per call",
+            "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": gemm_traffic if headline else None,
+            "traffic_note": "from profiles/sd3_1024_step_hbm_traffic.txt: rocprofv3 FETCH_SIZE and WRITE_SIZE, each scaled "
+                            "by what the counter reads for a 256 MiB copy, mean over the step's hdit_gemm_bf16 calls; "
+                            "algorithmic operand + residual + result bytes average 177.9 MB per call (activations of both streams, both weight sets, fp32 residual stream)",
             "launches_per_step": n_g // 3, "avg_launch_us": round(ms_g / max(n_g, 1) * 1e3, 2),
             "flops_per_launch": round(fl_g / max(n_g, 1), 1),
         },
         "roofline_attention": {
             "kernel": attn_kernel + " (joint flash attention)", "bound": "mfma", "achieved": round(attn_tflops, 1),
             "peak": attn_peak, "unit": "TFLOP/s", "frac": round(attn_tflops / attn_peak, 4),
-            "traffic": ATTN_TRAFFIC_BYTES_PER_LAUNCH if headline else None, "launches_per_step": n_a // 3, "avg_launch_us": round(ms_a / max(n_a, 1) * 1e3, 2),
+            "traffic": attn_traffic if headline else None, "launches_per_step": n_a // 3, "avg_launch_us": round(ms_a / max(n_a, 1) * 1e3, 2),
             "flops_per_launch": round(fl_a / max(n_a, 1), 1),
         },
         "roofline_glue": glue,
