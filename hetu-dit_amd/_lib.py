@@ -96,6 +96,31 @@ class LnJob(C.Structure):
     ]
 
 
+class Sd3BlockWeights(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in (
+        "norm1_w", "norm1_b", "norm1_context_w", "norm1_context_b", "qkv_w", "qkv_b", "add_qkv_w", "add_qkv_b",
+        "to_out_w", "to_out_b", "to_add_out_w", "to_add_out_b", "ff_in_w", "ff_in_b", "ff_out_w", "ff_out_b",
+        "ff_context_in_w", "ff_context_in_b", "ff_context_out_w", "ff_context_out_b")]
+
+
+class Sd3BlockArgs(C.Structure):
+    _fields_ = [
+        ("w", Sd3BlockWeights),
+        ("hidden", C.c_void_p),
+        ("encoder", C.c_void_p),
+        ("temb", C.c_void_p),
+        ("hidden_out", C.c_void_p),
+        ("encoder_out", C.c_void_p),
+        ("modulation_img", C.c_void_p),
+        ("modulation_txt", C.c_void_p),
+        ("kv_buffer", C.c_void_p),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_int64),
+    ] + [(n, C.c_int32) for n in (
+        "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "kv_rows", "kv_row0", "hidden_f32",
+        "encoder_f32", "out_f32", "context_pre_only", "skip_text_output")]
+
+
 # name -> (restype, argtypes); every symbol include/hdit.h declares
 SIGNATURES = {
     "hdit_abi_version": (C.c_int, []),
@@ -106,6 +131,8 @@ SIGNATURES = {
     "hdit_attn_fp8_workspace_bytes": (C.c_int64, [C.POINTER(AttnArgs)]),
     "hdit_attn_fwd_fp8": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p, C.c_void_p]),
     "hdit_attn_fwd_fp8_static": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p]),
+    "hdit_block_sd3_workspace_bytes": (C.c_int64, [C.POINTER(Sd3BlockArgs)]),
+    "hdit_block_sd3": (C.c_int, [C.POINTER(Sd3BlockArgs), C.c_void_p]),
     "hdit_layernorm_modulate": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,

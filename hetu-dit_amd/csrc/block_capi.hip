@@ -1,0 +1,247 @@
+// Whole-block entry points of the C ABI: the composition of the kernels that the Python blocks
+// (hetu_dit_amd/blocks.py) make, for hosts that are not Python.  Pure host code: every step is one of the
+// library's own entry points, enqueued on the caller's stream, with the intermediates in a caller workspace.
+#include <string.h>
+
+#include "hdit_common.h"
+
+namespace {
+
+constexpr int64_t ALIGN = 256;
+int64_t up(int64_t x) { return (x + ALIGN - 1) / ALIGN * ALIGN; }
+
+// Carves the workspace of one SD3 joint block; with base == nullptr it only measures.
+struct Sd3Workspace {
+  float* emb_img;   // [B, 6D]
+  float* emb_txt;   // [B, 6D] (context_pre_only: [B, 2D])
+  unsigned char* n_img;    // bf16 [B, Ni, D]: norm1 output, later norm2 output
+  unsigned char* n_txt;    // bf16 [B, Nt, D]
+  unsigned char* qkv_img;  // bf16 [B, Ni, 3D] (stale K/V buffer given: q only, [B, Ni, D])
+  unsigned char* qkv_txt;  // bf16 [B, Nt, 3D] (text output skipped: k|v only, [B, Nt, 2D])
+  unsigned char* o_img;    // bf16 [B, Ni, D]
+  unsigned char* o_txt;    // bf16 [B, Nt, D]
+  float* x1_img;           // f32 [B, Ni, D]: stream after the attention residual
+  float* x1_txt;           // f32 [B, Nt, D]
+  unsigned char* h_img;    // bf16 [B, Ni, F]
+  unsigned char* h_txt;    // bf16 [B, Nt, F]
+  int64_t bytes;
+};
+
+Sd3Workspace carve(const hdit_sd3_block_args* a, unsigned char* base) {
+  const int64_t B = a->batch, Ni = a->n_img, Nt = a->n_txt, D = a->dim, F = a->ff_dim;
+  const bool text_out = !a->context_pre_only && !a->skip_text_output;
+  Sd3Workspace w;
+  int64_t off = 0;
+  auto take = [&](int64_t nbytes) {
+    unsigned char* p = base ? base + off : nullptr;
+    off += up(nbytes);
+    return p;
+  };
+  w.emb_img = (float*)take(B * 6 * D * 4);
+  w.emb_txt = (float*)take(B * (a->context_pre_only ? 2 : 6) * D * 4);
+  w.n_img = take(B * Ni * D * 2);
+  w.n_txt = take(B * Nt * D * 2);
+  w.qkv_img = take(B * Ni * (a->kv_buffer ? 1 : 3) * D * 2);
+  w.qkv_txt = take(B * Nt * (a->skip_text_output ? 2 : 3) * D * 2);
+  w.o_img = take(B * Ni * D * 2);
+  w.o_txt = take(a->skip_text_output ? 0 : B * Nt * D * 2);
+  w.x1_img = (float*)take(B * Ni * D * 4);
+  w.x1_txt = (float*)take(text_out ? B * Nt * D * 4 : 0);
+  w.h_img = take(B * Ni * F * 2);
+  w.h_txt = take(text_out ? B * Nt * F * 2 : 0);
+  w.bytes = off;
+  return w;
+}
+
+int validate(const hdit_sd3_block_args* a) {
+  if (!a) return HDIT_EINVAL;
+  if (a->batch <= 0 || a->n_img <= 0 || a->n_txt <= 0 || a->dim <= 0 || a->heads <= 0 || a->ff_dim <= 0) return HDIT_EINVAL;
+  if (a->dim % a->heads) return HDIT_EINVAL;
+  const int hd = a->dim / a->heads;
+  if (hd != 64 && hd != 128) return HDIT_EUNSUPPORTED;
+  if (a->dim % 64 || a->ff_dim % 64) return HDIT_EUNSUPPORTED;
+  if (!a->hidden || !a->encoder || !a->temb || !a->hidden_out) return HDIT_EINVAL;
+  const hdit_sd3_block_weights& w = a->w;
+  if (!w.norm1_w || !w.norm1_b || !w.norm1_context_w || !w.norm1_context_b || !w.qkv_w || !w.add_qkv_w || !w.to_out_w ||
+      !w.ff_in_w || !w.ff_out_w)
+    return HDIT_EINVAL;
+  const bool text_out = !a->context_pre_only && !a->skip_text_output;
+  if (text_out && (!a->encoder_out || !w.to_add_out_w || !w.ff_context_in_w || !w.ff_context_out_w)) return HDIT_EINVAL;
+  if (a->kv_buffer && (a->kv_rows < a->n_img || a->kv_row0 < 0 || a->kv_row0 + a->n_img > a->kv_rows)) return HDIT_EINVAL;
+  return HDIT_OK;
+}
+
+hdit_gemm_problem problem(const void* x, int64_t lda, const void* w, const void* bias, void* c, int64_t ldc, int m, int n,
+                          int k, int epilogue) {
+  hdit_gemm_problem p;
+  memset(&p, 0, sizeof(p));
+  p.a = x, p.b = w, p.c = c, p.bias = bias;
+  p.lda = lda, p.ldb = k, p.ldc = ldc;
+  p.m = m, p.n = n, p.k = k;
+  p.epilogue = epilogue;
+  return p;
+}
+
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int64_t hdit_block_sd3_workspace_bytes(const hdit_sd3_block_args* a) {
+  if (validate(a) != HDIT_OK) return -1;
+  return carve(a, nullptr).bytes;
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_sd3_block_args* a, void* stream) {
+  int rc = validate(a);
+  if (rc != HDIT_OK) return rc;
+  if (!a->workspace || (((uintptr_t)a->workspace) & (ALIGN - 1))) return HDIT_EINVAL;
+  const Sd3Workspace ws = carve(a, (unsigned char*)a->workspace);
+  if (a->workspace_bytes < ws.bytes) return HDIT_EINVAL;
+  const hdit_sd3_block_weights& w = a->w;
+  const int B = a->batch, Ni = a->n_img, Nt = a->n_txt, D = a->dim, F = a->ff_dim, H = a->heads, hd = D / H;
+  const bool pre_only = a->context_pre_only != 0;
+  const bool text_out = !pre_only && !a->skip_text_output;
+  const float eps = 1e-6f;
+  const int64_t md = 6 * (int64_t)D;                 // batch stride of the image stream's modulation
+  const int64_t mdt = (pre_only ? 2 : 6) * (int64_t)D;
+  const int sz_in = a->hidden_f32 ? 4 : 2, sz_enc = a->encoder_f32 ? 4 : 2;
+  (void)sz_in, (void)sz_enc;
+
+  // 1. adaLN projections: linear(silu(temb)) for both streams (a caller that already holds them for this temb --
+  //    the projections of all blocks of a stack fit one launch -- passes them in and skips this step)
+  const float* emb_img = a->modulation_img;
+  const float* emb_txt = a->modulation_txt;
+  if (!emb_img) {
+    if ((rc = hdit_adaln_gemv(a->temb, w.norm1_w, w.norm1_b, ws.emb_img, B, 6 * D, a->temb_dim, stream))) return rc;
+    emb_img = ws.emb_img;
+  }
+  if (!emb_txt) {
+    if ((rc = hdit_adaln_gemv(a->temb, w.norm1_context_w, w.norm1_context_b, ws.emb_txt, B, (pre_only ? 2 : 6) * D,
+                              a->temb_dim, stream)))
+      return rc;
+    emb_txt = ws.emb_txt;
+  }
+  // chunks: shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp; AdaLayerNormContinuous: scale, shift
+  const float *sh_a = emb_img, *sc_a = emb_img + D, *g_a = emb_img + 2 * D, *sh_m = emb_img + 3 * D, *sc_m = emb_img + 4 * D,
+              *g_m = emb_img + 5 * D;
+  const float *c_sh_a, *c_sc_a, *c_g_a = nullptr, *c_sh_m = nullptr, *c_sc_m = nullptr, *c_g_m = nullptr;
+  if (pre_only) {
+    c_sc_a = emb_txt, c_sh_a = emb_txt + D;
+  } else {
+    c_sh_a = emb_txt, c_sc_a = emb_txt + D, c_g_a = emb_txt + 2 * D, c_sh_m = emb_txt + 3 * D, c_sc_m = emb_txt + 4 * D,
+    c_g_m = emb_txt + 5 * D;
+  }
+
+  // 2. norm1 + modulate, both streams in one launch
+  hdit_ln_job jobs[2];
+  memset(jobs, 0, sizeof(jobs));
+  jobs[0].x = a->hidden, jobs[0].y = ws.n_img, jobs[0].shift = sh_a, jobs[0].scale = sc_a;
+  jobs[0].x_sb = (int64_t)Ni * D, jobs[0].x_st = D, jobs[0].y_sb = (int64_t)Ni * D, jobs[0].y_st = D, jobs[0].mod_stride = md;
+  jobs[0].batch = B, jobs[0].tokens = Ni, jobs[0].x_f32 = a->hidden_f32;
+  jobs[1].x = a->encoder, jobs[1].y = ws.n_txt, jobs[1].shift = c_sh_a, jobs[1].scale = c_sc_a;
+  jobs[1].x_sb = (int64_t)Nt * D, jobs[1].x_st = D, jobs[1].y_sb = (int64_t)Nt * D, jobs[1].y_st = D, jobs[1].mod_stride = mdt;
+  jobs[1].batch = B, jobs[1].tokens = Nt, jobs[1].x_f32 = a->encoder_f32;
+  if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, nullptr, nullptr, eps, stream))) return rc;
+
+  // 3. q|k|v of both streams in one grouped launch.  With a stale K/V buffer the image stream's k|v rows go
+  //    straight into rows [kv_row0, kv_row0 + n_img) of it, one problem per batch element.
+  hdit_gemm_problem probs[HDIT_GEMM_MAX_PROBLEMS];
+  int np = 0;
+  const unsigned char* qkv_w = (const unsigned char*)w.qkv_w;
+  const unsigned char* qkv_b = (const unsigned char*)w.qkv_b;
+  const unsigned char* aqkv_w = (const unsigned char*)w.add_qkv_w;
+  const unsigned char* aqkv_b = (const unsigned char*)w.add_qkv_b;
+  int64_t q_ld, kv_ld;         // row strides (elements) of the image q and k|v
+  const unsigned char *q_img, *k_img, *v_img;
+  int kv_img_rows;
+  if (!a->kv_buffer) {
+    probs[np++] = problem(ws.n_img, D, qkv_w, qkv_b, ws.qkv_img, 3 * D, B * Ni, 3 * D, D, HDIT_EPI_BIAS);
+    q_ld = kv_ld = 3 * (int64_t)D;
+    q_img = ws.qkv_img, k_img = ws.qkv_img + (int64_t)D * 2, v_img = ws.qkv_img + (int64_t)2 * D * 2;
+    kv_img_rows = Ni;
+  } else {
+    if (B + 2 > HDIT_GEMM_MAX_PROBLEMS) return HDIT_EUNSUPPORTED;
+    probs[np++] = problem(ws.n_img, D, qkv_w, qkv_b, ws.qkv_img, D, B * Ni, D, D, HDIT_EPI_BIAS);
+    unsigned char* kvb = (unsigned char*)a->kv_buffer;
+    for (int b = 0; b < B; b++)
+      probs[np++] = problem(ws.n_img + (int64_t)b * Ni * D * 2, D, qkv_w + (int64_t)D * D * 2, qkv_b ? qkv_b + (int64_t)D * 2 : nullptr,
+                            kvb + ((int64_t)b * a->kv_rows + a->kv_row0) * 2 * D * 2, 2 * D, Ni, 2 * D, D, HDIT_EPI_BIAS);
+    q_ld = D, kv_ld = 2 * (int64_t)D;
+    q_img = ws.qkv_img, k_img = kvb, v_img = kvb + (int64_t)D * 2;
+    kv_img_rows = a->kv_rows;
+  }
+  int64_t tq_ld;
+  const unsigned char *q_txt = nullptr, *k_txt, *v_txt;
+  if (a->skip_text_output) {
+    probs[np++] = problem(ws.n_txt, D, aqkv_w + (int64_t)D * D * 2, aqkv_b ? aqkv_b + (int64_t)D * 2 : nullptr, ws.qkv_txt,
+                          2 * D, B * Nt, 2 * D, D, HDIT_EPI_BIAS);
+    tq_ld = 2 * (int64_t)D;
+    k_txt = ws.qkv_txt, v_txt = ws.qkv_txt + (int64_t)D * 2;
+  } else {
+    probs[np++] = problem(ws.n_txt, D, aqkv_w, aqkv_b, ws.qkv_txt, 3 * D, B * Nt, 3 * D, D, HDIT_EPI_BIAS);
+    tq_ld = 3 * (int64_t)D;
+    q_txt = ws.qkv_txt, k_txt = ws.qkv_txt + (int64_t)D * 2, v_txt = ws.qkv_txt + (int64_t)2 * D * 2;
+  }
+  if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
+
+  // 4. joint attention over [image, text]; image keys / values come from the stale buffer when there is one
+  hdit_attn_args at;
+  memset(&at, 0, sizeof(at));
+  auto seg = [&](hdit_seq_segment& s, const void* p, int64_t rows_per_batch, int64_t ld, int len) {
+    s.ptr = p, s.stride_b = rows_per_batch * ld, s.stride_s = ld, s.stride_h = hd, s.len = len;
+  };
+  seg(at.q[0], q_img, Ni, q_ld, Ni);
+  seg(at.k[0], k_img, kv_img_rows, kv_ld, kv_img_rows);
+  seg(at.v[0], v_img, kv_img_rows, kv_ld, kv_img_rows);
+  seg(at.k[1], k_txt, Nt, tq_ld, Nt);
+  seg(at.v[1], v_txt, Nt, tq_ld, Nt);
+  seg(at.o[0], ws.o_img, Ni, D, Ni);
+  if (!a->skip_text_output) {
+    seg(at.q[1], q_txt, Nt, tq_ld, Nt);
+    seg(at.o[1], ws.o_txt, Nt, D, Nt);
+  }
+  at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
+  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
+
+  // 5. out-projections with the gated residual; the stream stays fp32 inside the block
+  auto gated = [&](hdit_gemm_problem& p, const void* resid, int resid_f32, const float* gate, int64_t gate_stride, int rows,
+                   int out_f32) {
+    p.epilogue = HDIT_EPI_GATE_RESIDUAL | (resid_f32 ? HDIT_EPI_RESID_F32 : 0) | (out_f32 ? HDIT_EPI_OUT_F32 : 0);
+    p.resid = resid, p.ldr = p.n, p.gate = gate, p.gate_stride = (int32_t)gate_stride, p.rows_per_batch = rows;
+  };
+  np = 0;
+  probs[np] = problem(ws.o_img, D, w.to_out_w, w.to_out_b, ws.x1_img, D, B * Ni, D, D, 0);
+  gated(probs[np++], a->hidden, a->hidden_f32, g_a, md, Ni, 1);
+  if (text_out) {
+    probs[np] = problem(ws.o_txt, D, w.to_add_out_w, w.to_add_out_b, ws.x1_txt, D, B * Nt, D, D, 0);
+    gated(probs[np++], a->encoder, a->encoder_f32, c_g_a, mdt, Nt, 1);
+  }
+  if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
+
+  // 6. norm2 + modulate on the fp32 stream
+  int nj = 0;
+  memset(jobs, 0, sizeof(jobs));
+  jobs[nj].x = ws.x1_img, jobs[nj].y = ws.n_img, jobs[nj].shift = sh_m, jobs[nj].scale = sc_m;
+  jobs[nj].x_sb = (int64_t)Ni * D, jobs[nj].x_st = D, jobs[nj].y_sb = (int64_t)Ni * D, jobs[nj].y_st = D, jobs[nj].mod_stride = md;
+  jobs[nj].batch = B, jobs[nj].tokens = Ni, jobs[nj].x_f32 = 1;
+  nj++;
+  if (text_out) {
+    jobs[nj].x = ws.x1_txt, jobs[nj].y = ws.n_txt, jobs[nj].shift = c_sh_m, jobs[nj].scale = c_sc_m;
+    jobs[nj].x_sb = (int64_t)Nt * D, jobs[nj].x_st = D, jobs[nj].y_sb = (int64_t)Nt * D, jobs[nj].y_st = D, jobs[nj].mod_stride = mdt;
+    jobs[nj].batch = B, jobs[nj].tokens = Nt, jobs[nj].x_f32 = 1;
+    nj++;
+  }
+  if ((rc = hdit_layernorm_modulate_jobs(jobs, nj, D, nullptr, nullptr, eps, stream))) return rc;
+
+  // 7. MLP: bias + GELU-tanh in the first epilogue, gated residual in the second
+  np = 0;
+  probs[np++] = problem(ws.n_img, D, w.ff_in_w, w.ff_in_b, ws.h_img, F, B * Ni, F, D, HDIT_EPI_BIAS_GELU);
+  if (text_out) probs[np++] = problem(ws.n_txt, D, w.ff_context_in_w, w.ff_context_in_b, ws.h_txt, F, B * Nt, F, D, HDIT_EPI_BIAS_GELU);
+  if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
+  np = 0;
+  probs[np] = problem(ws.h_img, F, w.ff_out_w, w.ff_out_b, a->hidden_out, D, B * Ni, D, F, 0);
+  gated(probs[np++], ws.x1_img, 1, g_m, md, Ni, a->out_f32);
+  if (text_out) {
+    probs[np] = problem(ws.h_txt, F, w.ff_context_out_w, w.ff_context_out_b, a->encoder_out, D, B * Nt, D, F, 0);
+    gated(probs[np++], ws.x1_txt, 1, c_g_m, mdt, Nt, a->out_f32);
+  }
+  return hdit_gemm_bf16(probs, np, stream);
+}

@@ -231,6 +231,80 @@ def attention_fp8_static(args: AttnArgs, absmax: torch.Tensor):
 
 
 # ---------------------------------------------------------------------------
+# whole-block entry point
+# ---------------------------------------------------------------------------
+
+def block_sd3(block, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
+              out_dtype=bf16, skip_text_output: bool = False, kv_buffer: Optional[torch.Tensor] = None, kv_row0: int = 0):
+    """One SD3 joint block through ``hdit_block_sd3`` -- the single C-ABI call a non-Python host would make --
+    with the weights of a ``JointTransformerBlock``.  Returns ``(encoder_or_None, hidden)`` like the block.
+    ``kv_buffer``: bf16 [B, rows, 2*dim] stale K|V buffer of a PipeFusion patch whose rows
+    ``[kv_row0, kv_row0 + n_img)`` this call overwrites."""
+    attn, m = block.attn, block.attn.module
+    B, Ni, D = hidden_states.shape
+    Nt = encoder_hidden_states.shape[1]
+    for t, name in ((hidden_states, "hidden_states"), (encoder_hidden_states, "encoder_hidden_states")):
+        if not t.is_cuda or t.dtype not in (bf16, torch.float32) or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous bf16 or f32 GPU tensor")
+    _need(temb, bf16, "temb")
+    qkv_w, qkv_b = attn._qkv.get()
+    aqkv_w, aqkv_b = attn._add_qkv.get()
+    pre_only = bool(block.context_pre_only)
+    a = _lib.Sd3BlockArgs()
+    keep = [qkv_w, qkv_b, aqkv_w, aqkv_b]
+
+    def ptr(t):
+        if t is None:
+            return None
+        keep.append(t)
+        return t.data_ptr()
+
+    w = a.w
+    w.norm1_w, w.norm1_b = ptr(block.norm1.linear.weight.data), ptr(block.norm1.linear.bias.data)
+    w.norm1_context_w, w.norm1_context_b = ptr(block.norm1_context.linear.weight.data), ptr(block.norm1_context.linear.bias.data)
+    w.qkv_w, w.qkv_b, w.add_qkv_w, w.add_qkv_b = ptr(qkv_w), ptr(qkv_b), ptr(aqkv_w), ptr(aqkv_b)
+    w.to_out_w = ptr(m.to_out[0].weight.data)
+    w.to_out_b = ptr(attn.output_bias.data) if attn.has_output_bias else None
+    if not pre_only:
+        w.to_add_out_w = ptr(m.to_add_out.weight.data)
+        w.to_add_out_b = ptr(attn.encoder_output_bias.data) if attn.has_encoder_output_bias else None
+    ff = block.ff
+    w.ff_in_w, w.ff_in_b = ptr(ff.module.net[0].proj.weight.data), ptr(ff.module.net[0].proj.bias.data)
+    w.ff_out_w = ptr(ff.module.net[2].weight.data)
+    w.ff_out_b = ptr(ff.output_bias.data) if ff.has_output_bias else None
+    if block.ff_context is not None:
+        fc = block.ff_context
+        w.ff_context_in_w, w.ff_context_in_b = ptr(fc.module.net[0].proj.weight.data), ptr(fc.module.net[0].proj.bias.data)
+        w.ff_context_out_w = ptr(fc.module.net[2].weight.data)
+        w.ff_context_out_b = ptr(fc.output_bias.data) if fc.has_output_bias else None
+    text_out = not pre_only and not skip_text_output
+    hidden_out = torch.empty(B, Ni, D, dtype=out_dtype, device=hidden_states.device)
+    encoder_out = torch.empty(B, Nt, D, dtype=out_dtype, device=hidden_states.device) if text_out else None
+    a.hidden, a.encoder, a.temb = hidden_states.data_ptr(), encoder_hidden_states.data_ptr(), temb.contiguous().data_ptr()
+    a.hidden_out, a.encoder_out = hidden_out.data_ptr(), (encoder_out.data_ptr() if text_out else None)
+    a.batch, a.n_img, a.n_txt, a.dim, a.heads = B, Ni, Nt, D, attn.heads_per_device
+    a.ff_dim, a.temb_dim = ff.module.net[0].proj.weight.shape[0], temb.shape[1]
+    a.hidden_f32, a.encoder_f32 = int(hidden_states.dtype == torch.float32), int(encoder_hidden_states.dtype == torch.float32)
+    a.out_f32 = int(out_dtype == torch.float32)
+    a.context_pre_only, a.skip_text_output = int(pre_only), int(skip_text_output)
+    if kv_buffer is not None:
+        _need(kv_buffer, bf16, "kv_buffer")
+        if tuple(kv_buffer.shape[::2]) != (B, 2 * D) or not kv_buffer.is_contiguous():
+            raise ValueError("kv_buffer must be a contiguous bf16 [batch, rows, 2 * dim] tensor")
+        a.kv_buffer, a.kv_rows, a.kv_row0 = kv_buffer.data_ptr(), kv_buffer.shape[1], kv_row0
+    lib = _lib.lib()
+    nbytes = lib.hdit_block_sd3_workspace_bytes(C.byref(a))
+    if nbytes < 0:
+        raise _lib.HditError("hdit_block_sd3_workspace_bytes refused the arguments")
+    ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=hidden_states.device)
+    base = (ws.data_ptr() + 255) // 256 * 256
+    a.workspace, a.workspace_bytes = base, nbytes
+    check(lib.hdit_block_sd3(C.byref(a), _stream()), "hdit_block_sd3")
+    a._keep = (keep, ws, hidden_states, encoder_hidden_states, temb, kv_buffer)
+    return encoder_out, hidden_out
+
+
+# ---------------------------------------------------------------------------
 # glue
 # ---------------------------------------------------------------------------
 

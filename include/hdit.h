@@ -286,6 +286,63 @@ int hdit_silu(const void* x, void* y, int64_t count, void* stream);
 int hdit_cfg_euler_step(const void* noise_uncond, const void* noise_cond, const void* sample, void* out,
                         int64_t count, float guidance, float sigma, float sigma_next, void* stream);
 
+/* ------------------------------------------------------------------------
+ * One SD3 MMDiT joint block (diffusers JointTransformerBlock with the reference's
+ * attention / feed-forward wrappers applied) as one call: adaLN projections,
+ * norm1 + modulate, q|k|v of both streams, joint attention over [image, text],
+ * out-projections with the gated residual, norm2 + modulate, GELU-tanh MLP with
+ * the gated residual -- the launch sequence of the Python block, for hosts that
+ * are not Python.  It is what the block loop of
+ * models/transformers/transformer_sd3.py:107-152 calls per layer.
+ *
+ * All tensors are contiguous.  hidden [batch, n_img, dim], encoder [batch, n_txt,
+ * dim] are bf16, or f32 with hidden_f32 / encoder_f32 (the residual stream of a
+ * stack carried in fp32); temb bf16 [batch, temb_dim]; outputs bf16, or f32 with
+ * out_f32.  Weights are bf16 nn.Linear weights [out, in] and biases [out] (NULL =
+ * no bias): qkv_w = [to_q; to_k; to_v] packed [3 dim, dim], add_qkv_w likewise
+ * for the text stream, norm1_w [6 dim, temb_dim], norm1_context_w [6 dim,
+ * temb_dim] (context_pre_only: [2 dim, temb_dim], chunk order scale, shift).
+ * context_pre_only != 0: last block -- no text out-projection, no text MLP,
+ * encoder_out is not written.  skip_text_output != 0: the caller drops the text
+ * output (pipeline patches after the first): the text stream only supplies keys
+ * and values.  kv_buffer != NULL: the stale K|V buffer of a PipeFusion patch,
+ * bf16 [batch, kv_rows, 2 dim] (k | v per row): this call's image rows overwrite
+ * rows [kv_row0, kv_row0 + n_img) and attention reads all kv_rows
+ * (core/resource_manager/cache_manager.py:117-149).  modulation_img /
+ * modulation_txt: optional precomputed linear(silu(temb)) of norm1 /
+ * norm1_context (f32 [batch, 6 dim] / [batch, 6 dim or 2 dim]); NULL => computed
+ * here.  workspace: hdit_block_sd3_workspace_bytes(args) bytes, 256-byte aligned,
+ * caller-owned, contents undefined afterwards.
+ * ---------------------------------------------------------------------- */
+typedef struct hdit_sd3_block_weights {
+  const void *norm1_w, *norm1_b, *norm1_context_w, *norm1_context_b;
+  const void *qkv_w, *qkv_b, *add_qkv_w, *add_qkv_b;
+  const void *to_out_w, *to_out_b, *to_add_out_w, *to_add_out_b;
+  const void *ff_in_w, *ff_in_b, *ff_out_w, *ff_out_b;
+  const void *ff_context_in_w, *ff_context_in_b, *ff_context_out_w, *ff_context_out_b;
+} hdit_sd3_block_weights;
+
+typedef struct hdit_sd3_block_args {
+  hdit_sd3_block_weights w;
+  const void* hidden;
+  const void* encoder;
+  const void* temb;
+  void* hidden_out;
+  void* encoder_out;
+  const float* modulation_img;
+  const float* modulation_txt;
+  void* kv_buffer;
+  void* workspace;
+  int64_t workspace_bytes;
+  int32_t batch, n_img, n_txt, dim, heads, ff_dim, temb_dim;
+  int32_t kv_rows, kv_row0;
+  int32_t hidden_f32, encoder_f32, out_f32;
+  int32_t context_pre_only, skip_text_output;
+} hdit_sd3_block_args;
+
+int64_t hdit_block_sd3_workspace_bytes(const hdit_sd3_block_args* args);
+int hdit_block_sd3(const hdit_sd3_block_args* args, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

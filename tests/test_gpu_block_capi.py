@@ -1,0 +1,102 @@
+"""``hdit_block_sd3`` -- a whole SD3 joint block as ONE call of the C ABI, what a host that is not Python would
+bind -- against the Python block, which launches the same kernels one by one (bit-identical outputs), and
+against the fp32 oracle."""
+import ctypes as C
+
+import pytest
+import torch
+
+import oracle
+from tests.util import assert_parity, oracle_params
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(autouse=True)
+def fresh_state():
+    from hetu_dit_amd.cache_manager import reset_cache_manager
+    from hetu_dit_amd.runtime_state import reset_runtime_state
+
+    reset_runtime_state()
+    reset_cache_manager()
+    yield
+    reset_cache_manager()
+    reset_runtime_state()
+
+
+def make_block(pre_only, seed, D=512, H=8):
+    from hetu_dit_amd import blocks, synthetic
+
+    blk = blocks.JointTransformerBlock(D, H, 64, context_pre_only=pre_only)
+    synthetic.init_module_(blk, seed)
+    return blk.to(DEV), oracle_params(blk)
+
+
+@pytest.mark.parametrize("pre_only", [False, True])
+@pytest.mark.parametrize("stream_f32", [False, True])
+def test_block_sd3_one_call_matches_python_block(hdit, pre_only, stream_f32):
+    from hetu_dit_amd import synthetic
+
+    print(f"hdit_block_sd3 pre_only={pre_only} fp32 stream={stream_f32}", flush=True)
+    B, N, Nt, D, H = 2, 700, 77, 512, 8
+    blk, params = make_block(pre_only, 1, D, H)
+    x, e, t = synthetic.randn_bf16((B, N, D), 2), synthetic.randn_bf16((B, Nt, D), 3), synthetic.randn_bf16((B, D), 4)
+    xd, ed, td = x.to(DEV), e.to(DEV), t.to(DEV)
+    if stream_f32:  # the residual stream of a stack: f32 in, f32 out
+        xd, ed = xd.float() + 1e-3, ed.float() - 1e-3  # values bf16 cannot hold
+        blk.stream_dtype = torch.float32
+    enc_py, hid_py = blk(hidden_states=xd, encoder_hidden_states=ed, temb=td)
+    enc_c, hid_c = hdit.ops.block_sd3(blk, xd, ed, td, out_dtype=torch.float32 if stream_f32 else torch.bfloat16)
+    torch.cuda.synchronize()
+    assert hid_c.dtype == hid_py.dtype and torch.equal(hid_c, hid_py)
+    if pre_only:
+        assert enc_c is None and enc_py is None
+    else:
+        assert torch.equal(enc_c, enc_py)
+    o_enc, o_hid = oracle.sd3_joint_block(params, xd.float().cpu(), ed.float().cpu(), t.float(), H, context_pre_only=pre_only)
+    assert_parity(hid_c, o_hid, what="hdit_block_sd3 hidden")
+    if not pre_only:
+        assert_parity(enc_c, o_enc, what="hdit_block_sd3 encoder")
+
+
+def test_block_sd3_one_call_pipefusion_patch(hdit):
+    """A patch over a stale K|V buffer, with and without the text output, against the Python block driven through
+    the runtime state and cache manager."""
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.cache_manager import get_cache_manager
+    from hetu_dit_amd.runtime_state import get_runtime_state
+
+    B, N, Nt, D, H, P = 2, 512, 77, 512, 8, 4
+    starts = [N // P * i for i in range(P + 1)]
+    blk, params = make_block(False, 11, D, H)
+    x_prev, x_now = synthetic.randn_bf16((B, N, D), 12).to(DEV), synthetic.randn_bf16((B, N, D), 13).to(DEV)
+    e, t = synthetic.randn_bf16((B, Nt, D), 14).to(DEV), synthetic.randn_bf16((B, D), 15).to(DEV)
+    rs = get_runtime_state()
+    rs.set_token_patches(starts)
+    rs.set_patched_mode(False)
+    blk(hidden_states=x_prev, encoder_hidden_states=e, temb=t)  # fills the layer's buffer
+    torch.cuda.synchronize()
+    entry = get_cache_manager()._entry(blk.attn, "attn")
+    kv_c = entry.tensors[0].contiguous().clone()  # the C call's own copy of the stale buffer
+    entry.tensors[0] = entry.tensors[0].contiguous().clone()
+    rs.set_patched_mode(True)
+    for p, skip in ((0, False), (1, True), (2, True), (3, False)):
+        rs.pipeline_patch_idx = p
+        xp = x_now[:, starts[p]:starts[p + 1]].contiguous()
+        enc_py, hid_py = blk(hidden_states=xp, encoder_hidden_states=e, temb=t, skip_text_output=skip)
+        enc_c, hid_c = hdit.ops.block_sd3(blk, xp, e, t, skip_text_output=skip, kv_buffer=kv_c, kv_row0=starts[p])
+        torch.cuda.synchronize()
+        assert torch.equal(hid_c, hid_py), f"patch {p}"
+        assert (enc_c is None and enc_py is None) if skip else torch.equal(enc_c, enc_py)
+        assert torch.equal(kv_c, entry.tensors[0]), f"stale buffer after patch {p}"
+
+
+def test_block_sd3_refuses_bad_arguments(hdit):
+    from hetu_dit_amd import _lib
+
+    lib = _lib.lib()
+    a = _lib.Sd3BlockArgs()
+    assert lib.hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
+    assert lib.hdit_block_sd3(C.byref(a), None) == -1
+    assert lib.hdit_block_sd3(None, None) == -1
