@@ -121,6 +121,39 @@ class Sd3BlockArgs(C.Structure):
         "encoder_f32", "out_f32", "context_pre_only", "skip_text_output")]
 
 
+def _ptrs(*names):
+    return [(n, C.c_void_p) for n in names]
+
+
+def _ints(*names):
+    return [(n, C.c_int32) for n in names]
+
+
+class FluxDoubleBlockArgs(C.Structure):
+    _fields_ = ([("w", Sd3BlockWeights)] + _ptrs("norm_q_w", "norm_k_w", "norm_added_q_w", "norm_added_k_w", "hidden", "encoder",
+                                                  "temb", "rope_cos", "rope_sin", "hidden_out", "encoder_out", "workspace")
+                + [("workspace_bytes", C.c_int64), ("qk_norm_eps", C.c_float)]
+                + _ints("qk_norm_kind", "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "hidden_f32",
+                        "encoder_f32", "out_f32"))
+
+
+class FluxSingleBlockArgs(C.Structure):
+    _fields_ = (_ptrs("norm_w", "norm_b", "qkv_w", "qkv_b", "proj_mlp_w", "proj_mlp_b", "proj_out_w", "proj_out_b", "norm_q_w",
+                      "norm_k_w", "hidden", "temb", "rope_cos", "rope_sin", "hidden_out", "workspace")
+                + [("workspace_bytes", C.c_int64), ("qk_norm_eps", C.c_float)]
+                + _ints("qk_norm_kind", "batch", "seq", "dim", "heads", "ff_dim", "temb_dim", "hidden_f32", "out_f32"))
+
+
+class CogVideoXBlockArgs(C.Structure):
+    _fields_ = (_ptrs("norm1_w", "norm1_b", "norm1_ln_w", "norm1_ln_b", "norm2_w", "norm2_b", "norm2_ln_w", "norm2_ln_b",
+                      "qkv_w", "qkv_b", "to_out_w", "to_out_b", "norm_q_w", "norm_q_b", "norm_k_w", "norm_k_b",
+                      "ff_in_w", "ff_in_b", "ff_out_w", "ff_out_b", "hidden", "encoder", "temb", "rope_cos", "rope_sin",
+                      "hidden_out", "encoder_out", "workspace")
+                + [("workspace_bytes", C.c_int64), ("norm_eps", C.c_float), ("qk_norm_eps", C.c_float)]
+                + _ints("qk_norm_kind", "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "hidden_f32",
+                        "encoder_f32", "out_f32"))
+
+
 # name -> (restype, argtypes); every symbol include/hdit.h declares
 SIGNATURES = {
     "hdit_abi_version": (C.c_int, []),
@@ -133,6 +166,12 @@ SIGNATURES = {
     "hdit_attn_fwd_fp8_static": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p]),
     "hdit_block_sd3_workspace_bytes": (C.c_int64, [C.POINTER(Sd3BlockArgs)]),
     "hdit_block_sd3": (C.c_int, [C.POINTER(Sd3BlockArgs), C.c_void_p]),
+    "hdit_block_flux_double_workspace_bytes": (C.c_int64, [C.POINTER(FluxDoubleBlockArgs)]),
+    "hdit_block_flux_double": (C.c_int, [C.POINTER(FluxDoubleBlockArgs), C.c_void_p]),
+    "hdit_block_flux_single_workspace_bytes": (C.c_int64, [C.POINTER(FluxSingleBlockArgs)]),
+    "hdit_block_flux_single": (C.c_int, [C.POINTER(FluxSingleBlockArgs), C.c_void_p]),
+    "hdit_block_cogvideox_workspace_bytes": (C.c_int64, [C.POINTER(CogVideoXBlockArgs)]),
+    "hdit_block_cogvideox": (C.c_int, [C.POINTER(CogVideoXBlockArgs), C.c_void_p]),
     "hdit_layernorm_modulate": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,

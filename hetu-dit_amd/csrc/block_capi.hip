@@ -245,3 +245,302 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
   }
   return hdit_gemm_bf16(probs, np, stream);
 }
+
+// ---------------------------------------------------------------------------------------------------------
+// Flux and CogVideoX blocks
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+
+struct Carver {
+  unsigned char* base;
+  int64_t off = 0;
+  explicit Carver(void* b) : base((unsigned char*)b) {}
+  unsigned char* take(int64_t nbytes) {
+    unsigned char* p = base ? base + off : nullptr;
+    off += up(nbytes);
+    return p;
+  }
+};
+
+void ln_job(hdit_ln_job& j, const void* x, int x_f32, void* y, int64_t y_sb, const float* shift, const float* scale,
+            int64_t mod_stride, int batch, int tokens, int dim) {
+  memset(&j, 0, sizeof(j));
+  j.x = x, j.y = y, j.shift = shift, j.scale = scale;
+  j.x_sb = (int64_t)tokens * dim, j.x_st = dim, j.y_sb = y_sb, j.y_st = dim, j.mod_stride = mod_stride;
+  j.batch = batch, j.tokens = tokens, j.x_f32 = x_f32;
+}
+
+void gated(hdit_gemm_problem& p, const void* resid, int resid_f32, const float* gate, int64_t gate_stride, int rows,
+           int out_f32) {
+  p.epilogue = HDIT_EPI_GATE_RESIDUAL | (resid_f32 ? HDIT_EPI_RESID_F32 : 0) | (out_f32 ? HDIT_EPI_OUT_F32 : 0);
+  p.resid = resid, p.ldr = p.n, p.gate = gate, p.gate_stride = (int32_t)gate_stride, p.rows_per_batch = rows;
+}
+
+void qk_job(hdit_qknorm_job& j, void* x, int64_t rows_per_batch, int64_t ld, int hd, const void* weight, const void* bias,
+            const float* cos_t, const float* sin_t, int seq, int rope_row0, int rope_rows, int norm_kind) {
+  memset(&j, 0, sizeof(j));
+  j.x = x, j.stride_b = rows_per_batch * ld, j.stride_s = ld, j.stride_h = hd;
+  j.weight = weight, j.bias = bias, j.cos_table = cos_t, j.sin_table = sin_t;
+  j.seq = seq, j.rope_row0 = rope_row0, j.rope_rows = rope_rows, j.norm_kind = norm_kind;
+}
+
+void seg(hdit_seq_segment& s, const void* p, int64_t rows_per_batch, int64_t ld, int hd, int len) {
+  s.ptr = p, s.stride_b = rows_per_batch * ld, s.stride_s = ld, s.stride_h = hd, s.len = len;
+}
+
+bool head_dim_ok(int dim, int heads) { return heads > 0 && dim % heads == 0 && (dim / heads == 64 || dim / heads == 128); }
+
+struct FluxDoubleWs {
+  float *emb_img, *emb_txt, *x1_img, *x1_txt;
+  unsigned char *n_img, *n_txt, *qkv_img, *qkv_txt, *o_img, *o_txt, *h_img, *h_txt;
+  int64_t bytes;
+};
+FluxDoubleWs carve(const hdit_flux_double_block_args* a, void* base) {
+  const int64_t B = a->batch, Ni = a->n_img, Nt = a->n_txt, D = a->dim, F = a->ff_dim;
+  Carver c(base);
+  FluxDoubleWs w;
+  w.emb_img = (float*)c.take(B * 6 * D * 4), w.emb_txt = (float*)c.take(B * 6 * D * 4);
+  w.n_img = c.take(B * Ni * D * 2), w.n_txt = c.take(B * Nt * D * 2);
+  w.qkv_img = c.take(B * Ni * 3 * D * 2), w.qkv_txt = c.take(B * Nt * 3 * D * 2);
+  w.o_img = c.take(B * Ni * D * 2), w.o_txt = c.take(B * Nt * D * 2);
+  w.x1_img = (float*)c.take(B * Ni * D * 4), w.x1_txt = (float*)c.take(B * Nt * D * 4);
+  w.h_img = c.take(B * Ni * F * 2), w.h_txt = c.take(B * Nt * F * 2);
+  w.bytes = c.off;
+  return w;
+}
+int validate(const hdit_flux_double_block_args* a) {
+  if (!a || a->batch <= 0 || a->n_img <= 0 || a->n_txt <= 0 || a->dim <= 0 || a->ff_dim <= 0 || a->temb_dim <= 0) return HDIT_EINVAL;
+  if (!head_dim_ok(a->dim, a->heads)) return HDIT_EUNSUPPORTED;
+  if (a->dim % 64 || a->ff_dim % 64) return HDIT_EUNSUPPORTED;
+  const hdit_sd3_block_weights& w = a->w;
+  if (!a->hidden || !a->encoder || !a->temb || !a->hidden_out || !a->encoder_out) return HDIT_EINVAL;
+  if (!w.norm1_w || !w.norm1_b || !w.norm1_context_w || !w.norm1_context_b || !w.qkv_w || !w.add_qkv_w || !w.to_out_w ||
+      !w.to_add_out_w || !w.ff_in_w || !w.ff_out_w || !w.ff_context_in_w || !w.ff_context_out_w)
+    return HDIT_EINVAL;
+  if ((a->rope_cos == nullptr) != (a->rope_sin == nullptr)) return HDIT_EINVAL;
+  return HDIT_OK;
+}
+
+struct FluxSingleWs {
+  float* emb;
+  unsigned char *n, *qkv, *cat;
+  int64_t bytes;
+};
+FluxSingleWs carve(const hdit_flux_single_block_args* a, void* base) {
+  const int64_t B = a->batch, S = a->seq, D = a->dim, F = a->ff_dim;
+  Carver c(base);
+  FluxSingleWs w;
+  w.emb = (float*)c.take(B * 3 * D * 4);
+  w.n = c.take(B * S * D * 2);
+  w.qkv = c.take(B * S * 3 * D * 2);
+  w.cat = c.take(B * S * (D + F) * 2);
+  w.bytes = c.off;
+  return w;
+}
+int validate(const hdit_flux_single_block_args* a) {
+  if (!a || a->batch <= 0 || a->seq <= 0 || a->dim <= 0 || a->ff_dim <= 0 || a->temb_dim <= 0) return HDIT_EINVAL;
+  if (!head_dim_ok(a->dim, a->heads)) return HDIT_EUNSUPPORTED;
+  if (a->dim % 64 || a->ff_dim % 64) return HDIT_EUNSUPPORTED;
+  if (!a->hidden || !a->temb || !a->hidden_out || !a->norm_w || !a->norm_b || !a->qkv_w || !a->proj_mlp_w || !a->proj_out_w)
+    return HDIT_EINVAL;
+  if ((a->rope_cos == nullptr) != (a->rope_sin == nullptr)) return HDIT_EINVAL;
+  return HDIT_OK;
+}
+
+struct CogWs {
+  float *emb1, *emb2, *x1_h, *x1_e;
+  unsigned char *joint, *qkv, *o, *h;
+  int64_t bytes;
+};
+CogWs carve(const hdit_cogvideox_block_args* a, void* base) {
+  const int64_t B = a->batch, S = (int64_t)a->n_img + a->n_txt, D = a->dim, F = a->ff_dim;
+  Carver c(base);
+  CogWs w;
+  w.emb1 = (float*)c.take(B * 6 * D * 4), w.emb2 = (float*)c.take(B * 6 * D * 4);
+  w.joint = c.take(B * S * D * 2);
+  w.qkv = c.take(B * S * 3 * D * 2);
+  w.o = c.take(B * S * D * 2);
+  w.x1_h = (float*)c.take(B * a->n_img * D * 4), w.x1_e = (float*)c.take(B * a->n_txt * D * 4);
+  w.h = c.take(B * S * F * 2);
+  w.bytes = c.off;
+  return w;
+}
+int validate(const hdit_cogvideox_block_args* a) {
+  if (!a || a->batch <= 0 || a->n_img <= 0 || a->n_txt <= 0 || a->dim <= 0 || a->ff_dim <= 0 || a->temb_dim <= 0) return HDIT_EINVAL;
+  if (2 * a->batch > HDIT_GEMM_MAX_PROBLEMS) return HDIT_EUNSUPPORTED;
+  if (!head_dim_ok(a->dim, a->heads)) return HDIT_EUNSUPPORTED;
+  if (a->dim % 64 || a->ff_dim % 64) return HDIT_EUNSUPPORTED;
+  if (!a->hidden || !a->encoder || !a->temb || !a->hidden_out || !a->encoder_out) return HDIT_EINVAL;
+  if (!a->norm1_w || !a->norm1_b || !a->norm2_w || !a->norm2_b || !a->qkv_w || !a->to_out_w || !a->ff_in_w || !a->ff_out_w)
+    return HDIT_EINVAL;
+  if ((a->rope_cos == nullptr) != (a->rope_sin == nullptr)) return HDIT_EINVAL;
+  return HDIT_OK;
+}
+
+template <class Args>
+int check_workspace(const Args* a, int64_t need) {
+  if (!a->workspace || (((uintptr_t)a->workspace) & (ALIGN - 1)) || a->workspace_bytes < need) return HDIT_EINVAL;
+  return HDIT_OK;
+}
+
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int64_t hdit_block_flux_double_workspace_bytes(const hdit_flux_double_block_args* a) {
+  return validate(a) == HDIT_OK ? carve(a, nullptr).bytes : -1;
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_block_flux_double(const hdit_flux_double_block_args* a, void* stream) {
+  int rc = validate(a);
+  if (rc != HDIT_OK) return rc;
+  const FluxDoubleWs ws = carve(a, a->workspace);
+  if ((rc = check_workspace(a, ws.bytes))) return rc;
+  const hdit_sd3_block_weights& w = a->w;
+  const int B = a->batch, Ni = a->n_img, Nt = a->n_txt, D = a->dim, F = a->ff_dim, H = a->heads, hd = D / H;
+  const float eps = 1e-6f;
+  const int64_t md = 6 * (int64_t)D;
+  if ((rc = hdit_adaln_gemv(a->temb, w.norm1_w, w.norm1_b, ws.emb_img, B, 6 * D, a->temb_dim, stream))) return rc;
+  if ((rc = hdit_adaln_gemv(a->temb, w.norm1_context_w, w.norm1_context_b, ws.emb_txt, B, 6 * D, a->temb_dim, stream))) return rc;
+  const float *ei = ws.emb_img, *et = ws.emb_txt;  // shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp
+  hdit_ln_job jobs[2];
+  ln_job(jobs[0], a->hidden, a->hidden_f32, ws.n_img, (int64_t)Ni * D, ei, ei + D, md, B, Ni, D);
+  ln_job(jobs[1], a->encoder, a->encoder_f32, ws.n_txt, (int64_t)Nt * D, et, et + D, md, B, Nt, D);
+  if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, nullptr, nullptr, eps, stream))) return rc;
+  hdit_gemm_problem probs[4];
+  probs[0] = problem(ws.n_img, D, w.qkv_w, w.qkv_b, ws.qkv_img, 3 * D, B * Ni, 3 * D, D, HDIT_EPI_BIAS);
+  probs[1] = problem(ws.n_txt, D, w.add_qkv_w, w.add_qkv_b, ws.qkv_txt, 3 * D, B * Nt, 3 * D, D, HDIT_EPI_BIAS);
+  if ((rc = hdit_gemm_bf16(probs, 2, stream))) return rc;
+  // per-head RMSNorm on q, k of both streams, then the rotation of the joint [text, image] rows
+  const int64_t ld3 = 3 * (int64_t)D;
+  unsigned char *q_img = ws.qkv_img, *k_img = ws.qkv_img + (int64_t)D * 2, *v_img = ws.qkv_img + (int64_t)2 * D * 2;
+  unsigned char *q_txt = ws.qkv_txt, *k_txt = ws.qkv_txt + (int64_t)D * 2, *v_txt = ws.qkv_txt + (int64_t)2 * D * 2;
+  const float* cos_i = a->rope_cos ? a->rope_cos + (int64_t)Nt * hd : nullptr;
+  const float* sin_i = a->rope_sin ? a->rope_sin + (int64_t)Nt * hd : nullptr;
+  hdit_qknorm_job qj[4];
+  qk_job(qj[0], q_txt, Nt, ld3, hd, a->norm_added_q_w, nullptr, a->rope_cos, a->rope_sin, Nt, 0, Nt, a->qk_norm_kind);
+  qk_job(qj[1], k_txt, Nt, ld3, hd, a->norm_added_k_w, nullptr, a->rope_cos, a->rope_sin, Nt, 0, Nt, a->qk_norm_kind);
+  qk_job(qj[2], q_img, Ni, ld3, hd, a->norm_q_w, nullptr, cos_i, sin_i, Ni, 0, Ni, a->qk_norm_kind);
+  qk_job(qj[3], k_img, Ni, ld3, hd, a->norm_k_w, nullptr, cos_i, sin_i, Ni, 0, Ni, a->qk_norm_kind);
+  if ((rc = hdit_qk_norm_rope(qj, 4, B, H, hd, a->qk_norm_eps, stream))) return rc;
+  hdit_attn_args at;
+  memset(&at, 0, sizeof(at));
+  seg(at.q[0], q_txt, Nt, ld3, hd, Nt), seg(at.q[1], q_img, Ni, ld3, hd, Ni);
+  seg(at.k[0], k_txt, Nt, ld3, hd, Nt), seg(at.k[1], k_img, Ni, ld3, hd, Ni);
+  seg(at.v[0], v_txt, Nt, ld3, hd, Nt), seg(at.v[1], v_img, Ni, ld3, hd, Ni);
+  seg(at.o[0], ws.o_txt, Nt, D, hd, Nt), seg(at.o[1], ws.o_img, Ni, D, hd, Ni);
+  at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
+  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
+  // the reference's wrapper never adds the text out-projection bias back in its Flux branch
+  // (layers/attention_processor.py:176-192,:284-305): to_add_out runs without bias
+  probs[0] = problem(ws.o_img, D, w.to_out_w, w.to_out_b, ws.x1_img, D, B * Ni, D, D, 0);
+  gated(probs[0], a->hidden, a->hidden_f32, ei + 2 * D, md, Ni, 1);
+  probs[1] = problem(ws.o_txt, D, w.to_add_out_w, nullptr, ws.x1_txt, D, B * Nt, D, D, 0);
+  gated(probs[1], a->encoder, a->encoder_f32, et + 2 * D, md, Nt, 1);
+  if ((rc = hdit_gemm_bf16(probs, 2, stream))) return rc;
+  ln_job(jobs[0], ws.x1_img, 1, ws.n_img, (int64_t)Ni * D, ei + 3 * D, ei + 4 * D, md, B, Ni, D);
+  ln_job(jobs[1], ws.x1_txt, 1, ws.n_txt, (int64_t)Nt * D, et + 3 * D, et + 4 * D, md, B, Nt, D);
+  if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, nullptr, nullptr, eps, stream))) return rc;
+  probs[0] = problem(ws.n_img, D, w.ff_in_w, w.ff_in_b, ws.h_img, F, B * Ni, F, D, HDIT_EPI_BIAS_GELU);
+  probs[1] = problem(ws.n_txt, D, w.ff_context_in_w, w.ff_context_in_b, ws.h_txt, F, B * Nt, F, D, HDIT_EPI_BIAS_GELU);
+  if ((rc = hdit_gemm_bf16(probs, 2, stream))) return rc;
+  probs[0] = problem(ws.h_img, F, w.ff_out_w, w.ff_out_b, a->hidden_out, D, B * Ni, D, F, 0);
+  gated(probs[0], ws.x1_img, 1, ei + 5 * D, md, Ni, a->out_f32);
+  probs[1] = problem(ws.h_txt, F, w.ff_context_out_w, w.ff_context_out_b, a->encoder_out, D, B * Nt, D, F, 0);
+  gated(probs[1], ws.x1_txt, 1, et + 5 * D, md, Nt, a->out_f32);
+  return hdit_gemm_bf16(probs, 2, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int64_t hdit_block_flux_single_workspace_bytes(const hdit_flux_single_block_args* a) {
+  return validate(a) == HDIT_OK ? carve(a, nullptr).bytes : -1;
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_block_flux_single(const hdit_flux_single_block_args* a, void* stream) {
+  int rc = validate(a);
+  if (rc != HDIT_OK) return rc;
+  const FluxSingleWs ws = carve(a, a->workspace);
+  if ((rc = check_workspace(a, ws.bytes))) return rc;
+  const int B = a->batch, S = a->seq, D = a->dim, F = a->ff_dim, H = a->heads, hd = D / H;
+  const int64_t md = 3 * (int64_t)D, ldc = (int64_t)D + F, ld3 = 3 * (int64_t)D;
+  if ((rc = hdit_adaln_gemv(a->temb, a->norm_w, a->norm_b, ws.emb, B, 3 * D, a->temb_dim, stream))) return rc;
+  hdit_ln_job job;
+  ln_job(job, a->hidden, a->hidden_f32, ws.n, (int64_t)S * D, ws.emb, ws.emb + D, md, B, S, D);  // shift, scale, gate
+  if ((rc = hdit_layernorm_modulate_jobs(&job, 1, D, nullptr, nullptr, 1e-6f, stream))) return rc;
+  // q|k|v and the MLP-in projection share their input: one launch; GELU(MLP) lands beside the attention output
+  hdit_gemm_problem probs[2];
+  probs[0] = problem(ws.n, D, a->qkv_w, a->qkv_b, ws.qkv, ld3, B * S, 3 * D, D, HDIT_EPI_BIAS);
+  probs[1] = problem(ws.n, D, a->proj_mlp_w, a->proj_mlp_b, ws.cat + (int64_t)D * 2, ldc, B * S, F, D, HDIT_EPI_BIAS_GELU);
+  if ((rc = hdit_gemm_bf16(probs, 2, stream))) return rc;
+  unsigned char *q = ws.qkv, *k = ws.qkv + (int64_t)D * 2, *v = ws.qkv + (int64_t)2 * D * 2;
+  hdit_qknorm_job qj[2];
+  qk_job(qj[0], q, S, ld3, hd, a->norm_q_w, nullptr, a->rope_cos, a->rope_sin, S, 0, S, a->qk_norm_kind);
+  qk_job(qj[1], k, S, ld3, hd, a->norm_k_w, nullptr, a->rope_cos, a->rope_sin, S, 0, S, a->qk_norm_kind);
+  if ((rc = hdit_qk_norm_rope(qj, 2, B, H, hd, a->qk_norm_eps, stream))) return rc;
+  hdit_attn_args at;
+  memset(&at, 0, sizeof(at));
+  seg(at.q[0], q, S, ld3, hd, S), seg(at.k[0], k, S, ld3, hd, S), seg(at.v[0], v, S, ld3, hd, S);
+  seg(at.o[0], ws.cat, S, ldc, hd, S);
+  at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
+  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
+  probs[0] = problem(ws.cat, ldc, a->proj_out_w, a->proj_out_b, a->hidden_out, D, B * S, D, D + F, 0);
+  gated(probs[0], a->hidden, a->hidden_f32, ws.emb + 2 * D, md, S, a->out_f32);
+  return hdit_gemm_bf16(probs, 1, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int64_t hdit_block_cogvideox_workspace_bytes(const hdit_cogvideox_block_args* a) {
+  return validate(a) == HDIT_OK ? carve(a, nullptr).bytes : -1;
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_block_cogvideox(const hdit_cogvideox_block_args* a, void* stream) {
+  int rc = validate(a);
+  if (rc != HDIT_OK) return rc;
+  const CogWs ws = carve(a, a->workspace);
+  if ((rc = check_workspace(a, ws.bytes))) return rc;
+  const int B = a->batch, N = a->n_img, Nt = a->n_txt, S = N + Nt, D = a->dim, F = a->ff_dim, H = a->heads, hd = D / H;
+  const int64_t md = 6 * (int64_t)D, ld3 = 3 * (int64_t)D;
+  const int sz_h = a->hidden_f32 ? 4 : 2, sz_e = a->encoder_f32 ? 4 : 2, sz_o = a->out_f32 ? 4 : 2;
+  // norm1: chunks shift, scale, gate, enc_shift, enc_scale, enc_gate; one affine LayerNorm for both streams,
+  // both results written into one joint [text, video] buffer
+  if ((rc = hdit_adaln_gemv(a->temb, a->norm1_w, a->norm1_b, ws.emb1, B, 6 * D, a->temb_dim, stream))) return rc;
+  if ((rc = hdit_adaln_gemv(a->temb, a->norm2_w, a->norm2_b, ws.emb2, B, 6 * D, a->temb_dim, stream))) return rc;
+  hdit_ln_job jobs[2];
+  const float* e1 = ws.emb1;
+  ln_job(jobs[0], a->encoder, a->encoder_f32, ws.joint, (int64_t)S * D, e1 + 3 * D, e1 + 4 * D, md, B, Nt, D);
+  ln_job(jobs[1], a->hidden, a->hidden_f32, ws.joint + (int64_t)Nt * D * 2, (int64_t)S * D, e1, e1 + D, md, B, N, D);
+  if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, a->norm1_ln_w, a->norm1_ln_b, a->norm_eps, stream))) return rc;
+  hdit_gemm_problem probs[HDIT_GEMM_MAX_PROBLEMS];
+  probs[0] = problem(ws.joint, D, a->qkv_w, a->qkv_b, ws.qkv, ld3, B * S, 3 * D, D, HDIT_EPI_BIAS);
+  if ((rc = hdit_gemm_bf16(probs, 1, stream))) return rc;
+  unsigned char *q = ws.qkv, *k = ws.qkv + (int64_t)D * 2, *v = ws.qkv + (int64_t)2 * D * 2;
+  if (a->qk_norm_kind || a->rope_cos) {
+    hdit_qknorm_job qj[2];
+    qk_job(qj[0], q, S, ld3, hd, a->norm_q_w, a->norm_q_b, a->rope_cos, a->rope_sin, S, Nt, N, a->qk_norm_kind);
+    qk_job(qj[1], k, S, ld3, hd, a->norm_k_w, a->norm_k_b, a->rope_cos, a->rope_sin, S, Nt, N, a->qk_norm_kind);
+    if ((rc = hdit_qk_norm_rope(qj, 2, B, H, hd, a->qk_norm_eps, stream))) return rc;
+  }
+  hdit_attn_args at;
+  memset(&at, 0, sizeof(at));
+  seg(at.q[0], q, S, ld3, hd, S), seg(at.k[0], k, S, ld3, hd, S), seg(at.v[0], v, S, ld3, hd, S);
+  seg(at.o[0], ws.o, S, D, hd, S);
+  at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
+  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
+  // one weight set over the joint rows, per-stream gates: per batch element a text and a video problem
+  auto gated_pair = [&](const unsigned char* a_joint, int64_t lda, const void* wt, const void* bias, int kdim, const void* res_e,
+                        int re_sz, const void* res_h, int rh_sz, const float* emb, void* out_e, int oe_sz, void* out_h, int oh_sz) {
+    int np = 0;
+    for (int b = 0; b < B; b++) {
+      const unsigned char* ab = a_joint + (int64_t)b * S * lda * 2;
+      probs[np] = problem(ab, lda, wt, bias, (unsigned char*)out_e + (int64_t)b * Nt * D * oe_sz, D, Nt, D, kdim, 0);
+      gated(probs[np++], (const unsigned char*)res_e + (int64_t)b * Nt * D * re_sz, re_sz == 4, emb + b * md + 5 * D, md, Nt, oe_sz == 4);
+      probs[np] = problem(ab + (int64_t)Nt * lda * 2, lda, wt, bias, (unsigned char*)out_h + (int64_t)b * N * D * oh_sz, D, N, D, kdim, 0);
+      gated(probs[np++], (const unsigned char*)res_h + (int64_t)b * N * D * rh_sz, rh_sz == 4, emb + b * md + 2 * D, md, N, oh_sz == 4);
+    }
+    return hdit_gemm_bf16(probs, np, stream);
+  };
+  if ((rc = gated_pair(ws.o, D, a->to_out_w, a->to_out_b, D, a->encoder, sz_e, a->hidden, sz_h, ws.emb1, ws.x1_e, 4, ws.x1_h, 4))) return rc;
+  const float* e2 = ws.emb2;
+  ln_job(jobs[0], ws.x1_e, 1, ws.joint, (int64_t)S * D, e2 + 3 * D, e2 + 4 * D, md, B, Nt, D);
+  ln_job(jobs[1], ws.x1_h, 1, ws.joint + (int64_t)Nt * D * 2, (int64_t)S * D, e2, e2 + D, md, B, N, D);
+  if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, a->norm2_ln_w, a->norm2_ln_b, a->norm_eps, stream))) return rc;
+  probs[0] = problem(ws.joint, D, a->ff_in_w, a->ff_in_b, ws.h, F, B * S, F, D, HDIT_EPI_BIAS_GELU);
+  if ((rc = hdit_gemm_bf16(probs, 1, stream))) return rc;
+  return gated_pair(ws.h, F, a->ff_out_w, a->ff_out_b, F, ws.x1_e, 4, ws.x1_h, 4, ws.emb2, a->encoder_out, sz_o, a->hidden_out, sz_o);
+}

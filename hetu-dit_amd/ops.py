@@ -304,6 +304,169 @@ def block_sd3(block, hidden_states: torch.Tensor, encoder_hidden_states: torch.T
     return encoder_out, hidden_out
 
 
+class _ArgFiller:
+    """Pointer bookkeeping for the whole-block argument structs: keeps every tensor alive whose address went in."""
+
+    def __init__(self):
+        self.keep = []
+
+    def __call__(self, t):
+        if t is None:
+            return None
+        self.keep.append(t)
+        return t.data_ptr()
+
+
+def _stream_tensor(t: torch.Tensor, name: str) -> int:
+    if not t.is_cuda or t.dtype not in (bf16, torch.float32) or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous bf16 or f32 GPU tensor")
+    return int(t.dtype == torch.float32)
+
+
+def _run_block(a, size_fn, run_fn, what: str, device, keep):
+    nbytes = size_fn(C.byref(a))
+    if nbytes < 0:
+        raise _lib.HditError(f"{what}_workspace_bytes refused the arguments")
+    ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=device)
+    a.workspace, a.workspace_bytes = (ws.data_ptr() + 255) // 256 * 256, nbytes
+    check(run_fn(C.byref(a), _stream()), what)
+    a._keep = (keep, ws)
+
+
+def _norm_kind_of(norm) -> int:
+    if norm is None:
+        return 0
+    return 2 if isinstance(norm, torch.nn.LayerNorm) else 1
+
+
+def _fill_sd3_weights(w, block, ptr):
+    attn, m = block.attn, block.attn.module
+    qkv_w, qkv_b = attn._qkv.get()
+    aqkv_w, aqkv_b = attn._add_qkv.get()
+    w.norm1_w, w.norm1_b = ptr(block.norm1.linear.weight.data), ptr(block.norm1.linear.bias.data)
+    w.norm1_context_w, w.norm1_context_b = ptr(block.norm1_context.linear.weight.data), ptr(block.norm1_context.linear.bias.data)
+    w.qkv_w, w.qkv_b, w.add_qkv_w, w.add_qkv_b = ptr(qkv_w), ptr(qkv_b), ptr(aqkv_w), ptr(aqkv_b)
+    w.to_out_w = ptr(m.to_out[0].weight.data)
+    w.to_out_b = ptr(attn.output_bias.data) if attn.has_output_bias else None
+    if getattr(m, "to_add_out", None) is not None and not m.context_pre_only:
+        w.to_add_out_w = ptr(m.to_add_out.weight.data)
+        w.to_add_out_b = ptr(attn.encoder_output_bias.data) if attn.has_encoder_output_bias else None
+    for prefix, ff in (("ff", block.ff), ("ff_context", getattr(block, "ff_context", None))):
+        if ff is None:
+            continue
+        setattr(w, prefix + "_in_w", ptr(ff.module.net[0].proj.weight.data))
+        setattr(w, prefix + "_in_b", ptr(ff.module.net[0].proj.bias.data))
+        setattr(w, prefix + "_out_w", ptr(ff.module.net[2].weight.data))
+        setattr(w, prefix + "_out_b", ptr(ff.output_bias.data) if ff.has_output_bias else None)
+
+
+def block_flux_double(block, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None, out_dtype=bf16):
+    """One Flux double-stream block through ``hdit_block_flux_double``; returns ``(encoder, hidden)``."""
+    attn, m = block.attn, block.attn.module
+    B, Ni, D = hidden_states.shape
+    Nt = encoder_hidden_states.shape[1]
+    _need(temb, bf16, "temb")
+    a, ptr = _lib.FluxDoubleBlockArgs(), _ArgFiller()
+    _fill_sd3_weights(a.w, block, ptr)
+    for name in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"):
+        n = getattr(m, name)
+        setattr(a, name + "_w", ptr(n.weight.data) if n is not None and n.weight is not None else None)
+    a.qk_norm_kind, a.qk_norm_eps = _norm_kind_of(m.norm_q), float(m.norm_q.eps) if m.norm_q is not None else 1e-6
+    a.hidden_f32, a.encoder_f32 = _stream_tensor(hidden_states, "hidden_states"), _stream_tensor(encoder_hidden_states, "encoder_hidden_states")
+    if image_rotary_emb is not None:
+        cos, sin = image_rotary_emb
+        _need(cos, torch.float32, "cos"), _need(sin, torch.float32, "sin")
+        if tuple(cos.shape) != (Nt + Ni, D // attn.heads_per_device) or cos.shape != sin.shape or not (cos.is_contiguous() and sin.is_contiguous()):
+            raise ValueError("image_rotary_emb must be contiguous f32 [n_txt + n_img, head_dim] tables")
+        a.rope_cos, a.rope_sin = ptr(cos), ptr(sin)
+    hidden_out = torch.empty(B, Ni, D, dtype=out_dtype, device=hidden_states.device)
+    encoder_out = torch.empty(B, Nt, D, dtype=out_dtype, device=hidden_states.device)
+    a.hidden, a.encoder, a.temb = ptr(hidden_states), ptr(encoder_hidden_states), ptr(temb.contiguous())
+    a.hidden_out, a.encoder_out, a.out_f32 = hidden_out.data_ptr(), encoder_out.data_ptr(), int(out_dtype == torch.float32)
+    a.batch, a.n_img, a.n_txt, a.dim, a.heads = B, Ni, Nt, D, attn.heads_per_device
+    a.ff_dim, a.temb_dim = block.ff.module.net[0].proj.weight.shape[0], temb.shape[1]
+    lib = _lib.lib()
+    _run_block(a, lib.hdit_block_flux_double_workspace_bytes, lib.hdit_block_flux_double, "hdit_block_flux_double",
+               hidden_states.device, ptr.keep)
+    return encoder_out, hidden_out
+
+
+def block_flux_single(block, hidden_states, temb, image_rotary_emb=None, out_dtype=bf16):
+    """One Flux single-stream block through ``hdit_block_flux_single`` on the joint [text, image] rows."""
+    attn, m = block.attn, block.attn.module
+    B, S, D = hidden_states.shape
+    _need(temb, bf16, "temb")
+    a, ptr = _lib.FluxSingleBlockArgs(), _ArgFiller()
+    qkv_w, qkv_b = attn._qkv.get()
+    a.norm_w, a.norm_b = ptr(block.norm.linear.weight.data), ptr(block.norm.linear.bias.data)
+    a.qkv_w, a.qkv_b = ptr(qkv_w), ptr(qkv_b)
+    a.proj_mlp_w, a.proj_mlp_b = ptr(block.proj_mlp.weight.data), ptr(block.proj_mlp.bias.data)
+    a.proj_out_w, a.proj_out_b = ptr(block.proj_out.weight.data), ptr(block.proj_out.bias.data)
+    for name in ("norm_q", "norm_k"):
+        n = getattr(m, name)
+        setattr(a, name + "_w", ptr(n.weight.data) if n is not None and n.weight is not None else None)
+    a.qk_norm_kind, a.qk_norm_eps = _norm_kind_of(m.norm_q), float(m.norm_q.eps) if m.norm_q is not None else 1e-6
+    a.hidden_f32 = _stream_tensor(hidden_states, "hidden_states")
+    if image_rotary_emb is not None:
+        cos, sin = image_rotary_emb
+        _need(cos, torch.float32, "cos"), _need(sin, torch.float32, "sin")
+        if tuple(cos.shape) != (S, D // attn.heads_per_device) or cos.shape != sin.shape or not (cos.is_contiguous() and sin.is_contiguous()):
+            raise ValueError("image_rotary_emb must be contiguous f32 [seq, head_dim] tables")
+        a.rope_cos, a.rope_sin = ptr(cos), ptr(sin)
+    hidden_out = torch.empty(B, S, D, dtype=out_dtype, device=hidden_states.device)
+    a.hidden, a.temb, a.hidden_out, a.out_f32 = ptr(hidden_states), ptr(temb.contiguous()), hidden_out.data_ptr(), int(out_dtype == torch.float32)
+    a.batch, a.seq, a.dim, a.heads, a.ff_dim, a.temb_dim = B, S, D, attn.heads_per_device, block.mlp_hidden_dim, temb.shape[1]
+    lib = _lib.lib()
+    _run_block(a, lib.hdit_block_flux_single_workspace_bytes, lib.hdit_block_flux_single, "hdit_block_flux_single",
+               hidden_states.device, ptr.keep)
+    return hidden_out
+
+
+def block_cogvideox(block, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None, out_dtype=bf16):
+    """One CogVideoX block through ``hdit_block_cogvideox``; returns ``(hidden, encoder)`` like the block."""
+    attn, m = block.attn1, block.attn1.module
+    B, N, D = hidden_states.shape
+    Nt = encoder_hidden_states.shape[1]
+    _need(temb, bf16, "temb")
+    a, ptr = _lib.CogVideoXBlockArgs(), _ArgFiller()
+    qkv_w, qkv_b = attn._qkv.get()
+    for i, norm in ((1, block.norm1), (2, block.norm2)):
+        setattr(a, f"norm{i}_w", ptr(norm.linear.weight.data)), setattr(a, f"norm{i}_b", ptr(norm.linear.bias.data))
+        setattr(a, f"norm{i}_ln_w", ptr(norm.norm.weight.data)), setattr(a, f"norm{i}_ln_b", ptr(norm.norm.bias.data))
+    a.norm_eps = float(block.norm1.norm.eps)
+    a.qkv_w, a.qkv_b = ptr(qkv_w), ptr(qkv_b)
+    a.to_out_w = ptr(m.to_out[0].weight.data)
+    a.to_out_b = ptr(attn.output_bias.data) if attn.has_output_bias else None
+    for name in ("norm_q", "norm_k"):
+        n = getattr(m, name)
+        if n is not None:
+            setattr(a, name + "_w", ptr(n.weight.data) if n.weight is not None else None)
+            b = getattr(n, "bias", None)
+            setattr(a, name + "_b", ptr(b.data) if b is not None else None)
+    a.qk_norm_kind, a.qk_norm_eps = _norm_kind_of(m.norm_q), float(m.norm_q.eps) if m.norm_q is not None else 1e-6
+    ff = block.ff
+    a.ff_in_w, a.ff_in_b = ptr(ff.module.net[0].proj.weight.data), ptr(ff.module.net[0].proj.bias.data)
+    a.ff_out_w = ptr(ff.module.net[2].weight.data)
+    a.ff_out_b = ptr(ff.output_bias.data) if ff.has_output_bias else None
+    a.hidden_f32, a.encoder_f32 = _stream_tensor(hidden_states, "hidden_states"), _stream_tensor(encoder_hidden_states, "encoder_hidden_states")
+    if image_rotary_emb is not None:
+        cos, sin = image_rotary_emb
+        _need(cos, torch.float32, "cos"), _need(sin, torch.float32, "sin")
+        if tuple(cos.shape) != (N, D // attn.heads_per_device) or cos.shape != sin.shape or not (cos.is_contiguous() and sin.is_contiguous()):
+            raise ValueError("image_rotary_emb must be contiguous f32 [n_img, head_dim] tables")
+        a.rope_cos, a.rope_sin = ptr(cos), ptr(sin)
+    hidden_out = torch.empty(B, N, D, dtype=out_dtype, device=hidden_states.device)
+    encoder_out = torch.empty(B, Nt, D, dtype=out_dtype, device=hidden_states.device)
+    a.hidden, a.encoder, a.temb = ptr(hidden_states), ptr(encoder_hidden_states), ptr(temb.contiguous())
+    a.hidden_out, a.encoder_out, a.out_f32 = hidden_out.data_ptr(), encoder_out.data_ptr(), int(out_dtype == torch.float32)
+    a.batch, a.n_img, a.n_txt, a.dim, a.heads = B, N, Nt, D, attn.heads_per_device
+    a.ff_dim, a.temb_dim = ff.module.net[0].proj.weight.shape[0], temb.shape[1]
+    lib = _lib.lib()
+    _run_block(a, lib.hdit_block_cogvideox_workspace_bytes, lib.hdit_block_cogvideox, "hdit_block_cogvideox",
+               hidden_states.device, ptr.keep)
+    return hidden_out, encoder_out
+
+
 # ---------------------------------------------------------------------------
 # glue
 # ---------------------------------------------------------------------------

@@ -343,6 +343,91 @@ typedef struct hdit_sd3_block_args {
 int64_t hdit_block_sd3_workspace_bytes(const hdit_sd3_block_args* args);
 int hdit_block_sd3(const hdit_sd3_block_args* args, void* stream);
 
+/* The Flux double-stream block (diffusers FluxTransformerBlock, called at
+ * models/transformers/transformer_flux.py:160-165) as one call.  Weights as in
+ * hdit_sd3_block_weights (every member present; to_add_out_b is ignored: the
+ * reference's wrapper drops that bias in its Flux branch,
+ * layers/attention_processor.py:176-192,:284-305) plus the per-head norm weights
+ * of q, k of both streams (bf16 [head_dim] or NULL; qk_norm_kind as in
+ * hdit_qknorm_job, qk_norm_eps its eps).  rope_cos / rope_sin: f32 [n_txt + n_img,
+ * head_dim] over the joint [text, image] rows, or both NULL.  No stale K/V buffer
+ * at this level (the Python processor has it).  Tensor conventions and workspace
+ * as for hdit_block_sd3. */
+typedef struct hdit_flux_double_block_args {
+  hdit_sd3_block_weights w;
+  const void *norm_q_w, *norm_k_w, *norm_added_q_w, *norm_added_k_w;
+  const void* hidden;
+  const void* encoder;
+  const void* temb;
+  const float* rope_cos;
+  const float* rope_sin;
+  void* hidden_out;
+  void* encoder_out;
+  void* workspace;
+  int64_t workspace_bytes;
+  float qk_norm_eps;
+  int32_t qk_norm_kind;
+  int32_t batch, n_img, n_txt, dim, heads, ff_dim, temb_dim;
+  int32_t hidden_f32, encoder_f32, out_f32;
+} hdit_flux_double_block_args;
+
+int64_t hdit_block_flux_double_workspace_bytes(const hdit_flux_double_block_args* args);
+int hdit_block_flux_double(const hdit_flux_double_block_args* args, void* stream);
+
+/* The Flux single-stream block (diffusers FluxSingleTransformerBlock,
+ * transformer_flux.py:194-198) on the joint [text, image] sequence hidden
+ * [batch, seq, dim]: adaLN-ZeroSingle (norm_w [3 dim, temb_dim]: shift, scale,
+ * gate), q|k|v and proj_mlp in one launch, attention output and GELU(MLP) side by
+ * side in one buffer, proj_out [dim, dim + ff_dim] with the gated residual. */
+typedef struct hdit_flux_single_block_args {
+  const void *norm_w, *norm_b, *qkv_w, *qkv_b, *proj_mlp_w, *proj_mlp_b, *proj_out_w, *proj_out_b, *norm_q_w, *norm_k_w;
+  const void* hidden;
+  const void* temb;
+  const float* rope_cos;
+  const float* rope_sin;
+  void* hidden_out;
+  void* workspace;
+  int64_t workspace_bytes;
+  float qk_norm_eps;
+  int32_t qk_norm_kind;
+  int32_t batch, seq, dim, heads, ff_dim, temb_dim;
+  int32_t hidden_f32, out_f32;
+} hdit_flux_single_block_args;
+
+int64_t hdit_block_flux_single_workspace_bytes(const hdit_flux_single_block_args* args);
+int hdit_block_flux_single(const hdit_flux_single_block_args* args, void* stream);
+
+/* The CogVideoX block (diffusers CogVideoXBlock, called at
+ * models/transformers/cogvideox_transformer_3d.py:122-127): norm1_w / norm2_w
+ * [6 dim, temb_dim] (shift, scale, gate, enc_shift, enc_scale, enc_gate),
+ * norm*_ln_w / norm*_ln_b the affine LayerNorm [dim] shared by both streams
+ * (norm_eps), one projection set over the joint [text, video] rows, LayerNorm or
+ * RMSNorm per head on q, k (qk_norm_kind, weights / biases [head_dim]), rotation
+ * of the video rows only (rope_cos / rope_sin f32 [n_img, head_dim] or NULL),
+ * batch <= HDIT_GEMM_MAX_PROBLEMS / 2.  Returns hidden_out [batch, n_img, dim] and
+ * encoder_out [batch, n_txt, dim]. */
+typedef struct hdit_cogvideox_block_args {
+  const void *norm1_w, *norm1_b, *norm1_ln_w, *norm1_ln_b, *norm2_w, *norm2_b, *norm2_ln_w, *norm2_ln_b;
+  const void *qkv_w, *qkv_b, *to_out_w, *to_out_b, *norm_q_w, *norm_q_b, *norm_k_w, *norm_k_b;
+  const void *ff_in_w, *ff_in_b, *ff_out_w, *ff_out_b;
+  const void* hidden;
+  const void* encoder;
+  const void* temb;
+  const float* rope_cos;
+  const float* rope_sin;
+  void* hidden_out;
+  void* encoder_out;
+  void* workspace;
+  int64_t workspace_bytes;
+  float norm_eps, qk_norm_eps;
+  int32_t qk_norm_kind;
+  int32_t batch, n_img, n_txt, dim, heads, ff_dim, temb_dim;
+  int32_t hidden_f32, encoder_f32, out_f32;
+} hdit_cogvideox_block_args;
+
+int64_t hdit_block_cogvideox_workspace_bytes(const hdit_cogvideox_block_args* args);
+int hdit_block_cogvideox(const hdit_cogvideox_block_args* args, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -100,3 +100,67 @@ def test_block_sd3_refuses_bad_arguments(hdit):
     assert lib.hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
     assert lib.hdit_block_sd3(C.byref(a), None) == -1
     assert lib.hdit_block_sd3(None, None) == -1
+
+
+@pytest.mark.parametrize("stream_f32", [False, True])
+def test_block_flux_one_call_matches_python_blocks(hdit, stream_f32):
+    """``hdit_block_flux_double`` and ``hdit_block_flux_single`` against the Python blocks (bit-identical) and the
+    oracle."""
+    from hetu_dit_amd import blocks, synthetic
+    from hetu_dit_amd.runtime_state import get_runtime_state
+
+    print(f"hdit_block_flux_* fp32 stream={stream_f32}", flush=True)
+    B, Nt, gh, gw, D, H, hd = 2, 40, 12, 16, 512, 4, 128
+    N = gh * gw
+    cos, sin = synthetic.rope_table(synthetic.flux_ids(Nt, gh, gw), (16, 56, 56))
+    rope = (cos.to(DEV), sin.to(DEV))
+    dbl = synthetic.init_module_(blocks.FluxTransformerBlock(D, H, hd), 21)
+    sgl = synthetic.init_module_(blocks.FluxSingleTransformerBlock(D, H, hd), 22)
+    p_dbl, p_sgl = oracle_params(dbl), oracle_params(sgl)
+    dbl, sgl = dbl.to(DEV), sgl.to(DEV)
+    x, e, t = synthetic.randn_bf16((B, N, D), 23).to(DEV), synthetic.randn_bf16((B, Nt, D), 24).to(DEV), synthetic.randn_bf16((B, D), 25).to(DEV)
+    dt = torch.bfloat16
+    if stream_f32:
+        x, e, dt = x.float() + 1e-3, e.float() - 1e-3, torch.float32
+        dbl.stream_dtype = sgl.stream_dtype = torch.float32
+    enc_py, hid_py = dbl(hidden_states=x, encoder_hidden_states=e, temb=t, image_rotary_emb=rope)
+    enc_c, hid_c = hdit.ops.block_flux_double(dbl, x, e, t, rope, out_dtype=dt)
+    torch.cuda.synchronize()
+    assert torch.equal(hid_c, hid_py) and torch.equal(enc_c, enc_py)
+    o_enc, o_hid = oracle.flux_double_block(p_dbl, x.float().cpu(), e.float().cpu(), t.float().cpu(), (cos, sin), H)
+    assert_parity(hid_c, o_hid, what="hdit_block_flux_double hidden")
+    assert_parity(enc_c, o_enc, what="hdit_block_flux_double encoder")
+    get_runtime_state().max_condition_sequence_length = Nt
+    joint = torch.cat([e, x], 1).contiguous()
+    out_py = sgl(hidden_states=joint, temb=t, image_rotary_emb=rope)
+    out_c = hdit.ops.block_flux_single(sgl, joint, t, rope, out_dtype=dt)
+    torch.cuda.synchronize()
+    assert torch.equal(out_c, out_py)
+    assert_parity(out_c, oracle.flux_single_block(p_sgl, joint.float().cpu(), t.float().cpu(), (cos, sin), H, n_text=Nt),
+                  what="hdit_block_flux_single")
+
+
+@pytest.mark.parametrize("stream_f32", [False, True])
+def test_block_cogvideox_one_call_matches_python_block(hdit, stream_f32):
+    from hetu_dit_amd import blocks, synthetic
+
+    print(f"hdit_block_cogvideox fp32 stream={stream_f32}", flush=True)
+    B, Nt, grid, D, H, hd = 2, 26, (3, 6, 8), 256, 4, 64
+    N = grid[0] * grid[1] * grid[2]
+    cos, sin = synthetic.rope_table(synthetic.cogvideox_positions(*grid), (16, 24, 24))
+    rope = (cos.to(DEV), sin.to(DEV))
+    blk = synthetic.init_module_(blocks.CogVideoXBlock(D, H, hd, time_embed_dim=64), 31)
+    params = oracle_params(blk)
+    blk = blk.to(DEV)
+    x, e, t = synthetic.randn_bf16((B, N, D), 32).to(DEV), synthetic.randn_bf16((B, Nt, D), 33).to(DEV), synthetic.randn_bf16((B, 64), 34).to(DEV)
+    dt = torch.bfloat16
+    if stream_f32:
+        x, e, dt = x.float() + 1e-3, e.float() - 1e-3, torch.float32
+        blk.stream_dtype = torch.float32
+    hid_py, enc_py = blk(hidden_states=x, encoder_hidden_states=e, temb=t, image_rotary_emb=rope)
+    hid_c, enc_c = hdit.ops.block_cogvideox(blk, x, e, t, rope, out_dtype=dt)
+    torch.cuda.synchronize()
+    assert torch.equal(hid_c, hid_py) and torch.equal(enc_c, enc_py)
+    o_hid, o_enc = oracle.cogvideox_block(params, x.float().cpu(), e.float().cpu(), t.float().cpu(), (cos, sin), H)
+    assert_parity(hid_c, o_hid, what="hdit_block_cogvideox hidden")
+    assert_parity(enc_c, o_enc, what="hdit_block_cogvideox encoder")
