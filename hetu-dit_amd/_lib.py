@@ -160,8 +160,6 @@ SIGNATURES = {
     "hdit_last_error": (C.c_char_p, []),
     "hdit_gemm_bf16": (C.c_int, [C.POINTER(GemmProblem), C.c_int, C.c_void_p]),
     "hdit_attn_fwd_bf16": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p]),
-    "hdit_attn_workspace_bytes": (C.c_int64, [C.POINTER(AttnArgs)]),
-    "hdit_attn_fwd_bf16_ws": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_int64, C.c_void_p]),
     "hdit_attn_absmax": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p]),
     "hdit_attn_fp8_workspace_bytes": (C.c_int64, [C.POINTER(AttnArgs)]),
     "hdit_attn_fwd_fp8": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p, C.c_void_p]),

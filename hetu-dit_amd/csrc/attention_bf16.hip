@@ -50,32 +50,6 @@ struct AttnParams {
   float scale_log2;
 };
 
-// Work split of the balanced launch.  A "unit" is one query tile of one (batch, head) and costs NT key tiles;
-// a launch of whole units runs ceil(units / resident workgroups) rounds, the last one partly empty (1.69 -> 2
-// for the SD3 shape, 0.38 -> 1 for a PipeFusion patch).  The balanced launch instead lines all (unit, key tile)
-// pairs of a group up, unit-major, and gives each of the group's `slots` workgroups an equal contiguous share:
-// workgroup s works on pairs [s*I/slots, (s+1)*I/slots), I = units*NT.  A share covers the tail of one unit,
-// whole units, and the head of another; a unit that lies inside one share is finished and written as usual,
-// the (at most two) incomplete pieces of a share go to a workspace as un-normalised fp32 accumulators with their
-// running reference and row sums, and attn_merge_kernel adds the pieces of every divided unit up.  Groups are
-// the 8 XCDs when batch*heads divides by 8 (all query tiles of a (batch, head) then share one L2), else one.
-struct Balance {
-  float* part;   // [groups * slots][2] pieces of PART_FLOATS each
-  int groups, slots, units;  // per group: workgroups, units
-  int q_tiles, nt;
-};
-
-__host__ __device__ inline int64_t share_begin(int s, int slots, int64_t total) { return (int64_t)s * total / slots; }
-// the workgroup whose share holds pair i
-__host__ __device__ inline int share_of(int64_t i, int slots, int64_t total) {
-  int s = (int)(i * slots / total);
-  while (s + 1 < slots && share_begin(s + 1, slots, total) <= i) s++;
-  while (s > 0 && share_begin(s, slots, total) > i) s--;
-  return s;
-}
-template <int HD>
-constexpr int part_floats() { return NWAVE * (2 * (HD / 32) * 16 * 64 + 4 * 64); }
-
 template <int HD>
 struct Lds {
   // K and V tiles come straight from global memory (global_load_lds_dwordx4: no staging registers, no
@@ -125,31 +99,8 @@ __device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
 // accumulator rescale (the most expensive VALU block after the exponentials) is skipped for most tiles.
 constexpr float RESCALE_THRESHOLD = 8.0f;
 
-// normalise and write O[q][d] of one wave: lane owns q = qb*32 + l32, d = 32*db + 8*(v/4) + 4*lh + v%4
-template <int DB>
-__device__ __forceinline__ void write_output(const AttnParams& P, int b, int h, int q0, int l32, int lh,
-                                             const f32x16 (&oacc)[DB][2], const float (&l_run)[2]) {
-#pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(l_run[qb]), __float_as_int(l_run[qb]), false, false);
-    const float inv = 1.0f / (__int_as_float(sw[0]) + __int_as_float(sw[1]));
-    const int r = q0 + qb * 32 + l32;
-    if (r >= P.sq) continue;
-    __bf16* op = (__bf16*)row_ptr(P.o, b, h, r);
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        i32x2 out;
-        out[0] = (int)hdit::pack2(oacc[db][qb][g * 4 + 0] * inv, oacc[db][qb][g * 4 + 1] * inv);
-        out[1] = (int)hdit::pack2(oacc[db][qb][g * 4 + 2] * inv, oacc[db][qb][g * 4 + 3] * inv);
-        *(i32x2*)(op + db * 32 + g * 8 + lh * 4) = out;
-      }
-  }
-}
-
-template <int HD, bool BALANCED>
-__global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const AttnParams P, int q_tiles, const Balance bal) {
+template <int HD>
+__global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const AttnParams P, int q_tiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using L = Lds<HD>;
   constexpr int KS = HD / 16;       // k-steps of the S^T MFMA (over head dim)
@@ -163,45 +114,35 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
-  const int NT = (P.skv + BKV - 1) / BKV;
-  // ---- which (unit, key tile) pairs this workgroup works on
-  int group, units_loc;     // group = XCD when workgroups are dealt to XCDs by id
-  bool by_xcd;
-  int64_t it, it_end;       // pairs [it, it_end) of the group's unit-major list
-  if constexpr (BALANCED) {
-    by_xcd = bal.groups == 8;
-    group = by_xcd ? (int)(blockIdx.x & 7) : 0;
-    const int sl = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
-    units_loc = bal.units;
-    it = share_begin(sl, bal.slots, (int64_t)bal.units * NT);
-    it_end = share_begin(sl + 1, bal.slots, (int64_t)bal.units * NT);
-  } else {
-    // One unit per workgroup.  Workgroups go to the 8 XCDs round-robin by id, and each XCD has its own L2: all
-    // query tiles of one (batch, head) run on one XCD, so that its K and V are fetched into one L2 instead of
-    // eight.  Within that, the partly filled last query tiles (some of their waves have no rows and skip the
-    // arithmetic) come after all full ones: workgroups are placed in id order, one per CU first, so when a
-    // launch has a few more workgroups than CUs it is the light ones that share a CU with a full one.
-    const int nbh = gridDim.x / q_tiles;
-    by_xcd = nbh % 8 == 0;
-    group = by_xcd ? (int)(blockIdx.x & 7) : 0;
-    const int slot = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
-    const int nbh_loc = by_xcd ? nbh / 8 : nbh;
-    units_loc = nbh_loc * q_tiles;
-    int unit = slot;
-    if (q_tiles > 1 && P.sq % BQ != 0) {
-      const int heavy = nbh_loc * (q_tiles - 1);
-      unit = slot < heavy ? (slot / (q_tiles - 1)) * q_tiles + slot % (q_tiles - 1) : (slot - heavy) * q_tiles + q_tiles - 1;
+  // Workgroups go to the 8 XCDs round-robin by id, and each XCD has its own L2: all query tiles of one
+  // (batch, head) run on one XCD, so that its K and V are fetched into one L2 instead of eight.  Within that,
+  // the partly filled last query tiles (some of their waves have no rows and skip the arithmetic) come after
+  // all full ones: workgroups are placed in id order, one per CU first, so when a launch has a few more
+  // workgroups than CUs it is the light ones that share a CU with a full one.
+  const int nbh = gridDim.x / q_tiles;
+  const bool by_xcd = nbh % 8 == 0;
+  const int slot = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int nbh_loc = by_xcd ? nbh / 8 : nbh;
+  int qt = slot % q_tiles, bhl = slot / q_tiles;
+  if (q_tiles > 1 && P.sq % BQ != 0) {
+    const int heavy = nbh_loc * (q_tiles - 1);
+    if (slot < heavy) {
+      qt = slot % (q_tiles - 1);
+      bhl = slot / (q_tiles - 1);
+    } else {
+      qt = q_tiles - 1;
+      bhl = slot - heavy;
     }
-    it = (int64_t)unit * NT;
-    it_end = it + NT;
   }
-  (void)units_loc;
-  int b = 0, h = 0, q0 = 0;
-  bool active = false;
+  const int bh = by_xcd ? bhl * 8 + (int)(blockIdx.x & 7) : bhl;
+  const int b = bh / P.heads, h = bh % P.heads;
+  const int q0 = qt * BQ + wave * WQ;
+  // a wave past the last query row still stages K/V tiles and meets the barriers, but does no arithmetic
+  const bool active = __builtin_amdgcn_readfirstlane(q0 < P.sq);
+
   // ---- Q fragments: lane holds q row (qb*32 + l32), d = 16*ks + 8*lh .. +7
   bf16x8 qf[2][L::Q_IN_LDS ? 1 : KS];
   unsigned char* qlds = lds + L::Q_OFF + wave * L::Q_WAVE_BYTES;
-  auto load_q = [&]() __attribute__((always_inline)) {
   if constexpr (L::Q_IN_LDS) {
     // the wave's 64 query rows, 16 lanes per row (coalesced 256-byte rows), into its private LDS region;
     // only this wave reads them back, so its own wait for the writes is all the synchronisation needed
@@ -232,7 +173,6 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
       }
     }
   }
-  };
 
   // ---- K/V tile staging: global -> registers -> LDS.  A tile that lies inside one segment is addressed as
   // (wave-uniform base) + (loop-invariant per-thread offset); the tile that straddles the segment boundary
@@ -253,7 +193,10 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     voff[0][i] = (unsigned)((row * P.v.ss0 + dma_vc * 8) * 2);
     voff[1][i] = (unsigned)((row * P.v.ss1 + dma_vc * 8) * 2);
   }
-  const unsigned char *kb0 = nullptr, *kb1 = nullptr, *vb0 = nullptr, *vb1 = nullptr;  // K / V of the unit's (b, h)
+  const unsigned char* kb0 = (const unsigned char*)(P.k.p0 + b * P.k.sb0 + h * P.k.sh0);
+  const unsigned char* kb1 = (const unsigned char*)(P.k.p1 + b * P.k.sb1 + h * P.k.sh1);
+  const unsigned char* vb0 = (const unsigned char*)(P.v.p0 + b * P.v.sb0 + h * P.v.sh0);
+  const unsigned char* vb1 = (const unsigned char*)(P.v.p1 + b * P.v.sb1 + h * P.v.sh1);
   const int len0 = P.k.len0;
   // tile t straight into LDS stage `stage`
   auto dma_tile = [&](int t, int stage) {
@@ -285,29 +228,24 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
       }
     }
   };
+  f32x16 oacc[DB][2];
+#pragma unroll
+  for (int i = 0; i < DB; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) oacc[i][j][v] = 0.f;
   // running reference m of the online softmax (log2 units) and running sum per query column.  With FOLD the
   // accumulators of a score block start from negm = -m (the same value in all 16 entries: a lane owns one
   // query column per qb) and m starts at 0 until the first tile sets it to that tile's column maxima.
-  f32x16 oacc[DB][2];
-  float m_run[2], l_run[2];
+  float m_run[2] = {FOLD ? 0.f : -INFINITY, FOLD ? 0.f : -INFINITY};
+  float l_run[2] = {0.f, 0.f};
   f32x16 negm[2];
-  bool first;
-  auto reset_state = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < DB; i++)
+  for (int qb = 0; qb < 2; qb++)
 #pragma unroll
-      for (int j = 0; j < 2; j++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) oacc[i][j][v] = 0.f;
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-      m_run[qb] = FOLD ? 0.f : -INFINITY;
-      l_run[qb] = 0.f;
-#pragma unroll
-      for (int v = 0; v < 16; v++) negm[qb][v] = 0.f;
-    }
-    first = true;
-  };
+    for (int v = 0; v < 16; v++) negm[qb][v] = 0.f;
+  bool first = true;
 
   // lane-constant part of the V^T transpose-read address:
   // 16-lane group G = lane/16, x = lane%16: key row 4*(G/2) + x/4, column 16*(G%2) + 4*(x%4)
@@ -479,133 +417,54 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const
     }
   };
 
-  bool first_piece = true;
-  while (it < it_end) {
-    // ---- the next piece: key tiles [ka, kb) of one unit
-    const int unit = (int)(it / NT), ka = (int)(it - (int64_t)unit * NT);
-    const int kb = (int)min((int64_t)NT, (int64_t)ka + (it_end - it));
-    it += kb - ka;
-    const int qt = unit % q_tiles, bhl = unit / q_tiles;
-    const int bh = by_xcd ? bhl * 8 + group : bhl;
-    b = bh / P.heads;
-    h = bh % P.heads;
-    q0 = qt * BQ + wave * WQ;
-    // a wave past the last query row still stages K/V tiles and meets the barriers, but does no arithmetic
-    active = __builtin_amdgcn_readfirstlane(q0 < P.sq);
-    kb0 = (const unsigned char*)(P.k.p0 + b * P.k.sb0 + h * P.k.sh0);
-    kb1 = (const unsigned char*)(P.k.p1 + b * P.k.sb1 + h * P.k.sh1);
-    vb0 = (const unsigned char*)(P.v.p0 + b * P.v.sb0 + h * P.v.sh0);
-    vb1 = (const unsigned char*)(P.v.p1 + b * P.v.sb1 + h * P.v.sh1);
-    if constexpr (BALANCED) __syncthreads();  // every wave is done with the previous piece's tiles
-    load_q();
-    reset_state();
-
-    // Tile t+1 is fetched while tile t is worked on: its requests are issued behind the barrier that published
-    // tile t, into the stage tile t-1 vacated; every wave waits for its own requests before the next barrier.
-    dma_tile(ka, ka & 1);
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  const int NT = (P.skv + BKV - 1) / BKV;
+  // Tile t+1 is fetched while tile t is worked on: its requests are issued behind the barrier that published
+  // tile t, into the stage tile t-1 vacated; every wave waits for its own requests before the next barrier.
+  dma_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  if (NT > 1) dma_tile(1, 1);
+  auto next_tile = [&](int t) {  // end of iteration t: publish tile t+1, start fetching tile t+2
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile t+1 has landed
     __syncthreads();
-    if (ka + 1 < kb) dma_tile(ka + 1, (ka + 1) & 1);
-    auto next_tile = [&](int t) {  // end of iteration t: publish tile t+1, start fetching tile t+2
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile t+1 has landed
-      __syncthreads();
-      if (t + 2 < kb) dma_tile(t + 2, t & 1);
-    };
-
-    if (!active) {
-      // no query rows: stage this wave's share of every K/V tile and meet the same barriers, nothing else
-      for (int t = ka; t < kb - 1; t++) next_tile(t);
-      __builtin_amdgcn_s_waitcnt(0x0f70);
-      first_piece = false;
-      continue;
-    }
-    for (int t = ka; t < kb - 1; t++) {
-      tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
-      next_tile(t);
-    }
-    {
-      const int t = kb - 1;
-      const int valid = P.skv - t * BKV;
-      if (valid < BKV) tile_compute(lds + (t & 1) * L::STAGE, std::true_type{}, valid);
-      else tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
-    }
-
-    if (!BALANCED || (ka == 0 && kb == NT)) {
-      write_output<DB>(P, b, h, q0, l32, lh, oacc, l_run);
-    } else {
-      // an incomplete piece: accumulators as they lie in the registers ([qb][db][v/4][lane][4], every store a
-      // contiguous KiB per wave), then the running reference and this lane's half of the row sum per qb
-      float* pw = bal.part + ((int64_t)blockIdx.x * 2 + (first_piece ? 0 : 1)) * part_floats<HD>() + wave * (part_floats<HD>() / NWAVE);
-#pragma unroll
-      for (int qb = 0; qb < 2; qb++) {
-#pragma unroll
-        for (int db = 0; db < DB; db++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            f32x4 v4 = {oacc[db][qb][g * 4 + 0], oacc[db][qb][g * 4 + 1], oacc[db][qb][g * 4 + 2], oacc[db][qb][g * 4 + 3]};
-            *(f32x4*)(pw + (((qb * DB + db) * 4 + g) * 64 + lane) * 4) = v4;
-          }
-        pw[2 * DB * 16 * 64 + qb * 64 + lane] = m_run[qb];
-        pw[2 * DB * 16 * 64 + (2 + qb) * 64 + lane] = l_run[qb];
-      }
-    }
-    first_piece = false;
-  }
-}
-
-// Adds the pieces of every unit that the balanced launch divided between workgroups: one workgroup per unit, a
-// thread takes the role the same thread of attn_fwd_kernel had (same rows, same accumulator entries).
-template <int HD>
-__global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams P, const Balance bal) {
-  constexpr int DB = HD / 32;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lh = lane >> 5;
-  const bool by_xcd = bal.groups == 8;
-  const int group = by_xcd ? (int)(blockIdx.x & 7) : 0;
-  const int unit = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
-  const int64_t total = (int64_t)bal.units * bal.nt, u0 = (int64_t)unit * bal.nt;
-  const int s_first = share_of(u0, bal.slots, total), s_last = share_of(u0 + bal.nt - 1, bal.slots, total);
-  if (s_first == s_last) return;  // finished by one workgroup, already written
-  const int qt = unit % bal.q_tiles, bhl = unit / bal.q_tiles;
-  const int bh = by_xcd ? bhl * 8 + group : bhl;
-  const int b = bh / P.heads, h = bh % P.heads;
-  const int q0 = qt * BQ + wave * WQ;
-  if (q0 >= P.sq) return;
-  f32x16 oacc[DB][2];
-  float m_all[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
-  auto piece = [&](int s) {
-    // the piece of this unit in share s: its first piece if the share starts inside the unit, else its last
-    const bool is_first = share_begin(s, bal.slots, total) >= u0;
-    const int wg = by_xcd ? s * 8 + group : s;
-    return bal.part + ((int64_t)wg * 2 + (is_first ? 0 : 1)) * part_floats<HD>() + wave * (part_floats<HD>() / NWAVE);
+    if (t + 2 < NT) dma_tile(t + 2, t & 1);
   };
-  for (int s = s_first; s <= s_last; s++) {
-    const float* pw = piece(s);
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) m_all[qb] = fmaxf(m_all[qb], pw[2 * DB * 16 * 64 + qb * 64 + lane]);
+
+  if (!active) {
+    // no query rows: stage this wave's share of every K/V tile and meet the same barriers, nothing else
+    for (int t = 0; t < NT - 1; t++) next_tile(t);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    return;
   }
-#pragma unroll
-  for (int i = 0; i < DB; i++)
-#pragma unroll
-    for (int j = 0; j < 2; j++)
-#pragma unroll
-      for (int v = 0; v < 16; v++) oacc[i][j][v] = 0.f;
-  for (int s = s_first; s <= s_last; s++) {
-    const float* pw = piece(s);
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-      const float w = __builtin_amdgcn_exp2f(pw[2 * DB * 16 * 64 + qb * 64 + lane] - m_all[qb]);
-      l_run[qb] += w * pw[2 * DB * 16 * 64 + (2 + qb) * 64 + lane];
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const f32x4 v4 = *(const f32x4*)(pw + (((qb * DB + db) * 4 + g) * 64 + lane) * 4);
-#pragma unroll
-          for (int e = 0; e < 4; e++) oacc[db][qb][g * 4 + e] += w * v4[e];
-        }
-    }
+  for (int t = 0; t < NT - 1; t++) {
+    tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
+    next_tile(t);
   }
-  write_output<DB>(P, b, h, q0, l32, lh, oacc, l_run);
+  {
+    const int t = NT - 1;
+    const int valid = P.skv - t * BKV;
+    if (valid < BKV) tile_compute(lds + (t & 1) * L::STAGE, std::true_type{}, valid);
+    else tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
+  }
+
+  // ---- normalise and write O[q][d]: lane owns q = qb*32 + l32, d = 32*db + 8*(v/4) + 4*lh + v%4
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(l_run[qb]), __float_as_int(l_run[qb]), false, false);
+    const float inv = 1.0f / (__int_as_float(sw[0]) + __int_as_float(sw[1]));
+    const int r = q0 + qb * 32 + l32;
+    if (r >= P.sq) continue;
+    __bf16* op = (__bf16*)row_ptr(P.o, b, h, r);
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        i32x2 out;
+        out[0] = (int)hdit::pack2(oacc[db][qb][g * 4 + 0] * inv, oacc[db][qb][g * 4 + 1] * inv);
+        out[1] = (int)hdit::pack2(oacc[db][qb][g * 4 + 2] * inv, oacc[db][qb][g * 4 + 3] * inv);
+        *(i32x2*)(op + db * 32 + g * 8 + lh * 4) = out;
+      }
+  }
 }
 
 bool seg_ok(const hdit_seq_segment& s, bool need_ptr) {
@@ -649,80 +508,9 @@ int attn_validate(const hdit_attn_args* a) {
 }
 }  // namespace hdit_host
 
-namespace {
-constexpr int NUM_CU = 256;  // MI355X
-
-// The balanced launch is taken when a workspace is there and the equal shares (plus a few tiles of overhead per
-// piece: pipeline refill, Q reload, the piece written out and merged) are at least a quarter shorter than the
-// rounds of whole units -- in practice launches of less than one round (a PipeFusion patch: 192 units on 512
-// resident workgroups, 10-14 % faster).  Between one and two rounds (the SD3 step: 1.69) both launches take the
-// same time: the chip runs at its power limit, the CUs that idle in the last round of whole units lend their
-// power budget to the busy ones, and the balanced launch only trades that for the traffic of the pieces.
-struct Plan {
-  bool balanced;
-  Balance bal;
-  int q_tiles, wgs;
-};
-Plan make_plan(int batch, int heads, int head_dim, int sq, int skv, bool have_workspace) {
-  Plan p;
-  p.q_tiles = (sq + BQ - 1) / BQ;
-  const int nbh = batch * heads;
-  const int64_t units = (int64_t)nbh * p.q_tiles;
-  const int nt = (skv + BKV - 1) / BKV;
-  const int capacity = NUM_CU * (head_dim == 64 ? 2 : 1);
-  const int groups = nbh % 8 == 0 ? 8 : 1;
-  const int64_t plain = (units + capacity - 1) / capacity * nt;
-  const int64_t shares = (units * nt + capacity - 1) / capacity + 3;
-  p.balanced = have_workspace && shares * 4 <= plain * 3 && units / groups * nt >= capacity / groups && units < (1 << 24);
-  p.wgs = p.balanced ? capacity : (int)units;
-  p.bal.part = nullptr;
-  p.bal.groups = groups;
-  p.bal.slots = capacity / groups;
-  p.bal.units = (int)(units / groups);
-  p.bal.q_tiles = p.q_tiles;
-  p.bal.nt = nt;
-  return p;
-}
-int64_t plan_workspace_bytes(int head_dim) {
-  const int capacity = NUM_CU * (head_dim == 64 ? 2 : 1);
-  return (int64_t)capacity * 2 * (head_dim == 64 ? part_floats<64>() : part_floats<128>()) * 4;
-}
-
-template <int HD, bool BALANCED>
-int set_lds_limit() {
-  static std::atomic<bool> done{false};  // setting the attribute twice from two threads is harmless
-  if (Lds<HD>::TOTAL > 64 * 1024 && !done.load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute((const void*)attn_fwd_kernel<HD, BALANCED>, hipFuncAttributeMaxDynamicSharedMemorySize, Lds<HD>::TOTAL) != hipSuccess)
-      return HDIT_ELAUNCH;
-    done.store(true, std::memory_order_release);
-  }
-  return HDIT_OK;
-}
-
-template <int HD>
-int launch(const AttnParams& P, const Plan& plan, int units_total, hipStream_t s) {
-  if (plan.balanced) {
-    if (set_lds_limit<HD, true>() != HDIT_OK) return HDIT_ELAUNCH;
-    hipLaunchKernelGGL((attn_fwd_kernel<HD, true>), dim3((unsigned)plan.wgs), dim3(256), Lds<HD>::TOTAL, s, P, plan.q_tiles, plan.bal);
-    hipLaunchKernelGGL((attn_merge_kernel<HD>), dim3((unsigned)units_total), dim3(256), 0, s, P, plan.bal);
-  } else if constexpr (HD == 128) {
-    // one unit per workgroup, expressed as shares of exactly one unit each: this instantiation keeps its tile
-    // loop free of scratch reloads, the whole-unit one does not at d = 128
-    Balance one = plan.bal;
-    one.slots = one.units;
-    if (set_lds_limit<HD, true>() != HDIT_OK) return HDIT_ELAUNCH;
-    hipLaunchKernelGGL((attn_fwd_kernel<HD, true>), dim3((unsigned)plan.wgs), dim3(256), Lds<HD>::TOTAL, s, P, plan.q_tiles, one);
-  } else {
-    if (set_lds_limit<HD, false>() != HDIT_OK) return HDIT_ELAUNCH;
-    hipLaunchKernelGGL((attn_fwd_kernel<HD, false>), dim3((unsigned)plan.wgs), dim3(256), Lds<HD>::TOTAL, s, P, plan.q_tiles, plan.bal);
-  }
-  return HDIT_OK;
-}
-
-int fwd_bf16(const hdit_attn_args* a, void* workspace, int64_t workspace_bytes, void* stream, const char* what) {
+extern "C" __attribute__((visibility("default"))) int hdit_attn_fwd_bf16(const hdit_attn_args* a, void* stream) {
   int rc = hdit_host::attn_validate(a);
   if (rc != HDIT_OK) return rc;
-  if (workspace && (((uintptr_t)workspace) & 15)) return HDIT_EINVAL;
   AttnParams P;
   P.q = make_seg(a->q);
   P.k = make_seg(a->k);
@@ -734,32 +522,20 @@ int fwd_bf16(const hdit_attn_args* a, void* workspace, int64_t workspace_bytes, 
   if (P.sq == 0) return HDIT_OK;
   float scale = a->scale > 0.f ? a->scale : 1.0f / sqrtf((float)a->head_dim);
   P.scale_log2 = scale * 1.4426950408889634f;
-  Plan plan = make_plan(a->batch, a->heads, a->head_dim, P.sq, P.skv, workspace != nullptr && workspace_bytes >= plan_workspace_bytes(a->head_dim));
-  plan.bal.part = (float*)workspace;
-  const int units_total = plan.q_tiles * a->batch * a->heads;
-  rc = a->head_dim == 64 ? launch<64>(P, plan, units_total, (hipStream_t)stream) : launch<128>(P, plan, units_total, (hipStream_t)stream);
-  if (rc != HDIT_OK) return rc;
-  return hdit_host::check_launch(what);
-}
-}  // namespace
-
-extern "C" __attribute__((visibility("default"))) int hdit_attn_fwd_bf16(const hdit_attn_args* a, void* stream) {
-  return fwd_bf16(a, nullptr, 0, stream, "hdit_attn_fwd_bf16");
-}
-
-namespace hdit_host {
-int64_t attn_workspace_bytes_for(int batch, int heads, int head_dim, int sq, int skv) {
-  if (sq <= 0 || skv <= 0) return 0;
-  return make_plan(batch, heads, head_dim, sq, skv, true).balanced ? plan_workspace_bytes(head_dim) : 0;
-}
-}  // namespace hdit_host
-
-extern "C" __attribute__((visibility("default"))) int64_t hdit_attn_workspace_bytes(const hdit_attn_args* a) {
-  if (hdit_host::attn_validate(a) != HDIT_OK) return -1;
-  return hdit_host::attn_workspace_bytes_for(a->batch, a->heads, a->head_dim, a->q[0].len + a->q[1].len, a->k[0].len + a->k[1].len);
-}
-
-extern "C" __attribute__((visibility("default"))) int hdit_attn_fwd_bf16_ws(const hdit_attn_args* a, void* workspace,
-                                                                            int64_t workspace_bytes, void* stream) {
-  return fwd_bf16(a, workspace, workspace_bytes, stream, "hdit_attn_fwd_bf16_ws");
+  int q_tiles = (P.sq + BQ - 1) / BQ;
+  dim3 grid((unsigned)(q_tiles * a->batch * a->heads)), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  if (a->head_dim == 64) {
+    hipLaunchKernelGGL(attn_fwd_kernel<64>, grid, block, Lds<64>::TOTAL, s, P, q_tiles);
+  } else {
+    static std::atomic<bool> attr{false};  // setting the attribute twice from two threads is harmless
+    if (!attr.load(std::memory_order_acquire)) {
+      if (hipFuncSetAttribute((const void*)attn_fwd_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              Lds<128>::TOTAL) != hipSuccess)
+        return HDIT_ELAUNCH;
+      attr.store(true, std::memory_order_release);
+    }
+    hipLaunchKernelGGL(attn_fwd_kernel<128>, grid, block, Lds<128>::TOTAL, s, P, q_tiles);
+  }
+  return hdit_host::check_launch("hdit_attn_fwd_bf16");
 }

@@ -24,8 +24,6 @@ struct Sd3Workspace {
   float* x1_txt;           // f32 [B, Nt, D]
   unsigned char* h_img;    // bf16 [B, Ni, F]
   unsigned char* h_txt;    // bf16 [B, Nt, F]
-  unsigned char* attn;     // scratch of the attention launch (hdit_attn_workspace_bytes)
-  int64_t attn_bytes;
   int64_t bytes;
 };
 
@@ -51,9 +49,6 @@ Sd3Workspace carve(const hdit_sd3_block_args* a, unsigned char* base) {
   w.x1_txt = (float*)take(text_out ? B * Nt * D * 4 : 0);
   w.h_img = take(B * Ni * F * 2);
   w.h_txt = take(text_out ? B * Nt * F * 2 : 0);
-  w.attn_bytes = hdit_host::attn_workspace_bytes_for(a->batch, a->heads, a->dim / a->heads, a->n_img + (a->skip_text_output ? 0 : a->n_txt),
-                                                     a->n_txt + (a->kv_buffer ? a->kv_rows : a->n_img));
-  w.attn = take(w.attn_bytes);
   w.bytes = off;
   return w;
 }
@@ -204,7 +199,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
     seg(at.o[1], ws.o_txt, Nt, D, Nt);
   }
   at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
-  if ((rc = hdit_attn_fwd_bf16_ws(&at, ws.attn, ws.attn_bytes, stream))) return rc;
+  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
 
   // 5. out-projections with the gated residual; the stream stays fp32 inside the block
   auto gated = [&](hdit_gemm_problem& p, const void* resid, int resid_f32, const float* gate, int64_t gate_stride, int rows,
@@ -298,8 +293,6 @@ bool head_dim_ok(int dim, int heads) { return heads > 0 && dim % heads == 0 && (
 struct FluxDoubleWs {
   float *emb_img, *emb_txt, *x1_img, *x1_txt;
   unsigned char *n_img, *n_txt, *qkv_img, *qkv_txt, *o_img, *o_txt, *h_img, *h_txt;
-  unsigned char* attn;  // scratch of the attention launch
-  int64_t attn_bytes;
   int64_t bytes;
 };
 FluxDoubleWs carve(const hdit_flux_double_block_args* a, void* base) {
@@ -312,8 +305,6 @@ FluxDoubleWs carve(const hdit_flux_double_block_args* a, void* base) {
   w.o_img = c.take(B * Ni * D * 2), w.o_txt = c.take(B * Nt * D * 2);
   w.x1_img = (float*)c.take(B * Ni * D * 4), w.x1_txt = (float*)c.take(B * Nt * D * 4);
   w.h_img = c.take(B * Ni * F * 2), w.h_txt = c.take(B * Nt * F * 2);
-  w.attn_bytes = hdit_host::attn_workspace_bytes_for(a->batch, a->heads, a->dim / a->heads, a->n_img + a->n_txt, a->n_img + a->n_txt);
-  w.attn = c.take(w.attn_bytes);
   w.bytes = c.off;
   return w;
 }
@@ -333,8 +324,6 @@ int validate(const hdit_flux_double_block_args* a) {
 struct FluxSingleWs {
   float* emb;
   unsigned char *n, *qkv, *cat;
-  unsigned char* attn;  // scratch of the attention launch
-  int64_t attn_bytes;
   int64_t bytes;
 };
 FluxSingleWs carve(const hdit_flux_single_block_args* a, void* base) {
@@ -345,8 +334,6 @@ FluxSingleWs carve(const hdit_flux_single_block_args* a, void* base) {
   w.n = c.take(B * S * D * 2);
   w.qkv = c.take(B * S * 3 * D * 2);
   w.cat = c.take(B * S * (D + F) * 2);
-  w.attn_bytes = hdit_host::attn_workspace_bytes_for(a->batch, a->heads, a->dim / a->heads, a->seq, a->seq);
-  w.attn = c.take(w.attn_bytes);
   w.bytes = c.off;
   return w;
 }
@@ -363,8 +350,6 @@ int validate(const hdit_flux_single_block_args* a) {
 struct CogWs {
   float *emb1, *emb2, *x1_h, *x1_e;
   unsigned char *joint, *qkv, *o, *h;
-  unsigned char* attn;  // scratch of the attention launch
-  int64_t attn_bytes;
   int64_t bytes;
 };
 CogWs carve(const hdit_cogvideox_block_args* a, void* base) {
@@ -377,8 +362,6 @@ CogWs carve(const hdit_cogvideox_block_args* a, void* base) {
   w.o = c.take(B * S * D * 2);
   w.x1_h = (float*)c.take(B * a->n_img * D * 4), w.x1_e = (float*)c.take(B * a->n_txt * D * 4);
   w.h = c.take(B * S * F * 2);
-  w.attn_bytes = hdit_host::attn_workspace_bytes_for(a->batch, a->heads, a->dim / a->heads, a->n_img + a->n_txt, a->n_img + a->n_txt);
-  w.attn = c.take(w.attn_bytes);
   w.bytes = c.off;
   return w;
 }
@@ -445,7 +428,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_flux_double(con
   seg(at.v[0], v_txt, Nt, ld3, hd, Nt), seg(at.v[1], v_img, Ni, ld3, hd, Ni);
   seg(at.o[0], ws.o_txt, Nt, D, hd, Nt), seg(at.o[1], ws.o_img, Ni, D, hd, Ni);
   at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
-  if ((rc = hdit_attn_fwd_bf16_ws(&at, ws.attn, ws.attn_bytes, stream))) return rc;
+  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
   // the reference's wrapper never adds the text out-projection bias back in its Flux branch
   // (layers/attention_processor.py:176-192,:284-305): to_add_out runs without bias
   probs[0] = problem(ws.o_img, D, w.to_out_w, w.to_out_b, ws.x1_img, D, B * Ni, D, D, 0);
@@ -496,7 +479,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_flux_single(con
   seg(at.q[0], q, S, ld3, hd, S), seg(at.k[0], k, S, ld3, hd, S), seg(at.v[0], v, S, ld3, hd, S);
   seg(at.o[0], ws.cat, S, ldc, hd, S);
   at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
-  if ((rc = hdit_attn_fwd_bf16_ws(&at, ws.attn, ws.attn_bytes, stream))) return rc;
+  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
   probs[0] = problem(ws.cat, ldc, a->proj_out_w, a->proj_out_b, a->hidden_out, D, B * S, D, D + F, 0);
   gated(probs[0], a->hidden, a->hidden_f32, ws.emb + 2 * D, md, S, a->out_f32);
   return hdit_gemm_bf16(probs, 1, stream);
@@ -538,7 +521,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_cogvideox(const
   seg(at.q[0], q, S, ld3, hd, S), seg(at.k[0], k, S, ld3, hd, S), seg(at.v[0], v, S, ld3, hd, S);
   seg(at.o[0], ws.o, S, D, hd, S);
   at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
-  if ((rc = hdit_attn_fwd_bf16_ws(&at, ws.attn, ws.attn_bytes, stream))) return rc;
+  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
   // one weight set over the joint rows, per-stream gates: per batch element a text and a video problem
   auto gated_pair = [&](const unsigned char* a_joint, int64_t lda, const void* wt, const void* bias, int kdim, const void* res_e,
                         int re_sz, const void* res_h, int rh_sz, const float* emb, void* out_e, int oe_sz, void* out_h, int oh_sz) {

@@ -70,6 +70,4 @@ __device__ __forceinline__ float silu_f(float x) {
 namespace hdit_host {
 void set_error(const char* msg);
 int check_launch(const char* what);
-// hdit_attn_workspace_bytes from the shapes alone
-int64_t attn_workspace_bytes_for(int batch, int heads, int head_dim, int sq, int skv);
 }  // namespace hdit_host

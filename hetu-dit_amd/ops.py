@@ -174,10 +174,6 @@ def _fill_segments(dst, tensors: Sequence[torch.Tensor], name: str) -> Tuple[int
     return B, total, H, D
 
 
-# default of attention(balanced=...)
-BALANCED_ATTENTION = True
-
-
 def attention_args(q, k, v, o, scale: float = 0.0) -> AttnArgs:
     a = AttnArgs()
     B, sq, H, D = _fill_segments(a.q, q, "q")
@@ -192,17 +188,10 @@ def attention_args(q, k, v, o, scale: float = 0.0) -> AttnArgs:
 
 
 def attention(q: Sequence[torch.Tensor], k: Sequence[torch.Tensor], v: Sequence[torch.Tensor],
-              out: Optional[Sequence[torch.Tensor]] = None, scale: float = 0.0, fp8: bool = False,
-              balanced: Optional[bool] = None):
+              out: Optional[Sequence[torch.Tensor]] = None, scale: float = 0.0, fp8: bool = False):
     """Joint non-causal attention.  q/k/v are lists of one or two [B, S, H, d]
     bf16 views (the segments of the joint sequence).  Returns the list of
-    output segments (allocated [B, S, H, d] contiguous when not given).
-    ``balanced`` (default: ``BALANCED_ATTENTION``) lets the bf16 launch divide
-    query tiles between workgroups through a scratch workspace when whole tiles
-    would leave CUs idle; how a launch is divided depends on its shapes, so two
-    launches that differ in the number of query rows round differently."""
-    if balanced is None:
-        balanced = BALANCED_ATTENTION
+    output segments (allocated [B, S, H, d] contiguous when not given)."""
     if out is None:
         out = [torch.empty(t.shape, dtype=bf16, device=t.device) for t in q]
     args = attention_args(q, k, v, out, scale)
@@ -219,13 +208,7 @@ def attention(q: Sequence[torch.Tensor], k: Sequence[torch.Tensor], v: Sequence[
                    lambda: lib.hdit_attn_fwd_fp8(C.byref(args), absmax.data_ptr(), ws.data_ptr(), _stream())),
               "hdit_attn_fwd_fp8")
     else:
-        nbytes = lib.hdit_attn_workspace_bytes(C.byref(args)) if balanced else 0
-        if nbytes > 0:
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=q[0].device)
-            check(_run("attn_bf16", flops, lambda: lib.hdit_attn_fwd_bf16_ws(C.byref(args), ws.data_ptr(), nbytes, _stream())),
-                  "hdit_attn_fwd_bf16_ws")
-        else:
-            check(_run("attn_bf16", flops, lambda: lib.hdit_attn_fwd_bf16(C.byref(args), _stream())), "hdit_attn_fwd_bf16")
+        check(_run("attn_bf16", flops, lambda: lib.hdit_attn_fwd_bf16(C.byref(args), _stream())), "hdit_attn_fwd_bf16")
     return list(out)
 
 

@@ -127,22 +127,6 @@ typedef struct hdit_attn_args {
 
 int hdit_attn_fwd_bf16(const hdit_attn_args* args, void* stream);
 
-/* hdit_attn_fwd_bf16 with a scratch workspace, which lets the launch balance
- * its work: instead of whole (batch, head, 256-query tile) units in rounds --
- * the last round partly empty: 1.69 units per resident workgroup run as 2
- * rounds, 0.38 as 1 -- every resident workgroup takes an equal contiguous share
- * of all (unit, 64-key tile) pairs, the pieces of a unit that was divided
- * between two workgroups go through the workspace (un-normalised fp32
- * accumulators + softmax statistics) and a second small kernel adds them up.
- * hdit_attn_workspace_bytes(args) is the size that needs (16-byte aligned,
- * caller-owned, contents irrelevant before and after), or 0 when the problem
- * would not be divided; with workspace NULL or smaller the call is
- * hdit_attn_fwd_bf16.  Which path runs depends on the shapes only, so results
- * are reproducible; against hdit_attn_fwd_bf16 they differ by fp32 rounding of
- * the merge.  No counterpart in the reference (same call site). */
-int64_t hdit_attn_workspace_bytes(const hdit_attn_args* args);
-int hdit_attn_fwd_bf16_ws(const hdit_attn_args* args, void* workspace, int64_t workspace_bytes, void* stream);
-
 /* Same contract on the fp8-e4m3 (OCP) MFMA path: Q, K, V are quantised with one
  * absmax scale per (batch, head) taken from `absmax` (f32 [3, batch, heads]:
  * q, k, v; written by hdit_attn_absmax), P is re-quantised per tile.  K and V

@@ -171,34 +171,6 @@ def test_attention_large_logits_and_scale(hdit):
     assert_parity(o, want, what="attention large logits")
 
 
-@pytest.mark.parametrize("B,H,hd,sq,skv,gain", [
-    (1, 8, 64, [1024], [333, 1024], 1.0),    # 32 units on 512 resident workgroups: every unit in ~16 pieces
-    (1, 24, 64, [256], [333, 4096], 4.0),    # one query tile per head, ragged last key tile, large logits
-    (1, 5, 64, [2000], [1999], 1.0),         # batch*heads not a multiple of 8: one group instead of one per XCD
-    (1, 8, 128, [300], [300, 900], 2.0),     # d = 128, a partly filled query tile
-    (2, 4, 128, [1111], [1111], 1.0),
-])
-def test_attention_balanced_launch(hdit, B, H, hd, sq, skv, gain):
-    """Launches of less than one round of whole query tiles are divided into equal shares of (query tile, key
-    tile) pairs, the pieces of a divided tile going through a workspace and a merge kernel
-    (hdit_attn_fwd_bf16_ws).  Checked against the oracle, and against the undivided launch on the same inputs."""
-    import ctypes as C
-
-    print(f"balanced attention B={B} H={H} hd={hd} sq={sq} skv={skv}", flush=True)
-    q = [rnd(B, n, H, hd, scale=gain, seed=1 + i) for i, n in enumerate(sq)]
-    k = [rnd(B, n, H, hd, scale=gain, seed=11 + i) for i, n in enumerate(skv)]
-    v = [rnd(B, n, H, hd, seed=21 + i) for i, n in enumerate(skv)]
-    qd, kd, vd = [g(t) for t in q], [g(t) for t in k], [g(t) for t in v]
-    args = hdit.ops.attention_args(qd, kd, vd, [torch.empty_like(t) for t in qd])
-    assert hdit._lib.lib().hdit_attn_workspace_bytes(C.byref(args)) > 0, "this shape is meant to be divided"
-    got = torch.cat(hdit.ops.attention(qd, kd, vd, balanced=True), 1)
-    plain = torch.cat(hdit.ops.attention(qd, kd, vd, balanced=False), 1)
-    torch.cuda.synchronize()
-    want = O.attention(torch.cat(q, 1).transpose(1, 2), torch.cat(k, 1).transpose(1, 2), torch.cat(v, 1).transpose(1, 2)).transpose(1, 2)
-    assert_parity(got, want, what="balanced attention")
-    assert_parity(got, plain.float().cpu(), rel=5e-3, cos=0.9999, what="balanced against undivided launch")
-
-
 @pytest.mark.parametrize("dim", [64, 1536, 3072, 4096 + 8])
 def test_layernorm_modulate(hdit, dim):
     B, T = 2, 37

@@ -264,7 +264,7 @@ def test_block_called_alone_after_a_stack_run_uses_its_own_temb(hdit):
     assert_parity(enc, o_enc, what="block alone with a new temb, encoder")
 
 
-def test_sd3_patches_skip_the_dropped_text_stream_bit_exact(hdit, monkeypatch):
+def test_sd3_patches_skip_the_dropped_text_stream_bit_exact(hdit):
     """For pipeline patches after the first the block loop drops every block's text output
     (transformer_sd3.py:131-146); the runner therefore asks the blocks not to compute it.  The image output of
     every patch must equal, bit for bit, what the same blocks return when they do compute the text stream."""
@@ -273,9 +273,6 @@ def test_sd3_patches_skip_the_dropped_text_stream_bit_exact(hdit, monkeypatch):
     from hetu_dit_amd.runtime_state import get_runtime_state
 
     B, N, Nt, D, H, L, P = 2, 1024, 333, 512, 8, 3, 4
-    # a launch of few query tiles is divided between workgroups by shape, and a patch with and without its text
-    # query rows is a different shape: bit equality is checked with that division switched off
-    monkeypatch.setattr(hdit.ops, "BALANCED_ATTENTION", False)
     starts = [N // P * i for i in range(P + 1)]
     stack = transformer.SD3TransformerBlocks(L, D, H, 64)
     synthetic.init_module_(stack, 101)
