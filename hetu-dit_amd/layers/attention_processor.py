@@ -426,25 +426,34 @@ class hetuDiTFluxAttnProcessor2_0(FluxAttnProcessor2_0):
             ]
         else:
             # patch mode: text rows and the image patch rows form this call's joint input
+            # The queries of all rows go to one [B, S, inner] tensor, the text rows' K|V to a small tensor of their
+            # own, and the image rows' K|V straight into this patch's rows of the stale buffer (one problem per batch
+            # element and destination: the destinations differ in batch stride) -- no copy afterwards.
             buf, start, end = get_cache_manager().kv_buffer(attn, B, N, inner, dev)
-            qkv = torch.empty(B, S, 3 * inner, dtype=torch.bfloat16, device=dev)
-            ops.gemm_launch([ops.gemm_problem(x2, w, qkv.view(-1, 3 * inner), b)] + extra_problems)
-            ops.copy_rows(qkv[:, n_txt:, inner:], buf[:, start:end])
-            q = qkv[:, :, :inner]
+            q = torch.empty(B, S, inner, dtype=torch.bfloat16, device=dev)
+            kv_txt = torch.empty(B, n_txt, 2 * inner, dtype=torch.bfloat16, device=dev)
+            x3 = x2.view(B, S, -1)
+            wq_, bq_ = attn._qkv.rows(0, inner)
+            wkv, bkv = attn._qkv.rows(inner, 2 * inner)
+            problems = [ops.gemm_problem(x2, wq_, q.view(-1, inner), bq_)]
+            for bi in range(B):
+                problems.append(ops.gemm_problem(x3[bi, :n_txt], wkv, kv_txt[bi], bkv))
+                problems.append(ops.gemm_problem(x3[bi, n_txt:], wkv, buf[bi, start:end], bkv))
+            ops.gemm_launch(problems + extra_problems)
             if cos is not None:
                 qc, qs = cos, sin
                 kc, ks = cos[n_txt:], sin[n_txt:]
                 tc, ts = cos[:n_txt], sin[:n_txt]
             else:
                 qc = qs = kc = ks = tc = ts = None
-            k_txt = qkv[:, :n_txt, inner:2 * inner]
+            k_txt = kv_txt[:, :, :inner]
             jobs = [
                 ops.qk_norm_rope_job(_heads(q, H), _norm_kind(m.norm_q), wq, None, qc, qs),
                 ops.qk_norm_rope_job(_heads(k_txt, H), _norm_kind(m.norm_k), wk, None, tc, ts),
                 ops.qk_norm_rope_job(_heads(buf[:, start:end, :inner], H), _norm_kind(m.norm_k), wk, None, kc, ks),
             ]
             k_segs = [_heads(k_txt, H), _heads(buf[:, :, :inner], H)]
-            v_segs = [_heads(qkv[:, :n_txt, 2 * inner:], H), _heads(buf[:, :, inner:], H)]
+            v_segs = [_heads(kv_txt[:, :, inner:], H), _heads(buf[:, :, inner:], H)]
         ops.qk_norm_rope(jobs, B, H, hd, eps)
         if out is None:
             out = torch.empty(B, S, inner, dtype=torch.bfloat16, device=dev)
