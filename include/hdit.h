@@ -313,6 +313,10 @@ int hdit_cfg_euler_step(const void* noise_uncond, const void* noise_cond, const 
  * norm1_context (f32 [batch, 6 dim] / [batch, 6 dim or 2 dim]); NULL => computed
  * here.  workspace: hdit_block_sd3_workspace_bytes(args) bytes, 256-byte aligned,
  * caller-owned, contents undefined afterwards.
+ * Arguments are validated before anything is enqueued.  A block is a sequence of
+ * this library's launches, so if a later launch is refused (HDIT_ELAUNCH from the
+ * runtime) the earlier ones are already on the stream and the outputs are
+ * undefined; the return code is that launch's.
  * ---------------------------------------------------------------------- */
 typedef struct hdit_sd3_block_weights {
   const void *norm1_w, *norm1_b, *norm1_context_w, *norm1_context_b;
