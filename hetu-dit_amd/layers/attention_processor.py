@@ -246,12 +246,24 @@ class hetuDiTAttentionWrapper(hetuDiTAttentionBaseWrapper):
             return out[:, n_txt:], out[:, :n_txt]
         if isinstance(proc, hetuDiTFluxAttnProcessor2_0) and encoder_hidden_states is None:
             return proc(self, hidden_states, encoder_hidden_states=None, **kwargs)
+        # [B, C, H, W] inputs are token sequences in channel-major layout (attention_processor.py:672-683); the
+        # outputs go back to that layout (:436-443), each with its own height and width
+        shape_img = hidden_states.shape if hidden_states.ndim == 4 else None
+        shape_txt = encoder_hidden_states.shape if encoder_hidden_states is not None and encoder_hidden_states.ndim == 4 else None
+        if shape_img is not None:
+            hidden_states = hidden_states.flatten(2).transpose(1, 2).contiguous()
+        if shape_txt is not None:
+            encoder_hidden_states = encoder_hidden_states.flatten(2).transpose(1, 2).contiguous()
         o_img, o_txt = proc(self, hidden_states, encoder_hidden_states=encoder_hidden_states, **kwargs)
         problems, outs = self.out_proj_problems(o_img, o_txt)
         ops.gemm_launch(problems)
-        if len(outs) == 2:
-            return outs[0], outs[1]
-        return outs[0], o_txt  # context_pre_only: raw attention slice (attention_processor.py:420-421)
+        out_img = outs[0]
+        out_txt = outs[1] if len(outs) == 2 else o_txt  # context_pre_only: raw attention slice (:420-421)
+        if shape_img is not None:
+            out_img = out_img.transpose(-1, -2).reshape(shape_img[0], -1, shape_img[2], shape_img[3])
+        if shape_txt is not None and out_txt is not None:
+            out_txt = out_txt.transpose(-1, -2).reshape(shape_txt[0], -1, shape_txt[2], shape_txt[3])
+        return out_img, out_txt
 
     def forward_gated(self, hidden_states, encoder_hidden_states, resid_img, gate_img, resid_txt=None, gate_txt=None,
                       skip_txt: bool = False, **kwargs):

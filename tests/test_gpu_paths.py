@@ -318,3 +318,22 @@ def test_sd3_patches_skip_the_dropped_text_stream_bit_exact(hdit):
     enc, hid = stack.transformer_blocks[0](hidden_states=x_now[:, :starts[1]].contiguous(), encoder_hidden_states=e, temb=t,
                                            skip_text_output=True)
     assert enc is None and hid.shape == (B, starts[1], D)
+
+
+def test_sd3_attention_wrapper_takes_channel_major_4d_inputs(hdit):
+    """``[B, C, H, W]`` inputs to the wrapper are token sequences in channel-major layout
+    (attention_processor.py:672-683) and the outputs come back in that layout (:436-443): same numbers as the
+    ``[B, T, C]`` call, which is checked against the oracle elsewhere."""
+    from hetu_dit_amd import blocks, synthetic
+
+    B, D, H, gh, gw, th, tw = 2, 256, 4, 6, 10, 3, 7
+    blk, _ = make(blocks.JointTransformerBlock, 201, D, H, 64)
+    wrapper = blk.attn
+    x4 = synthetic.randn_bf16((B, D, gh, gw), 202).to(DEV)
+    e4 = synthetic.randn_bf16((B, D, th, tw), 203).to(DEV)
+    out4, enc4 = wrapper(x4, encoder_hidden_states=e4)
+    x3, e3 = x4.flatten(2).transpose(1, 2).contiguous(), e4.flatten(2).transpose(1, 2).contiguous()
+    out3, enc3 = wrapper(x3, encoder_hidden_states=e3)
+    torch.cuda.synchronize()
+    assert out4.shape == (B, D, gh, gw) and enc4.shape == (B, D, th, tw)
+    assert torch.equal(out4.flatten(2).transpose(1, 2), out3) and torch.equal(enc4.flatten(2).transpose(1, 2), enc3)
