@@ -9,8 +9,13 @@
 //     workspace laid out [batch, head, key (padded to 64), d] (every query
 //     tile would otherwise repeat the conversion); Q is quantised as its
 //     fragments are loaded;
-//   * the scores are de-scaled inside the exponent (the factor
-//     absmax_q * absmax_k / 448^2 is folded into the softmax scale);
+//   * the scores are de-scaled by the MFMA itself.  With d = 64 the Q scale is chosen (within a factor of two
+//     below the full-range one, which costs e4m3 nothing but headroom) so that softmax scale * log2(e) *
+//     de-quantisation factor of q and k is an exact power of two, and that power goes into the block-scale
+//     operand of the score MFMA; the running reference (and the +7 of the next item) is subtracted by letting
+//     the MFMA accumulate onto a vector holding it.  The accumulators then feed exp2 directly: no per-score
+//     multiply-add in a loop whose matrix and vector time add up.  (d = 128 has no registers for that vector and
+//     keeps the multiply-add.)
 //   * P is re-quantised per tile as exp2(s - m + 7): at most 2^8 = 256 < 448
 //     with the running maximum allowed to lag by one power of two, so small
 //     probabilities keep normal-range e4m3 precision;
@@ -74,15 +79,36 @@ __device__ __forceinline__ i32x2 quant8(const i32x4& raw, float s) {
   return r;
 }
 
+// K and V tiles (64 keys x HD bytes each) go straight from the pre-quantised workspace into LDS
+// (global_load_lds_dwordx4: no staging registers, no ds_write), which lands a wave's 64 x 16 bytes contiguously:
+// unpadded rows of HD bytes.  The spread over the 256-byte bank window comes from XOR swizzles of the 16-byte
+// chunk index, applied on the source side.  A ds_read_b128 pass covers 16 consecutive K rows, which must fall on
+// 16 distinct chunk slots: slot p of K row r holds chunk p ^ xk(r).  A transpose-read pass covers, per half wave,
+// key rows {0..3, 8..11} (or {4..7, 12..15}) x 32 bytes, which must fall on distinct 32-byte pieces: slot p of V
+// row r holds chunk p ^ xv(r), xv even (it moves whole 32-byte pieces).
 template <int HD>
 struct Lds8 {
-  static constexpr int K_ROW = HD + 16;
-  static constexpr int V_ROW = HD + 32;
+  static constexpr int K_ROW = HD;
+  static constexpr int V_ROW = HD;
   static constexpr int K_BYTES = BKV * K_ROW;
   static constexpr int V_BYTES = BKV * V_ROW;
   static constexpr int STAGE = K_BYTES + V_BYTES;
   static constexpr int TOTAL = 2 * STAGE;
+  __device__ static constexpr int xk(int r) { return HD == 64 ? ((r >> 2) & 3) : ((r >> 1) & 7); }
+  __device__ static constexpr int xv(int r) { return HD == 64 ? 2 * ((r >> 3) & 1) : 2 * (((r >> 1) & 1) | (((r >> 3) & 1) << 1)); }
 };
+
+// One wave-wide direct-to-LDS copy: lane l's 16 bytes land at LDS byte address lds_addr + 16*l.  Inline
+// assembly, so the compiler's wait-count bookkeeping does not see it; the tile loop waits for it explicitly.
+__device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr_uniform), "v"(voff), "s"(base_uniform)
+               : "m0", "memory");
+}
+__device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
+  return (unsigned)(uintptr_t)((const __attribute__((address_space(3))) unsigned char*)p);
+}
 
 template <int HD>
 __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const AttnParams P, int q_tiles) {
@@ -109,8 +135,20 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
   const float amq = fmaxf(P.absmax[bh], 1e-20f);
   const float amk = fmaxf(P.absmax[nbh + bh], 1e-20f);
   const float amv = fmaxf(P.absmax[2 * nbh + bh], 1e-20f);
-  const float qs = FP8_MAX / amq;
-  const float scale_log2 = P.scale * 1.4426950408889634f * (amq / FP8_MAX) * (amk / FP8_MAX);
+  constexpr bool FOLD = HD == 64;
+  // score = f * (q8 . k8), f = softmax scale * log2(e) * amk / (448 * qs).  FOLD: qs = full-range scale * f0 / 2^e
+  // with e = ceil(log2 f0), so that f = 2^e exactly and 2^e rides the MFMA's E8M0 block scale of the Q operand.
+  float qs = FP8_MAX / amq;
+  float scale_log2 = P.scale * 1.4426950408889634f * (amq / FP8_MAX) * (amk / FP8_MAX);
+  int q_block_scale = 0x7f7f7f7f;  // E8M0 127 = 2^0 in every byte
+  if constexpr (FOLD) {
+    int e = (int)ceilf(log2f(scale_log2));
+    e = max(-126, min(127, e));
+    const float pow2 = exp2f((float)e);
+    qs *= fminf(scale_log2 / pow2, 1.0f);
+    scale_log2 = pow2;
+    q_block_scale = 0x01010101 * (127 + e);
+  }
   const float o_descale = amv / FP8_MAX;
 
   // ---- Q fragments: lane holds q row qb*32 + l32, bytes d = 64*ks + 32*lh .. +31
@@ -129,27 +167,31 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
       }
   }
 
-  // K/V tiles come from the pre-quantised workspace: 64 rows x HD bytes each, 16 bytes per thread
-  constexpr int CPR8 = HD / 16;
-  constexpr int NCH8 = BKV * CPR8 / 256;
-  i32x4 kreg[NCH8], vreg[NCH8];
+  // K/V tiles come from the pre-quantised workspace, 64 rows x HD bytes each: request i of a wave covers rows
+  // RPR * (wave + 4 i) .. + RPR - 1, lane -> (row, slot lane % CPR8); the chunk fetched for a slot is the slot index
+  // XORed with the row's swizzle.  Rows past the last key are zero in the workspace.
+  constexpr int CPR8 = HD / 16;        // 16-byte chunks per row
+  constexpr int RPR = 64 / CPR8;       // rows per request
+  constexpr int NREQ = BKV / (RPR * NWAVE);
   const unsigned char* k8 = P.k8 + (size_t)bh * P.skv_pad * HD;
   const unsigned char* v8 = P.v8 + (size_t)bh * P.skv_pad * HD;
-  auto load_tile = [&](int t) {
+  unsigned koff[NREQ], voff[NREQ];
 #pragma unroll
-    for (int i = 0; i < NCH8; i++) {
-      const int c = tid + i * 256;
-      kreg[i] = *(const i32x4*)(k8 + (size_t)t * BKV * HD + c * 16);
-      vreg[i] = *(const i32x4*)(v8 + (size_t)t * BKV * HD + c * 16);
-    }
-  };
-  auto store_tile = [&](int stage) {
-    unsigned char* base = lds + stage * L::STAGE;
+  for (int i = 0; i < NREQ; i++) {
+    const int row = RPR * (wave + NWAVE * i) + lane / CPR8, slot = lane % CPR8;
+    koff[i] = (unsigned)(row * HD + ((slot ^ L::xk(row)) << 4));
+    voff[i] = (unsigned)(row * HD + ((slot ^ L::xv(row)) << 4));
+  }
+  const unsigned lds_base_addr = __builtin_amdgcn_readfirstlane(lds_address(lds));
+  const unsigned wave_dst = lds_base_addr + __builtin_amdgcn_readfirstlane(wave) * 1024;
+  auto dma_tile = [&](int t, int stage) {
+    const unsigned char* kb = k8 + (size_t)t * BKV * HD;
+    const unsigned char* vb = v8 + (size_t)t * BKV * HD;
+    const unsigned kdst = wave_dst + stage * L::STAGE;
 #pragma unroll
-    for (int i = 0; i < NCH8; i++) {
-      const int c = tid + i * 256, row = c / CPR8, cc = c % CPR8;
-      *(i32x4*)(base + row * L::K_ROW + cc * 16) = kreg[i];
-      *(i32x4*)(base + L::K_BYTES + row * L::V_ROW + cc * 16) = vreg[i];
+    for (int i = 0; i < NREQ; i++) {
+      lds_dma16(kb, koff[i], kdst + i * NWAVE * 1024);
+      lds_dma16(vb, voff[i], kdst + L::K_BYTES + i * NWAVE * 1024);
     }
   };
 
@@ -160,19 +202,32 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) oacc[i][j][v] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY};
+  // FOLD: m_run is the running reference in log2 units (0 until the first tile sets it); the score accumulators
+  // start from negm = P_SHIFT - m_run (one value in all 16 entries: a lane owns one query column per qb)
+  float m_run[2] = {FOLD ? 0.f : -INFINITY, FOLD ? 0.f : -INFINITY};
   float l_run[2] = {0.f, 0.f};
+  f32x16 negm[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) negm[qb][v] = P_SHIFT;
+  bool first = true;
 
   // byte-transpose read of V^T: in a 16-lane group lane x supplies the address of 8 bytes
   // (row = key of slot x>>1, column half x&1) and lane i receives byte i%8 of the rows of lanes 2j + i/8.
   // Slot jj of read r is key 16r + 8*(jj>>2) + 4*lh + (jj&3): the key order of a lane's accumulator bytes.
   const int jj = (lane & 15) >> 1;
-  const int vt_off = (8 * (jj >> 2) + 4 * lh + (jj & 3)) * L::V_ROW + 16 * ((lane >> 4) & 1) + 8 * (lane & 1);
-  const int k_off = l32 * L::K_ROW + lh * 32;
+  const int vt_row = 8 * (jj >> 2) + 4 * lh + (jj & 3);  // + 16 r: does not change the row's swizzle
+  const int vt_base = vt_row * L::V_ROW + 8 * (lane & 1);
+  const int vt_chunk = (lane >> 4) & 1;                  // + 2 db
+  const int vt_swz = L::xv(vt_row);
+  const int k_base = l32 * L::K_ROW;                       // + 32 kb rows: does not change the row's swizzle
+  const int k_swz = L::xk(l32);
   const int unit_scale = 0x7f7f7f7f;  // E8M0 exponent 127 = 2^0 for every block
 
-  auto tile_compute = [&](const unsigned char* sk, auto mask_tag, int valid) {
+  auto tile_compute = [&](const unsigned char* sk, auto mask_tag, int valid, auto last_tag) {
     constexpr bool MASK = decltype(mask_tag)::value;
+    constexpr bool LAST = decltype(last_tag)::value;
     const unsigned char* sv = sk + L::K_BYTES;
     f32x16 sacc[2][2];
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -180,13 +235,14 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
     for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
-        const unsigned char* ka = sk + k_off + kb * 32 * L::K_ROW + ks * 64;
-        i32x4 lo = *(const i32x4*)ka, hi = *(const i32x4*)(ka + 16);
+        const unsigned char* ka = sk + k_base + kb * 32 * L::K_ROW;
+        const int c0 = ks * 4 + lh * 2;  // this lane's 32 bytes are chunks c0, c0 + 1 of the row
+        i32x4 lo = *(const i32x4*)(ka + ((c0 ^ k_swz) << 4)), hi = *(const i32x4*)(ka + (((c0 + 1) ^ k_swz) << 4));
         i32x8 kf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
         for (int qb = 0; qb < 2; qb++)
-          sacc[kb][qb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[qb][ks], ks == 0 ? zero16 : sacc[kb][qb],
-                                                                         0, 0, 0, unit_scale, 0, unit_scale);
+          sacc[kb][qb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+              kf, qf[qb][ks], ks == 0 ? (FOLD ? negm[qb] : zero16) : sacc[kb][qb], 0, 0, 0, unit_scale, 0, q_block_scale);
       }
     }
     if (MASK) {
@@ -201,27 +257,63 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
           }
         }
     }
-    float mcand[2];
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-      float mx = fmaxf(sacc[0][qb][0], sacc[1][qb][0]);
-#pragma unroll
-      for (int v = 1; v < 16; v++) mx = fmaxf(mx, fmaxf(sacc[0][qb][v], sacc[1][qb][v]));
-      auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(mx), __float_as_int(mx), false, false);
-      mx = fmaxf(__int_as_float(sw[0]), __int_as_float(sw[1]));
-      mcand[qb] = fmaxf(m_run[qb], mx * scale_log2);
-    }
-    const bool grow = (mcand[0] - m_run[0] > RESCALE_THRESHOLD) || (mcand[1] - m_run[1] > RESCALE_THRESHOLD);
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+    if constexpr (FOLD) {
+      // the accumulators hold s - m + P_SHIFT; their column maxima, minus P_SHIFT, are relative to the reference
+      float mrel[2];
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
-        const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - mcand[qb]);
-        m_run[qb] = mcand[qb];
-        l_run[qb] *= alpha;
+        float mx = fmaxf(sacc[0][qb][0], sacc[1][qb][0]);
 #pragma unroll
-        for (int db = 0; db < DB; db++)
+        for (int v = 1; v < 16; v++) mx = fmaxf(mx, fmaxf(sacc[0][qb][v], sacc[1][qb][v]));
+        auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(mx), __float_as_int(mx), false, false);
+        mrel[qb] = fmaxf(__int_as_float(sw[0]), __int_as_float(sw[1])) - P_SHIFT;
+      }
+      const bool grow = first || mrel[0] > RESCALE_THRESHOLD || mrel[1] > RESCALE_THRESHOLD;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
-          for (int v = 0; v < 16; v++) oacc[db][qb][v] *= alpha;
+        for (int qb = 0; qb < 2; qb++) {
+          const float d = first ? mrel[qb] : fmaxf(mrel[qb], 0.f);
+          m_run[qb] += d;
+          if (!first) {
+            const float alpha = __builtin_amdgcn_exp2f(-d);
+            l_run[qb] *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+              for (int v = 0; v < 16; v++) oacc[db][qb][v] *= alpha;
+          }
+#pragma unroll
+          for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) sacc[kb][qb][v] -= d;
+#pragma unroll
+          for (int v = 0; v < 16; v++) negm[qb][v] = P_SHIFT - m_run[qb];
+        }
+        first = false;
+      }
+    } else {
+    float mcand[2];
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        float mx = fmaxf(sacc[0][qb][0], sacc[1][qb][0]);
+#pragma unroll
+        for (int v = 1; v < 16; v++) mx = fmaxf(mx, fmaxf(sacc[0][qb][v], sacc[1][qb][v]));
+        auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(mx), __float_as_int(mx), false, false);
+        mx = fmaxf(__int_as_float(sw[0]), __int_as_float(sw[1]));
+        mcand[qb] = fmaxf(m_run[qb], mx * scale_log2);
+      }
+      const bool grow = (mcand[0] - m_run[0] > RESCALE_THRESHOLD) || (mcand[1] - m_run[1] > RESCALE_THRESHOLD);
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+          const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - mcand[qb]);
+          m_run[qb] = mcand[qb];
+          l_run[qb] *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) oacc[db][qb][v] *= alpha;
+        }
       }
     }
     i32x8 pf[2];  // [qb]: 32 bytes, byte e = 16*kb + v
@@ -236,7 +328,7 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
           float p[4];
 #pragma unroll
           for (int e = 0; e < 4; e++)
-            p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][qb][w4 * 4 + e], scale_log2, -moff));
+            p[e] = __builtin_amdgcn_exp2f(FOLD ? sacc[kb][qb][w4 * 4 + e] : __builtin_fmaf(sacc[kb][qb][w4 * 4 + e], scale_log2, -moff));
           int w = 0;
           w = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], w, false);
           w = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], w, true);
@@ -250,7 +342,7 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
       i32x8 vf;
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const unsigned char* va = sv + vt_off + (16 * r) * L::V_ROW + db * 32;
+        const unsigned char* va = sv + vt_base + (16 * r) * L::V_ROW + (((2 * db + vt_chunk) ^ vt_swz) << 4);
         i32x2 t8 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i32x2 __attribute__((address_space(3)))*)(va));
         vf[2 * r] = t8[0];
         vf[2 * r + 1] = t8[1];
@@ -260,26 +352,37 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
         oacc[db][qb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf[qb], oacc[db][qb], 0, 0, 0, unit_scale, 0,
                                                                        unit_scale);
     }
+    if constexpr (LAST) {
+      // These PV MFMAs are 16-pass instructions and what follows the last tile reads their accumulators at once
+      // (the compiler shuffles them into other registers for the output code).  The no-ops it puts in front of
+      // that were seen to be too few for the last two registers of the last accumulator block -- wrong values in
+      // exactly those output columns when the masked tile ran last -- so the distance is made explicit here, once
+      // per workgroup.
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
   const int NT = (P.skv + BKV - 1) / BKV;
-  load_tile(0);
-  store_tile(0);
+  // Tile t+1 is fetched while tile t is worked on: its requests are issued behind the barrier that published
+  // tile t, into the stage tile t-1 vacated; every wave waits for its own requests before the next barrier.
+  dma_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
-  if (NT > 1) load_tile(1);
+  if (NT > 1) dma_tile(1, 1);
   for (int t = 0; t < NT - 1; t++) {
-    tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
-    store_tile((t + 1) & 1);
+    tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV, std::false_type{});
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile t+1 has landed
     __syncthreads();
-    if (t + 2 < NT) load_tile(t + 2);
+    if (t + 2 < NT) dma_tile(t + 2, t & 1);
   }
   {
     const int t = NT - 1;
     const int valid = P.skv - t * BKV;
-    if (valid < BKV) tile_compute(lds + (t & 1) * L::STAGE, std::true_type{}, valid);
-    else tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV);
+    if (valid < BKV) tile_compute(lds + (t & 1) * L::STAGE, std::true_type{}, valid, std::true_type{});
+    else tile_compute(lds + (t & 1) * L::STAGE, std::false_type{}, BKV, std::true_type{});
   }
-
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
     auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(l_run[qb]), __float_as_int(l_run[qb]), false, false);
@@ -355,6 +458,49 @@ __global__ void __launch_bounds__(256) absmax_kernel(const AttnParams P, float* 
   if ((threadIdx.x & 63) == 0 && r0 < r1) atomicMax((int*)absmax + blockIdx.y, __float_as_int(m));
 }
 
+// The same maxima when the heads of a row lie side by side in memory (stride_h == HD: column ranges of a packed
+// q|k|v tensor, the usual case): a workgroup streams whole rows -- every request a run of full cache lines --
+// instead of one 128- or 256-byte piece per row and head.  A 16-byte chunk belongs to one head; the lanes of a
+// head's chunks in a row are neighbours, so they reduce among themselves before one lane merges into the
+// workgroup's per-head maxima in LDS, and those go out with one atomic per head.
+template <int HD>
+__global__ void __launch_bounds__(256) absmax_rows_kernel(const AttnParams P, float* absmax, int rows_per_wg) {
+  constexpr int CPH = HD / 8;  // chunks per head
+  __shared__ int head_max[256];
+  const int which = blockIdx.y / P.batch, b = blockIdx.y % P.batch;
+  const Seg2& s = which == 0 ? P.q : (which == 1 ? P.k : P.v);
+  const int total = s.len0 + s.len1;
+  const int cpr = P.heads * CPH;  // chunks per row
+  for (int i = threadIdx.x; i < P.heads; i += 256) head_max[i] = 0;
+  __syncthreads();
+  const int r0 = blockIdx.x * rows_per_wg, r1 = min(r0 + rows_per_wg, total);
+  const int64_t chunks = (int64_t)(r1 - r0) * cpr;
+  for (int64_t c0 = 0; c0 < chunks; c0 += 256) {
+    const int64_t c = c0 + threadIdx.x;
+    float m = 0.f;
+    int head = 0;
+    if (c < chunks) {
+      const int r = r0 + (int)(c / cpr), cc = (int)(c % cpr);
+      head = cc / CPH;
+      float f[8];
+      hdit::unpack8(*(const i32x4*)(row_ptr(s, b, 0, r) + cc * 8), f);
+#pragma unroll
+      for (int e = 0; e < 8; e++) m = fmaxf(m, fabsf(f[e]));
+    }
+    // cpr and 256 are multiples of CPH, so the CPH lanes of one (row, head) are an aligned group of the wave
+#pragma unroll
+    for (int off = 1; off < CPH; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if ((threadIdx.x & (CPH - 1)) == 0 && c < chunks) atomicMax(&head_max[head], __float_as_int(m));
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < P.heads; i += 256)
+    if (r0 < r1) atomicMax((int*)absmax + (which * P.batch + b) * P.heads + i, head_max[i]);
+}
+
+bool heads_side_by_side(const Seg2& s, int hd) {
+  return (s.len0 == 0 || s.sh0 == hd) && (s.len1 == 0 || s.sh1 == hd);
+}
+
 Seg2 make_seg(const hdit_seq_segment* s) {
   Seg2 r;
   r.p0 = (const __bf16*)s[0].ptr;
@@ -410,6 +556,16 @@ extern "C" __attribute__((visibility("default"))) int hdit_attn_absmax(const hdi
   hipLaunchKernelGGL(absmax_zero_kernel, dim3((n + 63) / 64), dim3(64), 0, s, absmax, n);
   const int longest = P.sq > P.skv ? P.sq : P.skv;
   if (longest == 0) return hdit_host::check_launch("hdit_attn_absmax");
+  if (a->heads <= 256 && heads_side_by_side(P.q, a->head_dim) && heads_side_by_side(P.k, a->head_dim) &&
+      heads_side_by_side(P.v, a->head_dim)) {
+    const int rows = 32;
+    dim3 grid((longest + rows - 1) / rows, 3 * a->batch);
+    if (a->head_dim == 64)
+      hipLaunchKernelGGL(absmax_rows_kernel<64>, grid, dim3(256), 0, s, P, absmax, rows);
+    else
+      hipLaunchKernelGGL(absmax_rows_kernel<128>, grid, dim3(256), 0, s, P, absmax, rows);
+    return hdit_host::check_launch("hdit_attn_absmax");
+  }
   const int rows_per_wg = 256;
   dim3 grid((longest + rows_per_wg - 1) / rows_per_wg, n);
   if (a->head_dim == 64)
