@@ -358,9 +358,14 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
       // that were seen to be too few for the last two registers of the last accumulator block -- wrong values in
       // exactly those output columns when the masked tile ran last -- so the distance is made explicit here, once
       // per workgroup.
-      __builtin_amdgcn_sched_barrier(0);
-      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-      __builtin_amdgcn_sched_barrier(0);
+      // (The accumulators are operands of the statement, so it sits behind the MFMAs that write them and in front
+      // of every instruction that reads them.)
+      if constexpr (DB == 2)
+        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(oacc[0][0]), "+v"(oacc[0][1]), "+v"(oacc[1][0]), "+v"(oacc[1][1]));
+      else
+        asm volatile("s_nop 15\n\ts_nop 15"
+                     : "+v"(oacc[0][0]), "+v"(oacc[0][1]), "+v"(oacc[1][0]), "+v"(oacc[1][1]), "+v"(oacc[2][0]),
+                       "+v"(oacc[2][1]), "+v"(oacc[3][0]), "+v"(oacc[3][1]));
     }
   };
 
