@@ -222,6 +222,35 @@ def cpu_baseline(runs=3):
     }
 
 
+def probe_coissue():
+    """Times an MFMA wave and a softmax-VALU wave alone on a SIMD, two of a kind together, one of each together, and
+    both kinds interleaved in one wave; at 16 workgroups (no power limit) and at one per CU.  If the two units
+    overlapped, 'mfma | valu' would take the longer of the two; it takes their sum."""
+    import torch
+
+    import hetu_dit_amd  # noqa: F401
+    from hetu_dit_amd import ops
+
+    torch.cuda.set_device(0)
+    iters = 2000
+    I, M, V, X = ops.PROBE_IDLE, ops.PROBE_MFMA, ops.PROBE_VALU, ops.PROBE_INTERLEAVED
+    cases = [("mfma | idle", M, I), ("valu | idle", V, I), ("mfma | mfma", M, M), ("valu | valu", V, V), ("mfma | valu", M, V),
+             ("valu | mfma", V, M), ("interleaved | idle", X, I)]
+    result = {}
+    for wgs in (16, 256):
+        print(f"# {wgs} workgroups of 8 waves, {iters} iterations of 32 MFMAs / one 64-score softmax block; waves w and w+4 share a SIMD")
+        print(f"# {'waves 0-3 | waves 4-7':22s} {'kcycles A':>10s} {'us A':>9s} {'kcycles B':>10s} {'us B':>9s} {'GHz':>6s}")
+        for name, ra, rb in cases:
+            ops.probe_coissue(ra, rb, 50, wgs)
+            ca, ua, cb, ub = ops.probe_coissue(ra, rb, iters, wgs)
+            ghz = ca / ua / 1e3 if ua > 0 else 0.0
+            print(f"  {name:22s} {ca / 1e3:10.0f} {ua:9.1f} {cb / 1e3:10.0f} {ub:9.1f} {ghz:6.2f}")
+            result[f"{name} @{wgs}"] = {"kcycles_a": round(ca / 1e3), "kcycles_b": round(cb / 1e3), "us_a": round(ua, 1), "us_b": round(ub, 1)}
+    m, v, mv = result["mfma | idle @16"]["kcycles_a"], result["valu | idle @16"]["kcycles_a"], result["mfma | valu @16"]["kcycles_b"]
+    print(json.dumps({"probe": "coissue", "mfma_alone_kcycles": m, "valu_alone_kcycles": v, "valu_next_to_mfma_kcycles": mv,
+                      "overlap": round(1.0 - (mv - max(m, v)) / min(m, v), 3), "cases": result}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -231,7 +260,12 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--workload", choices=WORKLOADS, default="sd3_1024",
                     help="sd3_1024 (BASELINE.json configs[1]) is the headline metric; the others are for profiling")
+    ap.add_argument("--probe", choices=["coissue"], default=None,
+                    help="instead of a workload, run a hardware probe and print its table: coissue = do the matrix "
+                         "pipe and the vector ALU of a SIMD work side by side (hdit_probe_coissue)")
     args = ap.parse_args()
+    if args.probe == "coissue":
+        return probe_coissue()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only: run with --gpus 1 "
               "(the path is built and measured on a single GPU; nothing here launches collectives)", file=sys.stderr)

@@ -199,6 +199,7 @@ SIGNATURES = {
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_float, C.c_float, C.c_void_p],
     ),
     "hdit_clock_sample": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
+    "hdit_probe_coissue": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "hdit_gemm_force_config": (None, [C.c_int]),
     "hdit_rope_table": (
         C.c_int,

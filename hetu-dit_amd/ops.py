@@ -732,6 +732,20 @@ def rope_table(positions: torch.Tensor, axes_dim, theta: float = 10000.0) -> Tup
     return cos, sin
 
 
+PROBE_IDLE, PROBE_MFMA, PROBE_VALU, PROBE_INTERLEAVED = 0, 1, 2, 3
+
+
+def probe_coissue(role_a: int, role_b: int, iters: int = 2000, workgroups: int = 16):
+    """``hdit_probe_coissue``: waves 0-3 of every workgroup run ``role_a``, waves 4-7 (same SIMDs) ``role_b``.
+    Returns ``(cycles_a, us_a, cycles_b, us_b)``: mean shader cycles and microseconds per wave of each group."""
+    out = torch.zeros(workgroups * 16 + 1, dtype=torch.int64, device="cuda")
+    check(_lib.lib().hdit_probe_coissue(role_a, role_b, iters, workgroups, out.data_ptr(), _stream()), "hdit_probe_coissue")
+    torch.cuda.synchronize()
+    t = out[: workgroups * 16].view(workgroups, 8, 2).double().cpu()
+    a, b = t[:, :4].mean(dim=(0, 1)), t[:, 4:].mean(dim=(0, 1))
+    return a[0].item(), a[1].item() / 100.0, b[0].item(), b[1].item() / 100.0
+
+
 def clock_sample(slots: int = 1024) -> torch.Tensor:
     """int64 [slots, 4] on the device, filled on the current stream with (shader-clock counter, 100 MHz counter,
     XCD id, hardware id) of `slots` one-wave workgroups (enough of them to land on every CU)."""

@@ -40,6 +40,22 @@ const char* hdit_last_error(void);
  * the work being timed give the average shader clock the work ran at,
  * (d out[0]) / (d out[1]) x 100 MHz. */
 int hdit_clock_sample(void* out, int slots, void* stream);
+/* Second measurement aid, no counterpart in the reference: do the matrix pipe
+ * and the vector ALU of a SIMD work side by side?  `workgroups` (<= 1024)
+ * workgroups of 8 waves, one per CU; waves w and w + 4 share a SIMD.  Waves 0-3
+ * run role_a and waves 4-7 role_b for `iters` iterations: nothing, 32
+ * independent v_mfma_f32_32x32x16_bf16 per iteration (the matrix work of one
+ * 64 x 64 x 64 attention tile), that tile's softmax VALU work (64 v_exp_f32, 32
+ * packs, 32 pair sums, 32 v_max3, 64 subtractions), or both interleaved 1 : 7
+ * in one instruction stream.  out (device, 8-byte aligned, workgroups * 16 + 1
+ * 64-bit values): per wave the shader cycles and the 100 MHz ticks it took,
+ * out[(16 g + 2 w)], out[16 g + 2 w + 1].  bench.py --probe coissue prints the
+ * table. */
+#define HDIT_PROBE_IDLE 0
+#define HDIT_PROBE_MFMA 1
+#define HDIT_PROBE_VALU 2
+#define HDIT_PROBE_INTERLEAVED 3
+int hdit_probe_coissue(int role_a, int role_b, int iters, int workgroups, void* out, void* stream);
 
 /* ------------------------------------------------------------------------
  * Grouped bf16 GEMM with fused epilogue:  C = epilogue(A . B^T + bias)

@@ -515,3 +515,15 @@ def test_layernorm_modulate_fp32_rows(hdit, D, affine):
     ops.layernorm_modulate_many([(wide[:, :, D:], sh.to(DEV), sc.to(DEV), joint[:, 3:])], **args)
     torch.cuda.synchronize()
     assert torch.equal(joint[:, 3:], got) and not joint[:, :3].any()
+
+
+def test_probe_coissue_runs_and_counts_cycles(hdit):
+    """The measurement aid ``hdit_probe_coissue``: an MFMA wave alone issues one 32x32x16 MFMA per 32 cycles (the
+    pipe's rate: 8 passes), whatever the clock; an idle partner reports (almost) nothing."""
+    iters = 200
+    ca, ua, cb, ub = hdit.ops.probe_coissue(hdit.ops.PROBE_MFMA, hdit.ops.PROBE_IDLE, iters, 8)
+    per_mfma = ca / (iters * 32)
+    assert 31.5 <= per_mfma <= 40.0, per_mfma
+    assert cb < 0.05 * ca and ua > 0
+    with pytest.raises(Exception):
+        hdit.ops.probe_coissue(7, 0, iters, 8)
