@@ -39,9 +39,13 @@ struct Seg2 {
 };
 
 __device__ __forceinline__ const __bf16* row_ptr(const Seg2& s, int b, int h, int r) {
-  // r must be < len0 + len1
-  if (r < s.len0) return s.p0 + b * s.sb0 + (int64_t)r * s.ss0 + h * s.sh0;
-  return s.p1 + b * s.sb1 + (int64_t)(r - s.len0) * s.ss1 + h * s.sh1;
+  // r must be < len0 + len1.  Every field is read and the values are selected: with a branch the compiler may
+  // merge the two sides into one load through a selected address, which forces the kernel's parameter block
+  // out of the scalar registers into private memory.
+  const bool a = r < s.len0;
+  const __bf16* p = a ? s.p0 : s.p1;
+  const int64_t sb = a ? s.sb0 : s.sb1, ss = a ? s.ss0 : s.ss1, sh = a ? s.sh0 : s.sh1;
+  return p + b * sb + (int64_t)(a ? r : r - s.len0) * ss + h * sh;
 }
 
 struct AttnParams {
