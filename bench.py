@@ -128,7 +128,13 @@ def make_workload(name, dev):
             gemm, attn = algorithmic_flops(cfg)
             desc = ("configs[1]: SD3-shape denoise step, 24 joint blocks, B2 (CFG pair), 4096 image + 333 text "
                     "tokens, D1536, 24x64 heads, last block context_pre_only")
-            return (lambda: stack(x, e, t)), desc, gemm, attn, cfg["layers"], "attn_fwd_kernel<64>"
+            def step():
+                return stack(x, e, t)
+
+            # launched eagerly the stack runs the two batch elements as independent chains on two streams
+            step.multi_stream = "eager, the two batch elements as independent block chains on two streams"
+            step.set_single_stream = lambda on: setattr(stack, "batch_streams", 1 if on else 2)
+            return step, desc, gemm, attn, cfg["layers"], "attn_fwd_kernel<64>"
         # PipeFusion shard: a full-sequence pass fills the K/V buffers ("previous step"), then one step is
         # four patch passes of 1024 image tokens each against the stale full-length buffers
         P = cfg["patches"]
@@ -139,12 +145,19 @@ def make_workload(name, dev):
         rs.set_patched_mode(True)
         xs = [rnd(B, Ni // P, D) for _ in range(P)]
 
+        single = [False]
+
         def step():
+            if not single[0]:
+                return stack.forward_patches(xs, e, t, num_streams=2)[-1]
             out = None
             for p in range(P):
                 out = stack(xs[p], e, t)
                 rs.next_patch()
             return out
+
+        step.multi_stream = "eager, patch p one block behind patch p-1 on two streams"
+        step.set_single_stream = lambda on: single.__setitem__(0, bool(on))
 
         L = cfg["layers"]
         Np = Ni // P
@@ -258,6 +271,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--single-stream", action="store_true",
+                    help="sd3_1024 / sd3_pipefusion: time the pass on one stream (a HIP-graph replay unless --no-graph) "
+                         "instead of the eager form that runs independent chains (batch elements, neighbouring "
+                         "patches) on two streams")
     ap.add_argument("--workload", choices=WORKLOADS, default="sd3_1024",
                     help="sd3_1024 (BASELINE.json configs[1]) is the headline metric; the others are for profiling")
     ap.add_argument("--probe", choices=["coissue"], default=None,
@@ -283,6 +300,8 @@ def main():
     step, workload_desc, gemm_fl, attn_fl, n_blocks, attn_kernel = make_workload(args.workload, dev)
     headline = args.workload == "sd3_1024"
 
+    if hasattr(step, "set_single_stream"):
+        step.set_single_stream(args.single_stream)
     for _ in range(max(args.warmup, 1)):
         out = step()
     torch.cuda.synchronize()
@@ -295,7 +314,26 @@ def main():
         return [t for entry in get_cache_manager().cache.values() for t in entry.tensors if t is not None]
 
     use_graph = not args.no_graph
-    if use_graph:
+    launch = None
+    multi_stream = getattr(step, "multi_stream", None)
+    if multi_stream is not None and not args.single_stream:
+        # launched eagerly (a multi-stream pass is not recorded into a graph); from the same buffer state it must
+        # reproduce the single-stream pass bit for bit
+        saved = [t.clone() for t in kv_buffers()]
+        step.set_single_stream(True)
+        ref = step().clone()
+        for t, s0 in zip(kv_buffers(), saved):
+            t.copy_(s0)
+        step.set_single_stream(False)
+        got = step()
+        torch.cuda.synchronize()
+        if not torch.equal(got, ref):
+            raise SystemExit("the multi-stream pass does not reproduce the single-stream pass")
+        del saved, got, ref
+        use_graph = False
+        run = step
+        launch = multi_stream
+    elif use_graph:
         saved = [t.clone() for t in kv_buffers()]
         ref = step().clone()
         for t, s0 in zip(kv_buffers(), saved):
@@ -337,6 +375,8 @@ def main():
     del calib_src, calib_dst
 
     # instrumented eager pass: HIP events around every launch on the launch stream
+    if hasattr(step, "set_single_stream"):
+        step.set_single_stream(True)  # one launch at a time, so that a launch's events time that launch alone
     timer = ops.KernelTimer()
     ops.set_timer(timer)
     for _ in range(3):
@@ -386,7 +426,7 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic (seeded N(0,1) activations, N(0,0.02) random-init weights, resident in HBM)",
-        "config": {"workload": workload_desc, "launch": "hip-graph replay" if use_graph else "eager"},
+        "config": {"workload": workload_desc, "launch": launch or ("hip-graph replay" if use_graph else "eager")},
         "step_tflops": round((gemm_fl + attn_fl) / ms_step / 1e9, 1),
         "shader_clock_ghz": round(shader_clock_ghz, 3) if shader_clock_ghz else None,
         "shader_clock_note": "average over the timed passes, from the shader-clock and 100 MHz counters sampled on the "

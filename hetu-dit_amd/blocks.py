@@ -74,6 +74,7 @@ class StackModulation:
         kinds = (AdaLayerNormZero, AdaLayerNormZeroSingle, AdaLayerNormContinuous, CogVideoXLayerNormZero)
         self.norms = [m for b in blocks for m in b.modules() if isinstance(m, kinds)]
         self.packed = _PackedProjection([n.linear for n in self.norms])
+        self._gather = {}  # (batch, device) -> element indices that regroup [B, all rows] by module
 
     def precompute(self, temb: torch.Tensor):
         w, b = self.packed.get()
@@ -82,6 +83,26 @@ class StackModulation:
         for norm, rows in zip(self.norms, self.packed.splits):
             norm._stack_emb = (temb, temb._version, emb[:, off : off + rows])
             off += rows
+        return emb
+
+    def precompute_by_module(self, temb: torch.Tensor):
+        """``precompute`` plus the same numbers regrouped so that every module's [batch, rows] block is
+        contiguous (what the whole-block entry points take): returns ``(flat f32 tensor, {module: element
+        offset of its block})``; batch element b of a module starts ``b * rows`` elements into its block."""
+        emb = self.precompute(temb)
+        B, total = emb.shape
+        key = (B, emb.device)
+        cached = self._gather.get(key)
+        if cached is None:
+            parts, offsets, off = [], {}, 0
+            cols = torch.arange(total, device=emb.device)
+            for norm, rows in zip(self.norms, self.packed.splits):
+                offsets[norm] = B * off
+                parts.append((torch.arange(B, device=emb.device)[:, None] * total + cols[off : off + rows][None, :]).reshape(-1))
+                off += rows
+            cached = self._gather[key] = (torch.cat(parts), offsets)
+        index, offsets = cached
+        return emb.reshape(-1).index_select(0, index), offsets
 
 
 def _stream_out(resid: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:

@@ -304,6 +304,90 @@ def block_sd3(block, hidden_states: torch.Tensor, encoder_hidden_states: torch.T
     return encoder_out, hidden_out
 
 
+def timer_installed() -> bool:
+    """True while ``set_timer`` has a per-launch timer in place (the whole-block calls launch from C and are
+    not seen by it, so callers that want per-kernel times take the per-kernel path)."""
+    return _TIMER is not None
+
+
+class Sd3BlockCall:
+    """A reusable ``hdit_block_sd3`` call for one ``JointTransformerBlock``.
+
+    The weight pointers and the block's geometry are written into the argument struct once (``refresh``
+    re-reads them, e.g. after a weight hot-swap re-assigned a ``.data``); a call only sets the stream tensors,
+    the modulation and K/V buffer pointers and the flags, which keeps the host cost of a block at one foreign
+    call -- what a block stack launched eagerly on several streams needs."""
+
+    def __init__(self, block):
+        self.block = block
+        self.args = _lib.Sd3BlockArgs()
+        self._ws_bytes = {}
+        self.refresh()
+
+    def refresh(self):
+        block, a = self.block, self.args
+        fill = _ArgFiller()
+        _fill_sd3_weights(a.w, block, fill)
+        self._weights = fill.keep
+        a.dim = block.norm1.linear.weight.shape[1]
+        a.heads = block.attn.heads_per_device
+        a.ff_dim = block.ff.module.net[0].proj.weight.shape[0]
+        a.temb_dim = block.norm1.linear.weight.shape[1]
+        a.context_pre_only = int(bool(block.context_pre_only))
+
+    def __call__(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
+                 out_dtype=bf16, skip_text_output: bool = False, kv_buffer: Optional[torch.Tensor] = None,
+                 kv_row0: int = 0, modulation_img: Optional[int] = None, modulation_txt: Optional[int] = None,
+                 hidden_out: Optional[torch.Tensor] = None):
+        """Same contract as ``block_sd3``.  ``modulation_img`` / ``modulation_txt``: device addresses of the f32
+        [batch, 6 dim] (text stream of a ``context_pre_only`` block: [batch, 2 dim]) adaLN projections of this
+        block for this ``temb`` (the caller keeps their tensor alive), or None to have the call compute them.
+        ``hidden_out``: a contiguous [batch, n_img, dim] tensor of ``out_dtype`` to write the image stream to."""
+        a = self.args
+        B, Ni, D = hidden_states.shape
+        Nt = encoder_hidden_states.shape[1]
+        if D != a.dim or encoder_hidden_states.shape[2] != D or encoder_hidden_states.shape[0] != B:
+            raise ValueError("stream shapes do not match the block")
+        a.hidden_f32 = _stream_tensor(hidden_states, "hidden_states")
+        a.encoder_f32 = _stream_tensor(encoder_hidden_states, "encoder_hidden_states")
+        _need(temb, bf16, "temb")
+        if temb.shape != (B, a.temb_dim) or not temb.is_contiguous():
+            raise ValueError("temb must be a contiguous [batch, dim] tensor")
+        dev = hidden_states.device
+        text_out = not a.context_pre_only and not skip_text_output
+        if hidden_out is None:
+            hidden_out = torch.empty(B, Ni, D, dtype=out_dtype, device=dev)
+        elif hidden_out.shape != (B, Ni, D) or hidden_out.dtype != out_dtype or not hidden_out.is_contiguous():
+            raise ValueError("hidden_out must be a contiguous [batch, n_img, dim] tensor of out_dtype")
+        encoder_out = torch.empty(B, Nt, D, dtype=out_dtype, device=dev) if text_out else None
+        a.hidden, a.encoder, a.temb = hidden_states.data_ptr(), encoder_hidden_states.data_ptr(), temb.data_ptr()
+        a.hidden_out, a.encoder_out = hidden_out.data_ptr(), (encoder_out.data_ptr() if text_out else None)
+        a.modulation_img, a.modulation_txt = modulation_img, modulation_txt
+        a.batch, a.n_img, a.n_txt = B, Ni, Nt
+        a.out_f32, a.skip_text_output = int(out_dtype == torch.float32), int(skip_text_output)
+        if kv_buffer is not None:
+            if kv_buffer.dtype != bf16 or kv_buffer.dim() != 3 or tuple(kv_buffer.shape[::2]) != (B, 2 * D) \
+                    or not kv_buffer.is_contiguous():
+                raise ValueError("kv_buffer must be a contiguous bf16 [batch, rows, 2 * dim] tensor")
+            a.kv_buffer, a.kv_rows, a.kv_row0 = kv_buffer.data_ptr(), kv_buffer.shape[1], kv_row0
+        else:
+            a.kv_buffer, a.kv_rows, a.kv_row0 = None, 0, 0
+        lib = _lib.lib()
+        key = (B, Ni, Nt, bool(skip_text_output), kv_buffer is not None)
+        nbytes = self._ws_bytes.get(key)
+        if nbytes is None:
+            nbytes = lib.hdit_block_sd3_workspace_bytes(C.byref(a))
+            if nbytes < 0:
+                raise _lib.HditError("hdit_block_sd3_workspace_bytes refused the arguments")
+            self._ws_bytes[key] = nbytes
+        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)
+        a.workspace, a.workspace_bytes = (ws.data_ptr() + 255) // 256 * 256, nbytes
+        check(lib.hdit_block_sd3(C.byref(a), _stream()), "hdit_block_sd3")
+        # stream-ordered reuse: these may be freed by the caller as soon as the launches are queued
+        del ws
+        return encoder_out, hidden_out
+
+
 class _ArgFiller:
     """Pointer bookkeeping for the whole-block argument structs: keeps every tensor alive whose address went in."""
 

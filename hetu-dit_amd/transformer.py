@@ -14,12 +14,46 @@ from typing import List, Optional, Tuple
 import torch
 from torch import nn
 
+from . import ops
 from .blocks import (CogVideoXBlock, FluxSingleTransformerBlock, FluxTransformerBlock, JointTransformerBlock,
                      StackModulation, use_fp32_residual_stream)
+from .cache_manager import get_cache_manager
 from .runtime_state import get_runtime_state
 
 
+# Side streams are shared by every stack of the process and kept few: a process has GPU_MAX_HW_QUEUES (4 by
+# default) hardware queues, streams beyond that share one, and two chains on one hardware queue run one after
+# the other however many streams they were issued on.
+_SIDE_STREAMS = {}  # device -> list of streams
+MAX_SIDE_STREAMS = 3
+
+
+def side_streams(device: torch.device, count: int) -> List["torch.cuda.Stream"]:
+    device = torch.device(device)
+    if device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    have = _SIDE_STREAMS.setdefault(device, [])
+    while len(have) < min(count, MAX_SIDE_STREAMS):
+        have.append(torch.cuda.Stream(device=device))  # default priority, like the caller's stream
+    return have[: min(count, MAX_SIDE_STREAMS)]
+
+
 class SD3TransformerBlocks(nn.Module):
+    """The 24 joint blocks of the SD3 transformer with the reference's block loop.
+
+    ``use_block_entry_points``: run every block through ``hdit_block_sd3`` (one foreign call per block, the
+    same launches on the same operands as the Python block: results are bit for bit the same) instead of one
+    foreign call per kernel.  An eager pass is then bound by the GPU and not by the interpreter, which is what
+    lets independent work run side by side on several streams:
+
+    * ``batch_streams``: a full-sequence pass of B >= 2 batch elements (the CFG pair) runs the elements as
+      independent chains on that many side streams, blocks issued alternately -- one chain's launches fill the
+      CUs another's partial last round of tiles leaves idle (SD3 step at B2: 21.1 -> 19.x ms);
+    * ``forward_patches``: the patches of a PipeFusion step, one block apart.
+
+    Neither is recorded into a HIP graph: under capture, and whenever a per-launch timer is installed or a
+    block uses fp8 attention, the pass runs on the caller's stream alone."""
+
     def __init__(self, num_layers: int = 24, dim: int = 1536, num_attention_heads: int = 24,
                  attention_head_dim: int = 64):
         super().__init__()
@@ -33,28 +67,209 @@ class SD3TransformerBlocks(nn.Module):
         self.encoder_hidden_states_cache: List[Optional[torch.Tensor]] = [None] * num_layers
         self.modulation = StackModulation(self.transformer_blocks)
         use_fp32_residual_stream(self.transformer_blocks)
+        self.use_block_entry_points = True
+        self.batch_streams = 2
+        self._block_calls: Optional[List[ops.Sd3BlockCall]] = None
+        self._patch_events = {}  # (patch, block) -> "block done" event of forward_patches
 
+    # -- launching one block ------------------------------------------------------------------------------
+    def _entry_point_calls(self) -> Optional[List["ops.Sd3BlockCall"]]:
+        """The prefilled whole-block calls, weight pointers re-read, or None where the per-kernel path has to
+        run: switched off, a per-launch timer installed, or fp8 attention asked for (not in the entry point)."""
+        if not self.use_block_entry_points or ops.timer_installed():
+            return None
+        if any(getattr(b.attn, "fp8_attention", False) for b in self.transformer_blocks):
+            return None
+        if self._block_calls is None or len(self._block_calls) != len(self.transformer_blocks):
+            self._block_calls = [ops.Sd3BlockCall(b) for b in self.transformer_blocks]
+        else:
+            for call in self._block_calls:
+                call.refresh()
+        return self._block_calls
+
+    def _run_block(self, i: int, calls, mods, hidden, encoder, temb, skip_text_output: bool = False,
+                   kv_buffer=None, kv_row0: int = 0, batch0: int = 0, hidden_out=None):
+        """Block i on the current stream: ``(encoder_out_or_None, hidden_out)``.  ``batch0``: index of the
+        first batch element of ``hidden`` within the ``temb`` the modulation ``mods`` was computed for."""
+        block = self.transformer_blocks[i]
+        if calls is None:
+            return block(hidden_states=hidden, encoder_hidden_states=encoder, temb=temb,
+                         skip_text_output=skip_text_output)
+        flat, offsets = mods
+        dim = hidden.shape[2]
+        rows_txt = (2 if block.context_pre_only else 6) * dim
+        base = flat.data_ptr()
+        return calls[i](
+            hidden, encoder, temb, out_dtype=block.stream_dtype, skip_text_output=skip_text_output,
+            kv_buffer=kv_buffer, kv_row0=kv_row0,
+            modulation_img=base + 4 * (offsets[block.norm1] + batch0 * 6 * dim),
+            modulation_txt=base + 4 * (offsets[block.norm1_context] + batch0 * rows_txt),
+            hidden_out=hidden_out,
+        )
+
+    def _kv_buffer(self, i: int, hidden: torch.Tensor):
+        """``(buffer, first row)``: the K|V buffer block i's image stream writes into, from the cache manager --
+        a fresh full-length buffer with patch mode off, the persistent one and the current patch's rows in
+        patch mode."""
+        attn = self.transformer_blocks[i].attn
+        buf, start, _ = get_cache_manager().kv_buffer(attn, hidden.shape[0], hidden.shape[1], hidden.shape[2], hidden.device)
+        return buf, start
+
+    def _persistent_buffers_contiguous(self) -> bool:
+        """A full pass of the per-kernel path keeps q|k|v in one tensor and registers its k|v columns, a strided
+        view, as the layer's buffer; the whole-block entry point wants a contiguous [B, rows, 2 dim] buffer.  A
+        patch pass therefore stays on the path that filled the buffers."""
+        cm = get_cache_manager()
+        for block in self.transformer_blocks:
+            buf = cm._entry(block.attn, "attn").tensors[0]
+            if buf is None or not buf.is_contiguous():
+                return False
+        return True
+
+    # -- the reference's block loop -----------------------------------------------------------------------
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb):
         rs = get_runtime_state()
-        self.modulation.precompute(temb)
-        for i, block in enumerate(self.transformer_blocks):
+        calls = self._entry_point_calls()
+        if calls is not None and rs.patch_mode and not self._persistent_buffers_contiguous():
+            calls = None
+        if calls is None:
+            self.modulation.precompute(temb)
+            mods = None
+        else:
+            hidden_states, encoder_hidden_states = hidden_states.contiguous(), encoder_hidden_states.contiguous()
+            temb = temb.contiguous()
+            mods = self.modulation.precompute_by_module(temb)
+            lanes = min(self.batch_streams, hidden_states.shape[0])
+            if not rs.patch_mode and lanes > 1 and not torch.cuda.is_current_stream_capturing():
+                return self._forward_batch_lanes(calls, mods, hidden_states, encoder_hidden_states, temb, lanes)
+        for i in range(len(self.transformer_blocks)):
+            kv = self._kv_buffer(i, hidden_states) if calls is not None else (None, 0)
             if rs.patch_mode and rs.pipeline_patch_idx == 0:
                 self.encoder_hidden_states_cache[i] = encoder_hidden_states
-                encoder_hidden_states, hidden_states = block(
-                    hidden_states=hidden_states, encoder_hidden_states=encoder_hidden_states, temb=temb
-                )
+                encoder_hidden_states, hidden_states = self._run_block(
+                    i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1])
             elif rs.patch_mode:
                 # the text output of these calls is dropped: the block does not compute it
-                _, hidden_states = block(
-                    hidden_states=hidden_states, encoder_hidden_states=self.encoder_hidden_states_cache[i], temb=temb,
-                    skip_text_output=True,
-                )
+                _, hidden_states = self._run_block(
+                    i, calls, mods, hidden_states, self.encoder_hidden_states_cache[i], temb, skip_text_output=True,
+                    kv_buffer=kv[0], kv_row0=kv[1])
             else:
-                encoder_hidden_states, hidden_states = block(
-                    hidden_states=hidden_states, encoder_hidden_states=encoder_hidden_states, temb=temb
-                )
+                encoder_hidden_states, hidden_states = self._run_block(
+                    i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1])
         return hidden_states
+
+    def _forward_batch_lanes(self, calls, mods, hidden_states, encoder_hidden_states, temb, lanes: int):
+        """Full-sequence pass with the batch elements as ``lanes`` independent chains on side streams."""
+        B = hidden_states.shape[0]
+        L = len(self.transformer_blocks)
+        main = torch.cuda.current_stream()
+        streams = side_streams(hidden_states.device, lanes)
+        lanes = len(streams)
+        bounds = [B * k // lanes for k in range(lanes + 1)]
+        kv = [self._kv_buffer(i, hidden_states)[0] for i in range(L)]  # fresh [B, N, 2D] buffers, one per layer
+        out = torch.empty(hidden_states.shape, dtype=self.transformer_blocks[-1].stream_dtype, device=hidden_states.device)
+        start = torch.cuda.Event()
+        start.record(main)
+        state = []
+        for k, s in enumerate(streams):
+            s.wait_event(start)
+            b0, b1 = bounds[k], bounds[k + 1]
+            state.append([hidden_states[b0:b1], encoder_hidden_states[b0:b1], temb[b0:b1]])
+        for i in range(L):
+            for k, s in enumerate(streams):
+                b0, b1 = bounds[k], bounds[k + 1]
+                h, e, t = state[k]
+                with torch.cuda.stream(s):
+                    e, h = self._run_block(i, calls, mods, h, e, t, kv_buffer=kv[i][b0:b1], batch0=b0,
+                                           hidden_out=out[b0:b1] if i == L - 1 else None)
+                state[k][0], state[k][1] = h, e
+        for s in streams:
+            done = torch.cuda.Event()
+            done.record(s)
+            main.wait_event(done)
+        return out
+
+    @torch.no_grad()
+    def forward_patches(self, hidden_states_patches: List[torch.Tensor], encoder_hidden_states: torch.Tensor,
+                        temb: torch.Tensor, num_streams: int = 2) -> List[torch.Tensor]:
+        """One PipeFusion step of this stage: every patch through every block, the same kernels on the same
+        operands as ``forward`` called once per patch in patch order (the loop of
+        ``pipelines/pipeline_stable_diffusion_3.py:1549-1644``), with the patches spread over ``num_streams``
+        side streams so that the GPU works on neighbouring patches at once.
+
+        A patch-sized launch leaves CUs idle (1024-token problems make 48-192 tiles for 256 CUs); a second
+        patch's launches fill them.  Patch p runs block l once patch p-1 has finished block l: by then p-1 has
+        written its fresh K/V rows of layer l (which p must see), has read p's still stale rows (which p is about
+        to overwrite), and patch 0 has stored the text states p feeds to block l.  Every other pair of launches
+        touches different layers' buffers.  The modulation of all blocks is computed once for the step.
+
+        Expects patch mode with ``pipeline_patch_idx == 0`` and leaves it at 0, like one ``next_patch()`` per
+        patch.  Not to be recorded into a HIP graph with more than one stream (refused)."""
+        rs = get_runtime_state()
+        P, L = len(hidden_states_patches), len(self.transformer_blocks)
+        if not rs.patch_mode or rs.pipeline_patch_idx != 0 or P != rs.num_pipeline_patch:
+            raise ValueError("forward_patches needs patch mode, pipeline_patch_idx 0 and one input per patch")
+        if num_streams < 1:
+            raise ValueError("num_streams must be at least 1")
+        main = torch.cuda.current_stream()
+        if num_streams > 1 and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("forward_patches with several streams cannot be captured into a graph")
+        calls = self._entry_point_calls()
+        if calls is not None and not self._persistent_buffers_contiguous():
+            calls = None
+        hidden = list(hidden_states_patches)
+        if calls is None:
+            self.modulation.precompute(temb)
+            mods = None
+        else:
+            hidden = [h.contiguous() for h in hidden]
+            encoder_hidden_states, temb = encoder_hidden_states.contiguous(), temb.contiguous()
+            mods = self.modulation.precompute_by_module(temb)
+        device = hidden[0].device
+        streams = [main] if num_streams == 1 else side_streams(device, min(num_streams, P))
+        start = torch.cuda.Event()
+        start.record(main)
+        for s in streams:
+            if s is not main:
+                s.wait_event(start)
+        events = self._patch_events
+        cache = self.encoder_hidden_states_cache
+        try:
+            for front in range(L + P - 1):  # launches are issued along the diagonal, the order they can start in
+                for p in range(P):
+                    i = front - p
+                    if not 0 <= i < L:
+                        continue
+                    s = streams[p % len(streams)]
+                    rs.pipeline_patch_idx = p
+                    with torch.cuda.stream(s):
+                        if p > 0 and streams[(p - 1) % len(streams)] is not s:
+                            s.wait_event(events[(p - 1, i)])
+                        kv = self._kv_buffer(i, hidden[p]) if calls is not None else (None, 0)
+                        if p == 0:
+                            cache[i] = encoder_hidden_states
+                            encoder_hidden_states, hidden[0] = self._run_block(
+                                i, calls, mods, hidden[0], encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1])
+                        else:
+                            _, hidden[p] = self._run_block(
+                                i, calls, mods, hidden[p], cache[i], temb, skip_text_output=True,
+                                kv_buffer=kv[0], kv_row0=kv[1])
+                        if P > 1 and len(streams) > 1:
+                            done = events.get((p, i))
+                            if done is None:
+                                done = events[(p, i)] = torch.cuda.Event()
+                            done.record(s)
+        finally:
+            rs.pipeline_patch_idx = 0
+        for s in streams:
+            if s is not main:
+                joined = torch.cuda.Event()
+                joined.record(s)
+                main.wait_event(joined)
+        for h in hidden:
+            h.record_stream(main)  # allocated on a side stream, read by the caller on its own
+        return hidden
 
 
 class FluxTransformerBlocks(nn.Module):

@@ -25,6 +25,11 @@ def fresh_state():
     reset_runtime_state()
 
 
+def dev_randn(shape, seed, scale=1.0):
+    gen = torch.Generator(device=DEV).manual_seed(seed)
+    return (torch.randn(shape, generator=gen, device=DEV) * scale).to(torch.bfloat16)
+
+
 def make(cls, seed, *args, **kw):
     from hetu_dit_amd import synthetic
 
