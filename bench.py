@@ -440,6 +440,10 @@ def main():
                             "algorithmic operand + residual + result bytes average 177.9 MB per call (activations of both streams, both weight sets, fp32 residual stream)",
             "launches_per_step": n_g // 3, "avg_launch_us": round(ms_g / max(n_g, 1) * 1e3, 2),
             "flops_per_launch": round(fl_g / max(n_g, 1), 1),
+            "measured_in": "three instrumented passes after the timed ones: kernel by kernel on one stream, HIP events "
+                           "around every launch (a launch alone on the GPU); the rocprofv3 trace of `bench.py --single-stream "
+                           "--no-graph` is profiles/<workload>_kernel_stats.txt, that of this command "
+                           "profiles/<workload>_two_streams_kernel_stats.txt",
         },
         "roofline_attention": {
             "kernel": attn_kernel + " (joint flash attention)", "bound": "mfma", "achieved": round(attn_tflops, 1),
