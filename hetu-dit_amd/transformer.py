@@ -48,7 +48,7 @@ class SD3TransformerBlocks(nn.Module):
 
     * ``batch_streams``: a full-sequence pass of B >= 2 batch elements (the CFG pair) runs the elements as
       independent chains on that many side streams, blocks issued alternately -- one chain's launches fill the
-      CUs another's partial last round of tiles leaves idle (SD3 step at B2: 21.1 -> 19.x ms);
+      CUs another's partial last round of tiles leaves idle (about 5 % of the SD3 step at B = 2);
     * ``forward_patches``: the patches of a PipeFusion step, one block apart.
 
     Neither is recorded into a HIP graph: under capture, and whenever a per-launch timer is installed or a
