@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("HDIT_LIBRARY") or os.path.join(HERE, "libhdit.so")
 HDIT_GEMM_MAX_PROBLEMS = 16
 EPI_BIAS, EPI_BIAS_GELU, EPI_GATE_RESIDUAL = 0, 1, 2
 EPI_RESID_F32, EPI_OUT_F32 = 0x10, 0x20
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class GemmProblem(C.Structure):
@@ -118,7 +118,11 @@ class Sd3BlockArgs(C.Structure):
         ("workspace_bytes", C.c_int64),
     ] + [(n, C.c_int32) for n in (
         "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "kv_rows", "kv_row0", "hidden_f32",
-        "encoder_f32", "out_f32", "context_pre_only", "skip_text_output")]
+        "encoder_f32", "out_f32", "context_pre_only", "skip_text_output")] + [
+        ("text_kv", C.c_void_p), ("text_kv_mode", C.c_int32), ("reserved_", C.c_int32)]
+
+
+TEXT_KV_NONE, TEXT_KV_STORE, TEXT_KV_REUSE = 0, 1, 2
 
 
 def _ptrs(*names):

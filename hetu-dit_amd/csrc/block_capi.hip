@@ -42,7 +42,9 @@ Sd3Workspace carve(const hdit_sd3_block_args* a, unsigned char* base) {
   w.n_img = take(B * Ni * D * 2);
   w.n_txt = take(B * Nt * D * 2);
   w.qkv_img = take(B * Ni * (a->kv_buffer ? 1 : 3) * D * 2);
-  w.qkv_txt = take(B * Nt * (a->skip_text_output ? 2 : 3) * D * 2);
+  // text q|k|v; with a text_kv buffer the keys | values live there and only the queries (if any) are here
+  const int txt_cols = a->text_kv_mode != HDIT_TEXT_KV_NONE ? (a->skip_text_output ? 0 : 1) : (a->skip_text_output ? 2 : 3);
+  w.qkv_txt = take(B * Nt * txt_cols * D * 2);
   w.o_img = take(B * Ni * D * 2);
   w.o_txt = take(a->skip_text_output ? 0 : B * Nt * D * 2);
   w.x1_img = (float*)take(B * Ni * D * 4);
@@ -68,6 +70,9 @@ int validate(const hdit_sd3_block_args* a) {
   const bool text_out = !a->context_pre_only && !a->skip_text_output;
   if (text_out && (!a->encoder_out || !w.to_add_out_w || !w.ff_context_in_w || !w.ff_context_out_w)) return HDIT_EINVAL;
   if (a->kv_buffer && (a->kv_rows < a->n_img || a->kv_row0 < 0 || a->kv_row0 + a->n_img > a->kv_rows)) return HDIT_EINVAL;
+  if (a->text_kv_mode < HDIT_TEXT_KV_NONE || a->text_kv_mode > HDIT_TEXT_KV_REUSE) return HDIT_EINVAL;
+  if (a->text_kv_mode != HDIT_TEXT_KV_NONE && (!a->text_kv || (((uintptr_t)a->text_kv) & 15))) return HDIT_EINVAL;
+  if (a->text_kv_mode == HDIT_TEXT_KV_REUSE && !a->skip_text_output) return HDIT_EINVAL;
   return HDIT_OK;
 }
 
@@ -113,7 +118,8 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
     if ((rc = hdit_adaln_gemv(a->temb, w.norm1_w, w.norm1_b, ws.emb_img, B, 6 * D, a->temb_dim, stream))) return rc;
     emb_img = ws.emb_img;
   }
-  if (!emb_txt) {
+  const bool reuse_text_kv = a->text_kv_mode == HDIT_TEXT_KV_REUSE;  // the text stream is not touched at all
+  if (!emb_txt && !reuse_text_kv) {
     if ((rc = hdit_adaln_gemv(a->temb, w.norm1_context_w, w.norm1_context_b, ws.emb_txt, B, (pre_only ? 2 : 6) * D,
                               a->temb_dim, stream)))
       return rc;
@@ -122,8 +128,10 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
   // chunks: shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp; AdaLayerNormContinuous: scale, shift
   const float *sh_a = emb_img, *sc_a = emb_img + D, *g_a = emb_img + 2 * D, *sh_m = emb_img + 3 * D, *sc_m = emb_img + 4 * D,
               *g_m = emb_img + 5 * D;
-  const float *c_sh_a, *c_sc_a, *c_g_a = nullptr, *c_sh_m = nullptr, *c_sc_m = nullptr, *c_g_m = nullptr;
-  if (pre_only) {
+  const float *c_sh_a = nullptr, *c_sc_a = nullptr, *c_g_a = nullptr, *c_sh_m = nullptr, *c_sc_m = nullptr, *c_g_m = nullptr;
+  if (reuse_text_kv) {
+    // no text-stream modulation needed
+  } else if (pre_only) {
     c_sc_a = emb_txt, c_sh_a = emb_txt + D;
   } else {
     c_sh_a = emb_txt, c_sc_a = emb_txt + D, c_g_a = emb_txt + 2 * D, c_sh_m = emb_txt + 3 * D, c_sc_m = emb_txt + 4 * D,
@@ -139,7 +147,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
   jobs[1].x = a->encoder, jobs[1].y = ws.n_txt, jobs[1].shift = c_sh_a, jobs[1].scale = c_sc_a;
   jobs[1].x_sb = (int64_t)Nt * D, jobs[1].x_st = D, jobs[1].y_sb = (int64_t)Nt * D, jobs[1].y_st = D, jobs[1].mod_stride = mdt;
   jobs[1].batch = B, jobs[1].tokens = Nt, jobs[1].x_f32 = a->encoder_f32;
-  if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, nullptr, nullptr, eps, stream))) return rc;
+  if ((rc = hdit_layernorm_modulate_jobs(jobs, reuse_text_kv ? 1 : 2, D, nullptr, nullptr, eps, stream))) return rc;
 
   // 3. q|k|v of both streams in one grouped launch.  With a stale K/V buffer the image stream's k|v rows go
   //    straight into rows [kv_row0, kv_row0 + n_img) of it, one problem per batch element.
@@ -168,16 +176,29 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
     q_img = ws.qkv_img, k_img = kvb, v_img = kvb + (int64_t)D * 2;
     kv_img_rows = a->kv_rows;
   }
-  int64_t tq_ld;
+  int64_t tq_ld = 0, tkv_ld;  // row strides (elements) of the text q and k|v
   const unsigned char *q_txt = nullptr, *k_txt, *v_txt;
-  if (a->skip_text_output) {
+  if (a->text_kv_mode != HDIT_TEXT_KV_NONE) {
+    if (np + 2 > HDIT_GEMM_MAX_PROBLEMS) return HDIT_EUNSUPPORTED;
+    unsigned char* tkv = (unsigned char*)a->text_kv;
+    if (!reuse_text_kv) {
+      if (!a->skip_text_output) {
+        probs[np++] = problem(ws.n_txt, D, aqkv_w, aqkv_b, ws.qkv_txt, D, B * Nt, D, D, HDIT_EPI_BIAS);
+        q_txt = ws.qkv_txt, tq_ld = D;
+      }
+      probs[np++] = problem(ws.n_txt, D, aqkv_w + (int64_t)D * D * 2, aqkv_b ? aqkv_b + (int64_t)D * 2 : nullptr, tkv, 2 * D,
+                            B * Nt, 2 * D, D, HDIT_EPI_BIAS);
+    }
+    tkv_ld = 2 * (int64_t)D;
+    k_txt = tkv, v_txt = tkv + (int64_t)D * 2;
+  } else if (a->skip_text_output) {
     probs[np++] = problem(ws.n_txt, D, aqkv_w + (int64_t)D * D * 2, aqkv_b ? aqkv_b + (int64_t)D * 2 : nullptr, ws.qkv_txt,
                           2 * D, B * Nt, 2 * D, D, HDIT_EPI_BIAS);
-    tq_ld = 2 * (int64_t)D;
+    tkv_ld = 2 * (int64_t)D;
     k_txt = ws.qkv_txt, v_txt = ws.qkv_txt + (int64_t)D * 2;
   } else {
     probs[np++] = problem(ws.n_txt, D, aqkv_w, aqkv_b, ws.qkv_txt, 3 * D, B * Nt, 3 * D, D, HDIT_EPI_BIAS);
-    tq_ld = 3 * (int64_t)D;
+    tq_ld = tkv_ld = 3 * (int64_t)D;
     q_txt = ws.qkv_txt, k_txt = ws.qkv_txt + (int64_t)D * 2, v_txt = ws.qkv_txt + (int64_t)2 * D * 2;
   }
   if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
@@ -191,8 +212,8 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
   seg(at.q[0], q_img, Ni, q_ld, Ni);
   seg(at.k[0], k_img, kv_img_rows, kv_ld, kv_img_rows);
   seg(at.v[0], v_img, kv_img_rows, kv_ld, kv_img_rows);
-  seg(at.k[1], k_txt, Nt, tq_ld, Nt);
-  seg(at.v[1], v_txt, Nt, tq_ld, Nt);
+  seg(at.k[1], k_txt, Nt, tkv_ld, Nt);
+  seg(at.v[1], v_txt, Nt, tkv_ld, Nt);
   seg(at.o[0], ws.o_img, Ni, D, Ni);
   if (!a->skip_text_output) {
     seg(at.q[1], q_txt, Nt, tq_ld, Nt);

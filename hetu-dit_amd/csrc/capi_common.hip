@@ -23,7 +23,7 @@ int check_launch(const char* what) {
 }
 }  // namespace hdit_host
 
-extern "C" __attribute__((visibility("default"))) int hdit_abi_version(void) { return 2; }
+extern "C" __attribute__((visibility("default"))) int hdit_abi_version(void) { return 3; }
 extern "C" __attribute__((visibility("default"))) const char* hdit_last_error(void) { return g_err; }
 
 namespace {

@@ -338,11 +338,14 @@ class Sd3BlockCall:
     def __call__(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
                  out_dtype=bf16, skip_text_output: bool = False, kv_buffer: Optional[torch.Tensor] = None,
                  kv_row0: int = 0, modulation_img: Optional[int] = None, modulation_txt: Optional[int] = None,
-                 hidden_out: Optional[torch.Tensor] = None):
+                 hidden_out: Optional[torch.Tensor] = None, text_kv: Optional[torch.Tensor] = None,
+                 text_kv_mode: int = _lib.TEXT_KV_NONE):
         """Same contract as ``block_sd3``.  ``modulation_img`` / ``modulation_txt``: device addresses of the f32
         [batch, 6 dim] (text stream of a ``context_pre_only`` block: [batch, 2 dim]) adaLN projections of this
         block for this ``temb`` (the caller keeps their tensor alive), or None to have the call compute them.
-        ``hidden_out``: a contiguous [batch, n_img, dim] tensor of ``out_dtype`` to write the image stream to."""
+        ``hidden_out``: a contiguous [batch, n_img, dim] tensor of ``out_dtype`` to write the image stream to.
+        ``text_kv`` / ``text_kv_mode``: bf16 [batch, n_txt, 2 dim] buffer of the text stream's keys | values that
+        this call fills (``TEXT_KV_STORE``) or, with ``skip_text_output``, takes as they are (``TEXT_KV_REUSE``)."""
         a = self.args
         B, Ni, D = hidden_states.shape
         Nt = encoder_hidden_states.shape[1]
@@ -372,8 +375,14 @@ class Sd3BlockCall:
             a.kv_buffer, a.kv_rows, a.kv_row0 = kv_buffer.data_ptr(), kv_buffer.shape[1], kv_row0
         else:
             a.kv_buffer, a.kv_rows, a.kv_row0 = None, 0, 0
+        if text_kv_mode != _lib.TEXT_KV_NONE:
+            if text_kv is None or text_kv.dtype != bf16 or tuple(text_kv.shape) != (B, Nt, 2 * D) or not text_kv.is_contiguous():
+                raise ValueError("text_kv must be a contiguous bf16 [batch, n_txt, 2 * dim] tensor")
+            a.text_kv, a.text_kv_mode = text_kv.data_ptr(), text_kv_mode
+        else:
+            a.text_kv, a.text_kv_mode = None, _lib.TEXT_KV_NONE
         lib = _lib.lib()
-        key = (B, Ni, Nt, bool(skip_text_output), kv_buffer is not None)
+        key = (B, Ni, Nt, bool(skip_text_output), kv_buffer is not None, text_kv_mode)
         nbytes = self._ws_bytes.get(key)
         if nbytes is None:
             nbytes = lib.hdit_block_sd3_workspace_bytes(C.byref(a))

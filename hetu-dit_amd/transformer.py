@@ -14,7 +14,7 @@ from typing import List, Optional, Tuple
 import torch
 from torch import nn
 
-from . import ops
+from . import _lib, ops
 from .blocks import (CogVideoXBlock, FluxSingleTransformerBlock, FluxTransformerBlock, JointTransformerBlock,
                      StackModulation, use_fp32_residual_stream)
 from .cache_manager import get_cache_manager
@@ -69,7 +69,10 @@ class SD3TransformerBlocks(nn.Module):
         use_fp32_residual_stream(self.transformer_blocks)
         self.use_block_entry_points = True
         self.batch_streams = 2
+        self.reuse_text_kv = True  # patch mode: later patches take the text keys / values the first patch projected
         self._block_calls: Optional[List[ops.Sd3BlockCall]] = None
+        # per block: (k|v buffer of the text stream, the text states and temb it was projected from) -- patch mode
+        self._text_kv: List[Optional[tuple]] = [None] * num_layers
         self._patch_events = {}  # (patch, block) -> "block done" event of forward_patches
 
     # -- launching one block ------------------------------------------------------------------------------
@@ -88,13 +91,31 @@ class SD3TransformerBlocks(nn.Module):
         return self._block_calls
 
     def _run_block(self, i: int, calls, mods, hidden, encoder, temb, skip_text_output: bool = False,
-                   kv_buffer=None, kv_row0: int = 0, batch0: int = 0, hidden_out=None):
+                   kv_buffer=None, kv_row0: int = 0, batch0: int = 0, hidden_out=None, patch: Optional[int] = None):
         """Block i on the current stream: ``(encoder_out_or_None, hidden_out)``.  ``batch0``: index of the
-        first batch element of ``hidden`` within the ``temb`` the modulation ``mods`` was computed for."""
+        first batch element of ``hidden`` within the ``temb`` the modulation ``mods`` was computed for.
+        ``patch``: index of the pipeline patch in patch mode.  The later patches of a step are fed the text states
+        the first one stored (``transformer_sd3.py:131-146``), so the text stream's keys and values are the same
+        numbers for all of them: the first patch's call leaves them in a buffer and the later ones take them from
+        there -- as long as they really come with the same text states and the same ``temb``."""
         block = self.transformer_blocks[i]
         if calls is None:
             return block(hidden_states=hidden, encoder_hidden_states=encoder, temb=temb,
                          skip_text_output=skip_text_output)
+        text_kv, text_kv_mode = None, _lib.TEXT_KV_NONE
+        if not self.reuse_text_kv:
+            pass
+        elif patch == 0:
+            held = self._text_kv[i]
+            shape = (encoder.shape[0], encoder.shape[1], 2 * encoder.shape[2])
+            text_kv = held[0] if held is not None and tuple(held[0].shape) == shape and held[0].device == encoder.device \
+                else torch.empty(shape, dtype=torch.bfloat16, device=encoder.device)
+            self._text_kv[i] = (text_kv, encoder, temb, temb._version)
+            text_kv_mode = _lib.TEXT_KV_STORE
+        elif patch is not None and skip_text_output:
+            held = self._text_kv[i]
+            if held is not None and held[1] is encoder and held[2] is temb and held[3] == temb._version:
+                text_kv, text_kv_mode = held[0], _lib.TEXT_KV_REUSE
         flat, offsets = mods
         dim = hidden.shape[2]
         rows_txt = (2 if block.context_pre_only else 6) * dim
@@ -104,7 +125,7 @@ class SD3TransformerBlocks(nn.Module):
             kv_buffer=kv_buffer, kv_row0=kv_row0,
             modulation_img=base + 4 * (offsets[block.norm1] + batch0 * 6 * dim),
             modulation_txt=base + 4 * (offsets[block.norm1_context] + batch0 * rows_txt),
-            hidden_out=hidden_out,
+            hidden_out=hidden_out, text_kv=text_kv, text_kv_mode=text_kv_mode,
         )
 
     def _kv_buffer(self, i: int, hidden: torch.Tensor):
@@ -148,12 +169,12 @@ class SD3TransformerBlocks(nn.Module):
             if rs.patch_mode and rs.pipeline_patch_idx == 0:
                 self.encoder_hidden_states_cache[i] = encoder_hidden_states
                 encoder_hidden_states, hidden_states = self._run_block(
-                    i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1])
+                    i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1], patch=0)
             elif rs.patch_mode:
                 # the text output of these calls is dropped: the block does not compute it
                 _, hidden_states = self._run_block(
                     i, calls, mods, hidden_states, self.encoder_hidden_states_cache[i], temb, skip_text_output=True,
-                    kv_buffer=kv[0], kv_row0=kv[1])
+                    kv_buffer=kv[0], kv_row0=kv[1], patch=rs.pipeline_patch_idx)
             else:
                 encoder_hidden_states, hidden_states = self._run_block(
                     i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1])
@@ -250,11 +271,12 @@ class SD3TransformerBlocks(nn.Module):
                         if p == 0:
                             cache[i] = encoder_hidden_states
                             encoder_hidden_states, hidden[0] = self._run_block(
-                                i, calls, mods, hidden[0], encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1])
+                                i, calls, mods, hidden[0], encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1],
+                                patch=0)
                         else:
                             _, hidden[p] = self._run_block(
                                 i, calls, mods, hidden[p], cache[i], temb, skip_text_output=True,
-                                kv_buffer=kv[0], kv_row0=kv[1])
+                                kv_buffer=kv[0], kv_row0=kv[1], patch=p)
                         if P > 1 and len(streams) > 1:
                             done = events.get((p, i))
                             if done is None:

@@ -327,7 +327,14 @@ int hdit_cfg_euler_step(const void* noise_uncond, const void* noise_cond, const 
  * (core/resource_manager/cache_manager.py:117-149).  modulation_img /
  * modulation_txt: optional precomputed linear(silu(temb)) of norm1 /
  * norm1_context (f32 [batch, 6 dim] / [batch, 6 dim or 2 dim]); NULL => computed
- * here.  workspace: hdit_block_sd3_workspace_bytes(args) bytes, 256-byte aligned,
+ * here.  text_kv (optional): bf16 [batch, n_txt, 2 dim], the text stream's keys |
+ * values.  text_kv_mode HDIT_TEXT_KV_STORE: this call projects them into that
+ * buffer instead of the workspace.  HDIT_TEXT_KV_REUSE (only with
+ * skip_text_output): the buffer already holds them -- models/transformers/
+ * transformer_sd3.py:131-146 feeds every later patch of a step the text states
+ * the first patch stored, so with the same temb their keys and values are the
+ * numbers the first patch's call stored -- and the text stream's norm1 and
+ * projection are not run.  workspace: hdit_block_sd3_workspace_bytes(args) bytes, 256-byte aligned,
  * caller-owned, contents undefined afterwards.
  * Arguments are validated before anything is enqueued.  A block is a sequence of
  * this library's launches, so if a later launch is refused (HDIT_ELAUNCH from the
@@ -358,7 +365,14 @@ typedef struct hdit_sd3_block_args {
   int32_t kv_rows, kv_row0;
   int32_t hidden_f32, encoder_f32, out_f32;
   int32_t context_pre_only, skip_text_output;
+  void* text_kv;
+  int32_t text_kv_mode;
+  int32_t reserved_;
 } hdit_sd3_block_args;
+
+#define HDIT_TEXT_KV_NONE 0
+#define HDIT_TEXT_KV_STORE 1
+#define HDIT_TEXT_KV_REUSE 2
 
 int64_t hdit_block_sd3_workspace_bytes(const hdit_sd3_block_args* args);
 int hdit_block_sd3(const hdit_sd3_block_args* args, void* stream);

@@ -92,6 +92,51 @@ def test_block_sd3_one_call_pipefusion_patch(hdit):
         assert torch.equal(kv_c, entry.tensors[0]), f"stale buffer after patch {p}"
 
 
+def test_block_sd3_text_keys_and_values_stored_once_per_step(hdit):
+    """The first patch's call leaves the text stream's keys | values in a buffer (``HDIT_TEXT_KV_STORE``), the later
+    patches of the step take them from there (``HDIT_TEXT_KV_REUSE``) instead of normalising and projecting the same
+    text states again: same bits as the calls that project them every time, and as the Python block."""
+    from hetu_dit_amd import _lib, ops, synthetic
+    from hetu_dit_amd.cache_manager import get_cache_manager
+    from hetu_dit_amd.runtime_state import get_runtime_state
+
+    B, N, Nt, D, H, P = 2, 512, 77, 512, 8, 4
+    starts = [N // P * i for i in range(P + 1)]
+    blk, params = make_block(False, 11, D, H)
+    x_prev, x_now = synthetic.randn_bf16((B, N, D), 12).to(DEV), synthetic.randn_bf16((B, N, D), 13).to(DEV)
+    e, t = synthetic.randn_bf16((B, Nt, D), 14).to(DEV), synthetic.randn_bf16((B, D), 15).to(DEV)
+    rs = get_runtime_state()
+    rs.set_token_patches(starts)
+    rs.set_patched_mode(False)
+    blk(hidden_states=x_prev, encoder_hidden_states=e, temb=t)  # fills the layer's buffer
+    torch.cuda.synchronize()
+    entry = get_cache_manager()._entry(blk.attn, "attn")
+    kv_c = entry.tensors[0].contiguous().clone()
+    entry.tensors[0] = entry.tensors[0].contiguous().clone()
+    rs.set_patched_mode(True)
+    call = ops.Sd3BlockCall(blk)
+    text_kv = torch.full((B, Nt, 2 * D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    for p in range(P):
+        rs.pipeline_patch_idx = p
+        xp = x_now[:, starts[p]:starts[p + 1]].contiguous()
+        enc_py, hid_py = blk(hidden_states=xp, encoder_hidden_states=e, temb=t, skip_text_output=p > 0)
+        enc_c, hid_c = call(xp, e, t, skip_text_output=p > 0, kv_buffer=kv_c, kv_row0=starts[p], text_kv=text_kv,
+                            text_kv_mode=_lib.TEXT_KV_STORE if p == 0 else _lib.TEXT_KV_REUSE)
+        torch.cuda.synchronize()
+        assert torch.equal(hid_c, hid_py), f"patch {p}"
+        assert torch.equal(enc_c, enc_py) if p == 0 else enc_c is None
+        assert torch.equal(kv_c, entry.tensors[0]), f"stale buffer after patch {p}"
+        assert torch.isfinite(text_kv.float()).all()
+    # what cannot be meant is refused before anything is launched
+    with pytest.raises(_lib.HditError):
+        call(xp, e, t, skip_text_output=False, kv_buffer=kv_c, kv_row0=starts[1], text_kv=text_kv, text_kv_mode=_lib.TEXT_KV_REUSE)
+    with pytest.raises(ValueError):
+        call(xp, e, t, skip_text_output=True, kv_buffer=kv_c, kv_row0=starts[1], text_kv=text_kv[:, :10], text_kv_mode=_lib.TEXT_KV_REUSE)
+    a = call.args
+    a.text_kv, a.text_kv_mode = None, _lib.TEXT_KV_STORE
+    assert _lib.lib().hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
+
+
 def test_block_sd3_refuses_bad_arguments(hdit):
     from hetu_dit_amd import _lib
 
