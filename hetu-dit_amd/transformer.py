@@ -83,11 +83,17 @@ class SD3TransformerBlocks(nn.Module):
             return None
         if any(getattr(b.attn, "fp8_attention", False) for b in self.transformer_blocks):
             return None
-        if self._block_calls is None or len(self._block_calls) != len(self.transformer_blocks):
-            self._block_calls = [ops.Sd3BlockCall(b) for b in self.transformer_blocks]
-        else:
-            for call in self._block_calls:
-                call.refresh()
+        try:
+            if self._block_calls is None or len(self._block_calls) != len(self.transformer_blocks):
+                self._block_calls = [ops.Sd3BlockCall(b) for b in self.transformer_blocks]
+            else:
+                for call in self._block_calls:
+                    call.refresh()
+        except AttributeError:
+            # a block whose sub-modules were replaced by something the entry point's weight table cannot describe
+            self._block_calls = None
+            self.use_block_entry_points = False
+            return None
         return self._block_calls
 
     def _run_block(self, i: int, calls, mods, hidden, encoder, temb, skip_text_output: bool = False,
