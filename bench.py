@@ -336,13 +336,17 @@ def main():
         step.set_single_stream(False)
         got = step()
         torch.cuda.synchronize()
-        if not torch.equal(got, ref):
-            raise SystemExit("the multi-stream pass does not reproduce the single-stream pass")
+        same = torch.equal(got, ref)
         del saved, got, ref
-        use_graph = False
-        run = step
-        launch = multi_stream
-    elif use_graph:
+        if same:
+            use_graph = False
+            run = step
+            launch = multi_stream
+        else:
+            print("bench.py: the multi-stream pass does not reproduce the single-stream pass; timing the latter",
+                  file=sys.stderr)
+            step.set_single_stream(True)
+    if launch is None and use_graph:
         saved = [t.clone() for t in kv_buffers()]
         ref = step().clone()
         for t, s0 in zip(kv_buffers(), saved):
@@ -359,7 +363,7 @@ def main():
             use_graph = False
         del saved
         run = graph.replay if use_graph else step
-    else:
+    elif launch is None:
         run = step
 
     torch.cuda.synchronize()
