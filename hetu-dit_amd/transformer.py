@@ -71,7 +71,8 @@ class SD3TransformerBlocks(nn.Module):
         self.batch_streams = 2
         self.reuse_text_kv = True  # patch mode: later patches take the text keys / values the first patch projected
         self._block_calls: Optional[List[ops.Sd3BlockCall]] = None
-        # per block: (k|v buffer of the text stream, the text states and temb it was projected from) -- patch mode
+        # per block: (k|v buffer of the text stream, the text states and temb it was projected from, with their
+        # in-place modification counters) -- patch mode
         self._text_kv: List[Optional[tuple]] = [None] * num_layers
         self._patch_events = {}  # (patch, block) -> "block done" event of forward_patches
 
@@ -116,11 +117,12 @@ class SD3TransformerBlocks(nn.Module):
             shape = (encoder.shape[0], encoder.shape[1], 2 * encoder.shape[2])
             text_kv = held[0] if held is not None and tuple(held[0].shape) == shape and held[0].device == encoder.device \
                 else torch.empty(shape, dtype=torch.bfloat16, device=encoder.device)
-            self._text_kv[i] = (text_kv, encoder, temb, temb._version)
+            self._text_kv[i] = (text_kv, encoder, encoder._version, temb, temb._version)
             text_kv_mode = _lib.TEXT_KV_STORE
         elif patch is not None and skip_text_output:
             held = self._text_kv[i]
-            if held is not None and held[1] is encoder and held[2] is temb and held[3] == temb._version:
+            if held is not None and held[1] is encoder and held[2] == encoder._version and held[3] is temb \
+                    and held[4] == temb._version:
                 text_kv, text_kv_mode = held[0], _lib.TEXT_KV_REUSE
         flat, offsets = mods
         dim = hidden.shape[2]
