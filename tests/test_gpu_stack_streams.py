@@ -112,3 +112,22 @@ def test_forward_patches_refuses_what_it_cannot_run(hdit):
     with pytest.raises(ValueError):
         stack.forward_patches(xs, e, t, num_streams=0)
     assert len(stack.forward_patches(xs, e, t)) == P
+
+
+def test_stack_takes_changing_batch_and_sequence_sizes(hdit):
+    """One stack, passes of different batch sizes, token counts and stream element types one after the other: the
+    prefilled whole-block calls, the modulation regrouping and the side streams hold nothing that is tied to the
+    first shape they saw.  Every pass is compared with the kernel-by-kernel pass on one stream."""
+    D, H, L = 256, 4, 3
+    stack = make_stack(L, D, H, 77)
+    for k, (B, Ni, Nt, f32) in enumerate([(2, 512, 77, False), (1, 300, 40, False), (3, 1024, 8, True), (2, 512, 77, False)]):
+        x, e, t = dev_randn((B, Ni, D), 100 + k), dev_randn((B, Nt, D), 200 + k), dev_randn((B, D), 300 + k)
+        if f32:
+            x, e = x.float(), e.float()
+        stack.use_block_entry_points, stack.batch_streams = False, 1
+        want = stack(x, e, t).clone()
+        torch.cuda.synchronize()
+        stack.use_block_entry_points, stack.batch_streams = True, 2
+        got = stack(x, e, t)
+        torch.cuda.synchronize()
+        assert got.dtype == want.dtype and torch.equal(got, want), f"pass {k}: B {B}, {Ni}+{Nt} tokens"
