@@ -379,6 +379,22 @@ def main():
     # average shader clock over the timed passes (counter pairs per CU, median)
     shader_clock_ghz = ops.shader_clock_ghz(clk0, clk1)
 
+    # the same workload on one stream, beside the multi-stream figure: eager, then the same passes again, so that
+    # both forms are timed on this box in this run (HIP-graph replay of the single-stream pass: --single-stream)
+    single_stream = None
+    if launch is not None:
+        step.set_single_stream(True)
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        n = min(args.steps, 10)
+        t0 = time.perf_counter()
+        for _ in range(n):
+            step()
+        torch.cuda.synchronize()
+        single_stream = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / n, 3), "steps": n, "launch": "eager"}
+        step.set_single_stream(False)
+
     # one plain device copy of known size (256 MiB read + 256 MiB written): the scale reference for the
     # FETCH_SIZE / WRITE_SIZE hardware counters when this command runs under `rocprofv3 --pmc`
     calib_src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
@@ -440,6 +456,7 @@ def main():
         "dtype": "bf16",
         "data": "synthetic (seeded N(0,1) activations, N(0,0.02) random-init weights, resident in HBM)",
         "config": {"workload": workload_desc, "launch": launch or ("hip-graph replay" if use_graph else "eager")},
+        "single_stream": single_stream,
         "step_tflops": round((gemm_fl + attn_fl) / ms_step / 1e9, 1),
         "shader_clock_ghz": round(shader_clock_ghz, 3) if shader_clock_ghz else None,
         "shader_clock_note": "average over the timed passes, from the shader-clock and 100 MHz counters sampled on the "
