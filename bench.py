@@ -99,10 +99,6 @@ def make_workload(name, dev):
                 for m in obj.modules():
                     if isinstance(m, hetuDiTAttentionWrapper):
                         m.fp8_attention = True
-        # with fp8 attention the stack launches kernel by kernel on one stream: time the graph replay of that
-        for attr in ("multi_stream", "set_single_stream"):
-            if hasattr(step, attr):
-                delattr(step, attr)
         return step, desc + "; attention on the fp8-e4m3 path", gemm, attn, blocks, kernel.replace("attn_fwd_kernel", "attn_fp8_kernel")
     if name == "sd3_1024_transformer":
         # the same 24 blocks inside the whole transformer: latent in, guided and Euler-updated latent out

@@ -119,7 +119,7 @@ class Sd3BlockArgs(C.Structure):
     ] + [(n, C.c_int32) for n in (
         "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "kv_rows", "kv_row0", "hidden_f32",
         "encoder_f32", "out_f32", "context_pre_only", "skip_text_output")] + [
-        ("text_kv", C.c_void_p), ("text_kv_mode", C.c_int32), ("reserved_", C.c_int32)]
+        ("text_kv", C.c_void_p), ("text_kv_mode", C.c_int32), ("fp8_attention", C.c_int32)]
 
 
 TEXT_KV_NONE, TEXT_KV_STORE, TEXT_KV_REUSE = 0, 1, 2

@@ -24,8 +24,29 @@ struct Sd3Workspace {
   float* x1_txt;           // f32 [B, Nt, D]
   unsigned char* h_img;    // bf16 [B, Ni, F]
   unsigned char* h_txt;    // bf16 [B, Nt, F]
+  float* absmax;           // f32 [3, B, H]: scales of the fp8 attention path
+  unsigned char* fp8;      // its quantised K / V copy
   int64_t bytes;
 };
+
+// Workspace of the fp8 attention of this block: the size depends on the sequence lengths only, so the size query
+// describes the segments with a placeholder address.
+int64_t fp8_attention_bytes(const hdit_sd3_block_args* a) {
+  const int hd = a->dim / a->heads;
+  const int kv_rows = a->kv_buffer ? a->kv_rows : a->n_img;
+  hdit_attn_args at;
+  memset(&at, 0, sizeof(at));
+  const void* somewhere = (const void*)(uintptr_t)256;
+  auto seg = [&](hdit_seq_segment& s, int len) {
+    s.ptr = somewhere, s.stride_b = (int64_t)len * a->dim, s.stride_s = a->dim, s.stride_h = hd, s.len = len;
+  };
+  seg(at.q[0], a->n_img), seg(at.o[0], a->n_img);
+  seg(at.k[0], kv_rows), seg(at.v[0], kv_rows);
+  seg(at.k[1], a->n_txt), seg(at.v[1], a->n_txt);
+  if (!a->skip_text_output) seg(at.q[1], a->n_txt), seg(at.o[1], a->n_txt);
+  at.batch = a->batch, at.heads = a->heads, at.head_dim = hd;
+  return hdit_attn_fp8_workspace_bytes(&at);
+}
 
 Sd3Workspace carve(const hdit_sd3_block_args* a, unsigned char* base) {
   const int64_t B = a->batch, Ni = a->n_img, Nt = a->n_txt, D = a->dim, F = a->ff_dim;
@@ -51,6 +72,8 @@ Sd3Workspace carve(const hdit_sd3_block_args* a, unsigned char* base) {
   w.x1_txt = (float*)take(text_out ? B * Nt * D * 4 : 0);
   w.h_img = take(B * Ni * F * 2);
   w.h_txt = take(text_out ? B * Nt * F * 2 : 0);
+  w.absmax = (float*)take(a->fp8_attention ? 3 * B * a->heads * 4 : 0);
+  w.fp8 = take(a->fp8_attention ? fp8_attention_bytes(a) : 0);
   w.bytes = off;
   return w;
 }
@@ -73,6 +96,8 @@ int validate(const hdit_sd3_block_args* a) {
   if (a->text_kv_mode < HDIT_TEXT_KV_NONE || a->text_kv_mode > HDIT_TEXT_KV_REUSE) return HDIT_EINVAL;
   if (a->text_kv_mode != HDIT_TEXT_KV_NONE && (!a->text_kv || (((uintptr_t)a->text_kv) & 15))) return HDIT_EINVAL;
   if (a->text_kv_mode == HDIT_TEXT_KV_REUSE && !a->skip_text_output) return HDIT_EINVAL;
+  if (a->fp8_attention != 0 && a->fp8_attention != 1) return HDIT_EINVAL;
+  if (a->fp8_attention && fp8_attention_bytes(a) < 0) return HDIT_EINVAL;
   return HDIT_OK;
 }
 
@@ -220,7 +245,12 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
     seg(at.o[1], ws.o_txt, Nt, D, Nt);
   }
   at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
-  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
+  if (a->fp8_attention) {
+    if ((rc = hdit_attn_absmax(&at, ws.absmax, stream))) return rc;
+    if ((rc = hdit_attn_fwd_fp8(&at, ws.absmax, ws.fp8, stream))) return rc;
+  } else if ((rc = hdit_attn_fwd_bf16(&at, stream))) {
+    return rc;
+  }
 
   // 5. out-projections with the gated residual; the stream stays fp32 inside the block
   auto gated = [&](hdit_gemm_problem& p, const void* resid, int resid_f32, const float* gate, int64_t gate_stride, int rows,

@@ -334,6 +334,7 @@ class Sd3BlockCall:
         a.ff_dim = block.ff.module.net[0].proj.weight.shape[0]
         a.temb_dim = block.norm1.linear.weight.shape[1]
         a.context_pre_only = int(bool(block.context_pre_only))
+        a.fp8_attention = int(bool(getattr(block.attn, "fp8_attention", False)))
 
     def __call__(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
                  out_dtype=bf16, skip_text_output: bool = False, kv_buffer: Optional[torch.Tensor] = None,
@@ -382,7 +383,7 @@ class Sd3BlockCall:
         else:
             a.text_kv, a.text_kv_mode = None, _lib.TEXT_KV_NONE
         lib = _lib.lib()
-        key = (B, Ni, Nt, bool(skip_text_output), kv_buffer is not None, text_kv_mode)
+        key = (B, Ni, Nt, bool(skip_text_output), a.kv_rows, text_kv_mode, a.fp8_attention)
         nbytes = self._ws_bytes.get(key)
         if nbytes is None:
             nbytes = lib.hdit_block_sd3_workspace_bytes(C.byref(a))

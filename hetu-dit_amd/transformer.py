@@ -51,8 +51,8 @@ class SD3TransformerBlocks(nn.Module):
       CUs another's partial last round of tiles leaves idle (about 5 % of the SD3 step at B = 2);
     * ``forward_patches``: the patches of a PipeFusion step, one block apart.
 
-    Neither is recorded into a HIP graph: under capture, and whenever a per-launch timer is installed or a
-    block uses fp8 attention, the pass runs on the caller's stream alone."""
+    Neither is recorded into a HIP graph: under capture, and whenever a per-launch timer is installed, the pass
+    runs on the caller's stream alone."""
 
     def __init__(self, num_layers: int = 24, dim: int = 1536, num_attention_heads: int = 24,
                  attention_head_dim: int = 64):
@@ -78,11 +78,9 @@ class SD3TransformerBlocks(nn.Module):
 
     # -- launching one block ------------------------------------------------------------------------------
     def _entry_point_calls(self) -> Optional[List["ops.Sd3BlockCall"]]:
-        """The prefilled whole-block calls, weight pointers re-read, or None where the per-kernel path has to
-        run: switched off, a per-launch timer installed, or fp8 attention asked for (not in the entry point)."""
+        """The prefilled whole-block calls, weight pointers (and the fp8 attention switch) re-read, or None where
+        the per-kernel path has to run: switched off, or a per-launch timer installed."""
         if not self.use_block_entry_points or ops.timer_installed():
-            return None
-        if any(getattr(b.attn, "fp8_attention", False) for b in self.transformer_blocks):
             return None
         try:
             if self._block_calls is None or len(self._block_calls) != len(self.transformer_blocks):

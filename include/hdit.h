@@ -334,7 +334,9 @@ int hdit_cfg_euler_step(const void* noise_uncond, const void* noise_cond, const 
  * transformer_sd3.py:131-146 feeds every later patch of a step the text states
  * the first patch stored, so with the same temb their keys and values are the
  * numbers the first patch's call stored -- and the text stream's norm1 and
- * projection are not run.  workspace: hdit_block_sd3_workspace_bytes(args) bytes, 256-byte aligned,
+ * projection are not run.  fp8_attention != 0: the attention runs on the fp8-e4m3
+ * path (hdit_attn_absmax + hdit_attn_fwd_fp8, their scales and quantised K / V
+ * copy in the workspace).  workspace: hdit_block_sd3_workspace_bytes(args) bytes, 256-byte aligned,
  * caller-owned, contents undefined afterwards.
  * Arguments are validated before anything is enqueued.  A block is a sequence of
  * this library's launches, so if a later launch is refused (HDIT_ELAUNCH from the
@@ -367,7 +369,7 @@ typedef struct hdit_sd3_block_args {
   int32_t context_pre_only, skip_text_output;
   void* text_kv;
   int32_t text_kv_mode;
-  int32_t reserved_;
+  int32_t fp8_attention;
 } hdit_sd3_block_args;
 
 #define HDIT_TEXT_KV_NONE 0

@@ -137,6 +137,25 @@ def test_block_sd3_text_keys_and_values_stored_once_per_step(hdit):
     assert _lib.lib().hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
 
 
+def test_block_sd3_one_call_with_fp8_attention(hdit):
+    """``fp8_attention`` in the entry point's arguments: absmax scales, quantised K / V copy and the fp8 kernel from
+    inside the one call, against the Python block with its attention on the same path (bit-identical) and the
+    oracle at the fp8 tolerance."""
+    from hetu_dit_amd import ops, synthetic
+
+    B, N, Nt, D, H = 2, 700, 77, 512, 8
+    blk, params = make_block(False, 41, D, H)
+    blk.attn.fp8_attention = True
+    x, e, t = synthetic.randn_bf16((B, N, D), 42), synthetic.randn_bf16((B, Nt, D), 43), synthetic.randn_bf16((B, D), 44)
+    enc_py, hid_py = blk(hidden_states=x.to(DEV), encoder_hidden_states=e.to(DEV), temb=t.to(DEV))
+    enc_c, hid_c = ops.Sd3BlockCall(blk)(x.to(DEV), e.to(DEV), t.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(hid_c, hid_py) and torch.equal(enc_c, enc_py)
+    want_e, want_h = oracle.sd3_joint_block(params, x.float(), e.float(), t.float(), H)
+    assert_parity(hid_c, want_h, rel=3e-2, cos=0.999, what="fp8 block hidden")
+    assert_parity(enc_c, want_e, rel=3e-2, cos=0.999, what="fp8 block encoder")
+
+
 def test_block_sd3_refuses_bad_arguments(hdit):
     from hetu_dit_amd import _lib
 

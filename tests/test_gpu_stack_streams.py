@@ -70,12 +70,15 @@ def run_step_sequence(stack, B, Ni, Nt, D, P, entry_points, batch_streams, patch
     return seen
 
 
+@pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("B", [1, 2, 3])
-def test_entry_point_blocks_lanes_and_overlapped_patches_give_the_same_bits(hdit, B):
+def test_entry_point_blocks_lanes_and_overlapped_patches_give_the_same_bits(hdit, B, fp8):
     from hetu_dit_amd.runtime_state import reset_runtime_state
 
     Ni, Nt, D, H, P, L = 1024, 77, 256, 4, 4, 5
     stack = make_stack(L, D, H, 31)
+    for block in stack.transformer_blocks:
+        block.attn.fp8_attention = fp8  # the attention of every form on the fp8-e4m3 path
     want = run_step_sequence(stack, B, Ni, Nt, D, P, entry_points=False, batch_streams=1, patch_streams=0)
     forms = [
         ("entry points, one stream", True, 1, 0),
