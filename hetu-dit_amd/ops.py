@@ -316,7 +316,9 @@ class Sd3BlockCall:
     The weight pointers and the block's geometry are written into the argument struct once (``refresh``
     re-reads them, e.g. after a weight hot-swap re-assigned a ``.data``); a call only sets the stream tensors,
     the modulation and K/V buffer pointers and the flags, which keeps the host cost of a block at one foreign
-    call -- what a block stack launched eagerly on several streams needs."""
+    call -- what a block stack launched eagerly on several streams needs.  The struct is rewritten by every call
+    (the library copies it before returning), so one object serves any number of streams from ONE host thread at
+    a time."""
 
     def __init__(self, block):
         self.block = block
