@@ -150,6 +150,25 @@ def test_sd3_stack_full_size_properties(hdit):
         torch.cuda.synchronize()
         assert_parity(got, full[:, sl].float(), what=f"patch {p} against the rows of the full pass")
         rs.next_patch()
+    # the same step with neighbouring patches one block apart on two streams: the bits of one patch after the other
+    from hetu_dit_amd.cache_manager import get_cache_manager
+
+    buffers = [b for entry in get_cache_manager().cache.values() for b in entry.tensors if b is not None]
+    saved = [b.clone() for b in buffers]
+    xs = [dev_randn((B, Ni // P, D), 20 + p) for p in range(P)]
+    want = []
+    for p in range(P):
+        want.append(stack(xs[p], e, t).clone())
+        rs.next_patch()
+    torch.cuda.synchronize()
+    after = [b.clone() for b in buffers]
+    for b, s0 in zip(buffers, saved):
+        b.copy_(s0)
+    got = stack.forward_patches(xs, e, t, num_streams=2)
+    torch.cuda.synchronize()
+    for p in range(P):
+        assert torch.equal(got[p], want[p]), f"overlapped patch {p}"
+    assert all(torch.equal(a, b) for a, b in zip(buffers, after))
     rs.set_patched_mode(False)
 
     # adaLN-Zero: with the modulation projections zeroed every gate is zero and the stack is the identity
