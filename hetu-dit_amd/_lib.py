@@ -155,7 +155,7 @@ class CogVideoXBlockArgs(C.Structure):
                       "hidden_out", "encoder_out", "workspace")
                 + [("workspace_bytes", C.c_int64), ("norm_eps", C.c_float), ("qk_norm_eps", C.c_float)]
                 + _ints("qk_norm_kind", "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "hidden_f32",
-                        "encoder_f32", "out_f32"))
+                        "encoder_f32", "out_f32", "fp8_attention"))
 
 
 # name -> (restype, argtypes); every symbol include/hdit.h declares

@@ -399,10 +399,25 @@ int validate(const hdit_flux_single_block_args* a) {
 }
 
 struct CogWs {
-  float *emb1, *emb2, *x1_h, *x1_e;
-  unsigned char *joint, *qkv, *o, *h;
+  float *emb1, *emb2, *x1_h, *x1_e, *absmax;
+  unsigned char *joint, *qkv, *o, *h, *fp8;
   int64_t bytes;
 };
+// one joint [text, video] segment per tensor, q | k | v as column ranges of the packed projection
+void cog_attn_args(const hdit_cogvideox_block_args* a, hdit_attn_args& at, const void* q, const void* k, const void* v,
+                   void* o) {
+  const int S = a->n_img + a->n_txt, D = a->dim, hd = D / a->heads;
+  memset(&at, 0, sizeof(at));
+  seg(at.q[0], q, S, 3 * (int64_t)D, hd, S), seg(at.k[0], k, S, 3 * (int64_t)D, hd, S), seg(at.v[0], v, S, 3 * (int64_t)D, hd, S);
+  seg(at.o[0], o, S, D, hd, S);
+  at.batch = a->batch, at.heads = a->heads, at.head_dim = hd, at.scale = 0.f;
+}
+int64_t cog_fp8_bytes(const hdit_cogvideox_block_args* a) {
+  hdit_attn_args at;
+  void* somewhere = (void*)(uintptr_t)256;  // the size depends on the lengths only
+  cog_attn_args(a, at, somewhere, somewhere, somewhere, somewhere);
+  return hdit_attn_fp8_workspace_bytes(&at);
+}
 CogWs carve(const hdit_cogvideox_block_args* a, void* base) {
   const int64_t B = a->batch, S = (int64_t)a->n_img + a->n_txt, D = a->dim, F = a->ff_dim;
   Carver c(base);
@@ -413,6 +428,8 @@ CogWs carve(const hdit_cogvideox_block_args* a, void* base) {
   w.o = c.take(B * S * D * 2);
   w.x1_h = (float*)c.take(B * a->n_img * D * 4), w.x1_e = (float*)c.take(B * a->n_txt * D * 4);
   w.h = c.take(B * S * F * 2);
+  w.absmax = (float*)c.take(a->fp8_attention ? 3 * B * a->heads * 4 : 0);
+  w.fp8 = c.take(a->fp8_attention ? cog_fp8_bytes(a) : 0);
   w.bytes = c.off;
   return w;
 }
@@ -425,6 +442,8 @@ int validate(const hdit_cogvideox_block_args* a) {
   if (!a->norm1_w || !a->norm1_b || !a->norm2_w || !a->norm2_b || !a->qkv_w || !a->to_out_w || !a->ff_in_w || !a->ff_out_w)
     return HDIT_EINVAL;
   if ((a->rope_cos == nullptr) != (a->rope_sin == nullptr)) return HDIT_EINVAL;
+  if (a->fp8_attention != 0 && a->fp8_attention != 1) return HDIT_EINVAL;
+  if (a->fp8_attention && cog_fp8_bytes(a) < 0) return HDIT_EINVAL;
   return HDIT_OK;
 }
 
@@ -568,11 +587,13 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_cogvideox(const
     if ((rc = hdit_qk_norm_rope(qj, 2, B, H, hd, a->qk_norm_eps, stream))) return rc;
   }
   hdit_attn_args at;
-  memset(&at, 0, sizeof(at));
-  seg(at.q[0], q, S, ld3, hd, S), seg(at.k[0], k, S, ld3, hd, S), seg(at.v[0], v, S, ld3, hd, S);
-  seg(at.o[0], ws.o, S, D, hd, S);
-  at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
-  if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
+  cog_attn_args(a, at, q, k, v, ws.o);
+  if (a->fp8_attention) {
+    if ((rc = hdit_attn_absmax(&at, ws.absmax, stream))) return rc;
+    if ((rc = hdit_attn_fwd_fp8(&at, ws.absmax, ws.fp8, stream))) return rc;
+  } else if ((rc = hdit_attn_fwd_bf16(&at, stream))) {
+    return rc;
+  }
   // one weight set over the joint rows, per-stream gates: per batch element a text and a video problem
   auto gated_pair = [&](const unsigned char* a_joint, int64_t lda, const void* wt, const void* bias, int kdim, const void* res_e,
                         int re_sz, const void* res_h, int rh_sz, const float* emb, void* out_e, int oe_sz, void* out_h, int oh_sz) {

@@ -557,6 +557,7 @@ def block_cogvideox(block, hidden_states, encoder_hidden_states, temb, image_rot
     a.hidden_out, a.encoder_out, a.out_f32 = hidden_out.data_ptr(), encoder_out.data_ptr(), int(out_dtype == torch.float32)
     a.batch, a.n_img, a.n_txt, a.dim, a.heads = B, N, Nt, D, attn.heads_per_device
     a.ff_dim, a.temb_dim = ff.module.net[0].proj.weight.shape[0], temb.shape[1]
+    a.fp8_attention = int(bool(getattr(attn, "fp8_attention", False)))
     lib = _lib.lib()
     _run_block(a, lib.hdit_block_cogvideox_workspace_bytes, lib.hdit_block_cogvideox, "hdit_block_cogvideox",
                hidden_states.device, ptr.keep)

@@ -440,7 +440,8 @@ int hdit_block_flux_single(const hdit_flux_single_block_args* args, void* stream
  * (norm_eps), one projection set over the joint [text, video] rows, LayerNorm or
  * RMSNorm per head on q, k (qk_norm_kind, weights / biases [head_dim]), rotation
  * of the video rows only (rope_cos / rope_sin f32 [n_img, head_dim] or NULL),
- * batch <= HDIT_GEMM_MAX_PROBLEMS / 2.  Returns hidden_out [batch, n_img, dim] and
+ * batch <= HDIT_GEMM_MAX_PROBLEMS / 2.  fp8_attention != 0: the attention on the
+ * fp8-e4m3 path, as in hdit_block_sd3.  Returns hidden_out [batch, n_img, dim] and
  * encoder_out [batch, n_txt, dim]. */
 typedef struct hdit_cogvideox_block_args {
   const void *norm1_w, *norm1_b, *norm1_ln_w, *norm1_ln_b, *norm2_w, *norm2_b, *norm2_ln_w, *norm2_ln_b;
@@ -459,6 +460,7 @@ typedef struct hdit_cogvideox_block_args {
   int32_t qk_norm_kind;
   int32_t batch, n_img, n_txt, dim, heads, ff_dim, temb_dim;
   int32_t hidden_f32, encoder_f32, out_f32;
+  int32_t fp8_attention;
 } hdit_cogvideox_block_args;
 
 int64_t hdit_block_cogvideox_workspace_bytes(const hdit_cogvideox_block_args* args);
