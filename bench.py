@@ -73,7 +73,7 @@ def randomize_(module, device, seed=0):
     return module
 
 
-WORKLOADS = ("sd3_1024", "sd3_1024_transformer", "sd3_pipefusion", "flux_1024", "cogvideox_5b", "sd3_1024_fp8",
+WORKLOADS = ("sd3_1024", "sd3_1024_transformer", "sd3_pipefusion", "sd3_pipefusion_b1", "flux_1024", "cogvideox_5b", "sd3_1024_fp8",
              "cogvideox_5b_fp8")
 
 
@@ -125,7 +125,7 @@ def make_workload(name, dev):
     cfg = synthetic.CONFIGS[name]
     B, Ni, Nt, D = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"]
     S = Ni + Nt
-    if name in ("sd3_1024", "sd3_pipefusion"):
+    if name in ("sd3_1024", "sd3_pipefusion", "sd3_pipefusion_b1"):
         stack = build_stack(cfg, dev)
         e, t = rnd(B, Nt, D), rnd(B, D)
         if name == "sd3_1024":
@@ -171,7 +171,7 @@ def make_workload(name, dev):
         # stream only supplies keys and values (k|v projection, no query rows, no out-projection, no MLP)
         gemm = (24.0 * Sq * D * D * B * L - 18.0 * Nt * D * D * B) + (P - 1) * (24.0 * Np + 4.0 * Nt) * D * D * B * L
         attn = 4.0 * Sq * S * D * B * L + (P - 1) * 4.0 * Np * S * D * B * L
-        desc = ("configs[3]: SD3 PipeFusion shard, 24 joint blocks x 4 patches, B2, query 1024 image + 333 text tokens "
+        desc = (f"configs[3]: SD3 PipeFusion shard, 24 joint blocks x 4 patches, B{B}, query 1024 image + 333 text tokens "
                 "against the 4096 + 333 stale K/V buffer")
         return step, desc, gemm, attn, L * P, "attn_fwd_kernel<64>"
     if name == "flux_1024":

@@ -64,6 +64,8 @@ CONFIGS: Dict[str, dict] = {
     "flux_1024": dict(family="flux", batch=1, n_img=4096, n_txt=512, dim=3072, heads=24, head_dim=128, grid=(64, 64)),
     "sd3_pipefusion": dict(family="sd3", batch=2, n_img=4096, n_txt=333, dim=1536, heads=24, head_dim=64, layers=24,
                            patches=4),
+    "sd3_pipefusion_b1": dict(family="sd3", batch=1, n_img=4096, n_txt=333, dim=1536, heads=24, head_dim=64, layers=24,
+                              patches=4),
     "cogvideox_5b": dict(family="cogvideox", batch=1, n_img=17550, n_txt=226, dim=3072, heads=48, head_dim=64,
                          grid=(13, 30, 45), temb_dim=512),
 }
