@@ -2,15 +2,18 @@
 reference's ``hetuDiTBaseWrapper._wrap_layers`` / ``_register_cache``
 (``model_executor/diffusion_executor/models/base_model.py:59-112,:162-178``): every child whose *name* is in
 ``submodule_name_to_wrap`` or whose *class* is in ``submodule_classes_to_wrap`` is replaced by
-``hetuDiTLayerWrappersRegister.get_wrapper(child)(child, **submodule_addition_args.get(name, {}))``, children
-of a wrapper are not descended into, and every attention wrapper gets a cache entry **keyed by the wrapper
-object** -- the object the attention processors later pass as ``layer=attn``
+``hetuDiTLayerWrappersRegister.get_wrapper(child)(child, **submodule_addition_args.get(name, {}))``.  A wrapper
+itself is skipped by the walk, but the module it wraps is not: the walk goes on into ``wrapper.module`` and wraps
+what matches there too (with the reference's SD3 class list ``[FeedForward, nn.Conv2d, PatchEmbed]`` that is how
+``pos_embed.module.proj`` becomes a ``hetuDiTConv2dWrapper``).  Every attention wrapper gets a cache entry
+**keyed by the wrapper object** -- the object the attention processors later pass as ``layer=attn``
 (``layers/attention_processor.py:702-707``)."""
 from typing import Dict, List, Optional, Sequence, Type
 
 from torch import nn
 
 from .cache_manager import get_cache_manager
+from .layers import conv as _conv  # noqa: F401  (registers the nn.Conv2d wrapper)
 from .layers.base_layer import hetuDiTDiffusionLayerBaseWrapper
 from .parallel_state import get_sequence_parallel_world_size
 from .registry import hetuDiTLayerWrappersRegister

@@ -359,7 +359,10 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fp8_kernel(const
       // exactly those output columns when the masked tile ran last -- so the distance is made explicit here, once
       // per workgroup.
       // (The accumulators are operands of the statement, so it sits behind the MFMAs that write them and in front
-      // of every instruction that reads them.)
+      // of every instruction that reads them.)  Regression case: tests/test_gpu_ops.py,
+      // test_attention_fp8_masked_last_tile_tail_columns (constant-V outputs, masked last tile, both head sizes).
+      // The other reads of an MFMA result in this kernel (the column maxima behind the score MFMAs, the
+      // multiply-add of the d = 128 path) rely on the compiler's own wait states.
       if constexpr (DB == 2)
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(oacc[0][0]), "+v"(oacc[0][1]), "+v"(oacc[1][0]), "+v"(oacc[1][1]));
       else

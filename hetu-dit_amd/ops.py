@@ -280,7 +280,8 @@ def block_sd3(block, hidden_states: torch.Tensor, encoder_hidden_states: torch.T
     text_out = not pre_only and not skip_text_output
     hidden_out = torch.empty(B, Ni, D, dtype=out_dtype, device=hidden_states.device)
     encoder_out = torch.empty(B, Nt, D, dtype=out_dtype, device=hidden_states.device) if text_out else None
-    a.hidden, a.encoder, a.temb = hidden_states.data_ptr(), encoder_hidden_states.data_ptr(), temb.contiguous().data_ptr()
+    temb = temb.contiguous()  # bound to a name and kept below: a temporary's memory could be handed to the workspace
+    a.hidden, a.encoder, a.temb = hidden_states.data_ptr(), encoder_hidden_states.data_ptr(), temb.data_ptr()
     a.hidden_out, a.encoder_out = hidden_out.data_ptr(), (encoder_out.data_ptr() if text_out else None)
     a.batch, a.n_img, a.n_txt, a.dim, a.heads = B, Ni, Nt, D, attn.heads_per_device
     a.ff_dim, a.temb_dim = ff.module.net[0].proj.weight.shape[0], temb.shape[1]
@@ -325,6 +326,28 @@ class Sd3BlockCall:
         self.args = _lib.Sd3BlockArgs()
         self._ws_bytes = {}
         self.refresh()
+
+    @staticmethod
+    def describes(block) -> bool:
+        """Whether ``block`` has the sub-modules the entry point's weight table is filled from (an explicit
+        check of the structure, so that a genuine ``AttributeError`` in ``refresh`` is not mistaken for it)."""
+        from .layers.attention_processor import hetuDiTAttentionWrapper
+        from .layers.feedforward import hetuDiTFeedForwardWrapper
+
+        def adaln(n):
+            return isinstance(getattr(n, "linear", None), torch.nn.Linear) and n.linear.bias is not None
+
+        attn = getattr(block, "attn", None)
+        if not isinstance(attn, hetuDiTAttentionWrapper) or getattr(attn, "_add_qkv", None) is None:
+            return False
+        if not (adaln(getattr(block, "norm1", None)) and adaln(getattr(block, "norm1_context", None))):
+            return False
+        ffs = [getattr(block, "ff", None)]
+        if not getattr(block, "context_pre_only", False):
+            ffs.append(getattr(block, "ff_context", None))
+            if getattr(attn.module, "to_add_out", None) is None:
+                return False
+        return all(isinstance(f, hetuDiTFeedForwardWrapper) and f.module.net[0].proj.bias is not None for f in ffs)
 
     def refresh(self):
         block, a = self.block, self.args

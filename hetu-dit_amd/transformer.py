@@ -9,6 +9,7 @@ blocks" with each model family's call convention and patch-mode rules.
   ``cat([text, image])``, single blocks on the joint sequence, split.
 * CogVideoX (``cogvideox_transformer_3d.py:99-127``).
 """
+import warnings
 from typing import List, Optional, Tuple
 
 import torch
@@ -82,17 +83,19 @@ class SD3TransformerBlocks(nn.Module):
         the per-kernel path has to run: switched off, or a per-launch timer installed."""
         if not self.use_block_entry_points or ops.timer_installed():
             return None
-        try:
-            if self._block_calls is None or len(self._block_calls) != len(self.transformer_blocks):
-                self._block_calls = [ops.Sd3BlockCall(b) for b in self.transformer_blocks]
-            else:
-                for call in self._block_calls:
-                    call.refresh()
-        except AttributeError:
-            # a block whose sub-modules were replaced by something the entry point's weight table cannot describe
-            self._block_calls = None
-            self.use_block_entry_points = False
-            return None
+        if self._block_calls is None or len(self._block_calls) != len(self.transformer_blocks):
+            unfit = [i for i, b in enumerate(self.transformer_blocks) if not ops.Sd3BlockCall.describes(b)]
+            if unfit:
+                # sub-modules replaced by something the entry point's weight table cannot describe
+                warnings.warn(f"SD3TransformerBlocks: blocks {unfit} do not have the layout hdit_block_sd3 takes; "
+                              "the stack runs kernel by kernel on one stream from now on", RuntimeWarning)
+                self._block_calls = None
+                self.use_block_entry_points = False
+                return None
+            self._block_calls = [ops.Sd3BlockCall(b) for b in self.transformer_blocks]
+        else:
+            for call in self._block_calls:
+                call.refresh()
         return self._block_calls
 
     def _run_block(self, i: int, calls, mods, hidden, encoder, temb, skip_text_output: bool = False,

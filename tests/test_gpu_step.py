@@ -149,6 +149,65 @@ def test_sd3_transformer_latent_to_noise(hdit):
     assert_parity(new, want.float(), what="denoise step")
 
 
+def test_conv2d_wrapper_patch_convolution(hdit):
+    """``hetuDiTConv2dWrapper`` (reference layers/conv.py:19-113) on one GPU: the p x p stride-p convolution
+    against ``F.conv2d`` in fp32; other geometries are refused."""
+    from torch import nn
+
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.layers.conv import hetuDiTConv2dWrapper
+
+    for (cin, cout, p, H, W, bias) in [(16, 256, 2, 32, 48, True), (4, 64, 4, 16, 16, False), (8, 128, 1, 6, 10, True)]:
+        print(f"conv wrapper {cin} {cout} {p} {H} {W} {bias}", flush=True)
+        conv = nn.Conv2d(cin, cout, p, stride=p, bias=bias)
+        synthetic.init_module_(conv, 21)
+        w = conv.weight.detach().float()
+        b = conv.bias.detach().float() if bias else None
+        wrap = hetuDiTConv2dWrapper(conv, is_first_layer=True).to(DEV)
+        x = synthetic.randn_bf16((2, cin, H, W), 22)
+        got = wrap(x.to(DEV))
+        want = torch.nn.functional.conv2d(x.float(), w, b, stride=p)
+        assert got.shape == want.shape
+        assert_parity(got, want, what="conv2d wrapper")
+    bad = hetuDiTConv2dWrapper(nn.Conv2d(4, 8, 3, padding=1)).to(DEV).to(torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        bad(torch.zeros(1, 4, 8, 8, dtype=torch.bfloat16, device=DEV))
+
+
+def test_sd3_transformer_wrapped_with_the_reference_class_list(hdit):
+    """The transformer after ``wrap_layers(model, [FeedForward, nn.Conv2d, PatchEmbed], ["attn"])`` -- the call
+    of the reference's SD3 wrapper (transformer_sd3.py:36) -- computes what it did before: the patch embedding
+    reads its weights through the Conv2d wrapper."""
+    from torch import nn
+
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.base_model import wrap_layers
+    from hetu_dit_amd.layers.conv import hetuDiTConv2dWrapper
+    from hetu_dit_amd.layers.modules import FeedForward, PatchEmbed
+    from hetu_dit_amd.transformer_sd3 import SD3Transformer2DModel
+
+    L, heads = 2, 4
+    model = SD3Transformer2DModel(sample_size=32, patch_size=2, in_channels=16, num_layers=L, attention_head_dim=64,
+                                  num_attention_heads=heads, joint_attention_dim=128, caption_projection_dim=256,
+                                  pooled_projection_dim=64, out_channels=16, pos_embed_max_size=24)
+    synthetic.init_module_(model, 7)
+    model = model.to(DEV)
+    lat = synthetic.randn_bf16((2, 16, 32, 40), 8).to(DEV)
+    enc = synthetic.randn_bf16((2, 77, 128), 9).to(DEV)
+    pooled = synthetic.randn_bf16((2, 64), 10).to(DEV)
+    t = torch.tensor([981.0, 981.0], device=DEV)
+    before = model(lat, enc, pooled, t).clone()
+    wrapped = wrap_layers(model, [FeedForward, nn.Conv2d, PatchEmbed], ["attn"])
+    assert len(wrapped) == 1 and isinstance(model.pos_embed.module.proj, hetuDiTConv2dWrapper)
+    params = step_params(model)
+    assert "pos_embed.proj.weight" in params
+    after = model(lat, enc, pooled, t)
+    torch.cuda.synchronize()
+    assert torch.equal(before, after)
+    want = S.sd3_transformer(params, lat.float().cpu(), enc.float().cpu(), pooled.float().cpu(), t.cpu(), heads, L, 2, 24)
+    assert_parity(after, want, what="sd3 transformer through the Conv2d wrapper")
+
+
 def test_rope_table_kernel(hdit):
     from hetu_dit_amd import synthetic
     from oracle import ops as O

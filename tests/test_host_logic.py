@@ -192,6 +192,48 @@ def test_wrap_layers_and_register_cache_follow_the_reference_rules():
     reset_cache_manager()
 
 
+def test_wrap_layers_with_the_reference_sd3_class_list():
+    """The reference wraps the SD3 transformer with ``submodule_classes_to_wrap=[FeedForward, nn.Conv2d,
+    PatchEmbed]``, ``submodule_name_to_wrap=["attn"]`` (models/transformers/transformer_sd3.py:36).  The walk
+    skips a wrapper but goes on into the module it wraps, so the patch embedding's ``proj`` gets the Conv2d
+    wrapper (layers/conv.py:19-31) and the patch-embedding wrapper must still find ``proj.weight`` / ``.bias``
+    through it."""
+    from hetu_dit_amd.base_model import wrap_layers
+    from hetu_dit_amd.layers.conv import hetuDiTConv2dWrapper
+    from hetu_dit_amd.layers.embeddings import hetuDiTPatchEmbedWrapper
+    from hetu_dit_amd.layers.modules import FeedForward, PatchEmbed
+    from hetu_dit_amd.registry import hetuDiTLayerWrappersRegister
+    from hetu_dit_amd.transformer_sd3 import SD3Transformer2DModel
+
+    assert hetuDiTLayerWrappersRegister.get_wrapper(nn.Conv2d(3, 4, 2, 2)) is hetuDiTConv2dWrapper
+    model = SD3Transformer2DModel(sample_size=16, num_layers=2, attention_head_dim=64, num_attention_heads=2,
+                                  joint_attention_dim=64, caption_projection_dim=128, pooled_projection_dim=64,
+                                  pos_embed_max_size=16)
+    conv = model.pos_embed.module.proj
+    wrapped = wrap_layers(model, [FeedForward, nn.Conv2d, PatchEmbed], ["attn"])
+    assert len(wrapped) == 1 and wrapped[0] is model.pos_embed.module.proj
+    w = model.pos_embed.module.proj
+    assert isinstance(w, hetuDiTConv2dWrapper) and w.module is conv and w.is_first_layer
+    assert isinstance(model.pos_embed, hetuDiTPatchEmbedWrapper)
+    # attribute fall-through: what the patch-embedding wrapper reads
+    assert model.pos_embed.module.proj.weight is conv.weight and model.pos_embed.module.proj.bias is conv.bias
+    assert "pos_embed.module.proj.module.weight" in dict(model.named_parameters())
+    # an unwrapped model gets the same result from the same call: PatchEmbed first, then its proj
+    class Bare(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.pos_embed = PatchEmbed(16, 16, 2, 4, 64, pos_embed_max_size=8)
+
+    bare = Bare()
+    wrapped = wrap_layers(bare, [FeedForward, nn.Conv2d, PatchEmbed], ["attn"])
+    assert [type(x) for x in wrapped] == [hetuDiTPatchEmbedWrapper, hetuDiTConv2dWrapper]
+    assert isinstance(bare.pos_embed.module.proj, hetuDiTConv2dWrapper)
+    # geometry the wrapper does not run is refused, not handed to a library convolution
+    odd = hetuDiTConv2dWrapper(nn.Conv2d(4, 8, 3, stride=1, padding=1), is_first_layer=False)
+    with pytest.raises(NotImplementedError, match="kernel = stride"):
+        odd._patch_size()
+
+
 def test_patch_embed_height_from_input_config():
     """The patch-embedding wrapper takes the whole image's latent rows from input_config.height //
     vae_scale_factor like the reference (layers/embeddings.py:33-36), else from set_patches."""
