@@ -47,6 +47,9 @@ class hetuDiTConv2dWrapper(hetuDiTDiffusionLayerBaseWrapper):
         if H % p or W % p:
             raise ValueError(f"input {H}x{W} is not a multiple of the kernel size {p}")
         D = m.weight.shape[0]
+        if (C * p * p) % 64 or D % 8:
+            raise NotImplementedError(f"the GEMM behind this wrapper needs in_channels * p * p ({C * p * p}) to be a "
+                                      f"multiple of 64 and out_channels ({D}) a multiple of 8")
         rows = ops.patchify(x.contiguous(), p)  # [B, T, C p p]
         out = torch.empty(B, rows.shape[1], D, dtype=torch.bfloat16, device=x.device)
         bias = m.bias.data if m.bias is not None else None

@@ -83,6 +83,137 @@ def test_gemm_full_size_sampled_rows(hdit, m_img, m_txt, n, k, epi):
         assert torch.isfinite(out.float()).all()
 
 
+# One launch per case, a list of problems (rows, n, k, epilogue, f32 stream?, problems that share the left operand
+# with the first one): the launches of the Flux (configs[2]) and CogVideoX (configs[4]) blocks whose tile shapes and
+# two-phase plans differ from the SD3 ones -- the Flux single block's [q|k|v] + GELU(proj_mlp) call on one operand,
+# its proj_out (k = 15360, gated onto the fp32 stream), the Flux double block's QKV and FF2 (k = 12288, gated fp32)
+# over image + text rows, and CogVideoX's QKV / out-projection / FF2 over 226 text + 17550 video rows.
+WIDE_GEMM_CASES = {
+    "flux_single_qkv_mlp": [(4608, 9216, 3072, "bias", False, False), (4608, 12288, 3072, "gelu", False, True)],
+    "flux_single_proj_out": [(4608, 3072, 15360, "gate", True, False)],
+    "flux_double_qkv": [(4096, 9216, 3072, "bias", False, False), (512, 9216, 3072, "bias", False, False)],
+    "flux_double_ff2": [(4096, 3072, 12288, "gate", True, False), (512, 3072, 12288, "gate", True, False)],
+    "cogvideox_qkv": [(17776, 9216, 3072, "bias", False, False)],
+    "cogvideox_out": [(226, 3072, 3072, "gate", True, False), (17550, 3072, 3072, "gate", True, False)],
+    "cogvideox_ff2": [(226, 3072, 12288, "gate", True, False), (17550, 3072, 12288, "gate", True, False)],
+}
+
+
+@pytest.mark.parametrize("case", sorted(WIDE_GEMM_CASES))
+def test_gemm_full_size_flux_cogvideox_launches(hdit, case):
+    print(f"gemm full size launch {case}", flush=True)
+    ops = hdit.ops
+    probs, checks, first_a = [], [], None
+    for i, (m, n, k, epi, f32, share) in enumerate(WIDE_GEMM_CASES[case]):
+        a = first_a if share else dev_randn((m, k), 10 + i)
+        first_a = a if first_a is None else first_a
+        w, b = dev_randn((n, k), 20 + i, 0.02), dev_randn((n,), 30 + i)
+        rows = sample_rows(m, 40, 40 + i)
+        res = gate = None
+        if epi == "gate":
+            res = dev_randn((m, n), 50 + i)
+            res = res.float() + 2.0 ** -12 if f32 else res  # an fp32 stream value that bf16 cannot hold
+            gate = torch.randn(1, n, generator=torch.Generator(device=DEV).manual_seed(60 + i), device=DEV)
+            out = torch.empty(m, n, dtype=res.dtype, device=DEV)
+            probs.append(ops.gemm_problem(a, w, out, b, ops.EPI_GATE_RESIDUAL, resid=res, gate=gate, rows_per_batch=m))
+        else:
+            out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+            probs.append(ops.gemm_problem(a, w, out, b, ops.EPI_BIAS_GELU if epi == "gelu" else ops.EPI_BIAS))
+        checks.append((a, w, b, res, gate, out, rows, m, epi))
+    ops.gemm_launch(probs)
+    torch.cuda.synchronize()
+    for a, w, b, res, gate, out, rows, m, epi in checks:
+        lin = O.linear(a[rows.to(DEV)].float().cpu(), w.float().cpu(), b.float().cpu())
+        if epi == "gelu":
+            want = O.gelu_tanh(lin)
+        elif epi == "gate":
+            want = res[rows.to(DEV)].float().cpu() + gate.cpu() * lin
+        else:
+            want = lin
+        assert_parity(out[rows.to(DEV)], want, what=f"{case}: {epi} rows of m={m}")
+        assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("S,n_txt,H,hd,kind,axes", [(4608, 512, 24, 128, 1, (16, 56, 56)), (17776, 226, 48, 64, 2, (16, 24, 24))])
+def test_qk_norm_rope_full_size_sampled_rows(hdit, S, n_txt, H, hd, kind, axes):
+    """``hdit_qk_norm_rope`` on q and k of a packed [1, S, 3 H d] projection at the Flux (RMS norm, d 128, 4608
+    rows) and CogVideoX (LayerNorm, d 64, 17776 rows) sizes: sampled rows against the oracle, text rows not rotated,
+    and the v columns untouched."""
+    print(f"qk_norm_rope full size S={S} H={H} d={hd} kind={kind}", flush=True)
+    ops = hdit.ops
+    inner = H * hd
+    qkv = dev_randn((1, S, 3 * inner), 1)
+    before = qkv.clone()
+    wq, wk = dev_randn((hd,), 2, 0.1) + 1.0, dev_randn((hd,), 3, 0.1) + 1.0
+    bq, bk = (dev_randn((hd,), 4, 0.1), dev_randn((hd,), 5, 0.1)) if kind == 2 else (None, None)
+    pos = torch.stack([torch.zeros(S - n_txt), (torch.arange(S - n_txt) // 64).float(), (torch.arange(S - n_txt) % 64).float()], 1)
+    cos, sin = O.flux_rope_table(pos, axes)
+    q = qkv[:, :, :inner].view(1, S, H, hd)
+    k = qkv[:, :, inner : 2 * inner].view(1, S, H, hd)
+    jobs = [ops.qk_norm_rope_job(q, kind, wq, bq, cos.to(DEV), sin.to(DEV), rope_row0=n_txt),
+            ops.qk_norm_rope_job(k, kind, wk, bk, cos.to(DEV), sin.to(DEV), rope_row0=n_txt)]
+    ops.qk_norm_rope(jobs, 1, H, hd, eps=1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(qkv[:, :, 2 * inner :], before[:, :, 2 * inner :])
+    rows = sample_rows(S, 64, 6)
+    rows[2], rows[3] = n_txt - 1, n_txt  # last text row (not rotated), first rotated row
+    for col0, w, b, name in ((0, wq, bq, "q"), (inner, wk, bk, "k")):
+        x = before[0, rows.to(DEV), col0 : col0 + inner].float().cpu().view(-1, H, hd)
+        wf = w.float().cpu()
+        xn = O.rms_norm(x, 1e-6, wf) if kind == 1 else O.layer_norm(x, 1e-6, wf, b.float().cpu())
+        want = xn.clone()
+        for j, r in enumerate(rows.tolist()):
+            if r >= n_txt:
+                want[j] = O.apply_rotary_emb(xn[j][None, :, None, :], cos[r - n_txt][None], sin[r - n_txt][None])[0, :, 0]
+        got = qkv[0, rows.to(DEV), col0 : col0 + inner].view(-1, H, hd)
+        assert_parity(got, want, what=f"qk_norm_rope {name} rows")
+
+
+def test_flux_blocks_full_size_against_oracle(hdit):
+    """configs[2] at its real size -- B1, 512 text + 4096 image tokens (64 x 64 grid), D 3072, 24 heads of 128 --
+    one double-stream block and one single-stream block, each against the fp32 oracle (about 1.3 TFLOP of CPU
+    work apiece).  At this width the planner picks tile shapes and two-phase launches the small-width block tests
+    never see."""
+    import oracle
+    from hetu_dit_amd import blocks, synthetic
+    from hetu_dit_amd.runtime_state import get_runtime_state
+    from tests.util import oracle_params
+
+    cfg = synthetic.CONFIGS["flux_1024"]
+    B, Ni, Nt, D, H, hd = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"], cfg["heads"], cfg["head_dim"]
+    ids = synthetic.flux_ids(Nt, *cfg["grid"])
+    cos, sin = synthetic.rope_table(ids, (16, 56, 56))
+    rope = (cos.to(DEV), sin.to(DEV))
+    x, e, t = synthetic.randn_bf16((B, Ni, D), 23), synthetic.randn_bf16((B, Nt, D), 24), synthetic.randn_bf16((B, D), 25)
+    print("flux double block full size", flush=True)
+    dbl = synthetic.init_module_(blocks.FluxTransformerBlock(D, H, hd), 21)
+    p_dbl = oracle_params(dbl)
+    dbl = dbl.to(DEV)
+    enc, hid = dbl(hidden_states=x.to(DEV), encoder_hidden_states=e.to(DEV), temb=t.to(DEV), image_rotary_emb=rope)
+    torch.cuda.synchronize()
+    o_enc, o_hid = oracle.flux_double_block(p_dbl, x.float(), e.float(), t.float(), (cos, sin), H)
+    assert_parity(hid, o_hid, what="flux double hidden (full size)")
+    assert_parity(enc, o_enc, what="flux double encoder (full size)")
+    # the same block through its one-call entry point: same launches, same bits
+    enc2, hid2 = hdit.ops.block_flux_double(dbl, x.to(DEV), e.to(DEV), t.to(DEV), rope)
+    torch.cuda.synchronize()
+    assert torch.equal(hid2, hid) and torch.equal(enc2, enc)
+    del dbl, p_dbl, o_enc, o_hid
+    print("flux single block full size", flush=True)
+    sgl = synthetic.init_module_(blocks.FluxSingleTransformerBlock(D, H, hd), 22)
+    p_sgl = oracle_params(sgl)
+    sgl = sgl.to(DEV)
+    get_runtime_state().max_condition_sequence_length = Nt
+    joint = torch.cat([e, x], dim=1)
+    out = sgl(hidden_states=joint.to(DEV), temb=t.to(DEV), image_rotary_emb=rope)
+    torch.cuda.synchronize()
+    o_out = oracle.flux_single_block(p_sgl, joint.float(), t.float(), (cos, sin), H, n_text=Nt)
+    assert_parity(out, o_out, what="flux single (full size)")
+    out2 = hdit.ops.block_flux_single(sgl, joint.to(DEV), t.to(DEV), rope)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out)
+
+
 # (batch, heads, image tokens, text tokens, head dim): configs[1], [2], [4]
 ATTN_CASES = [(2, 24, 4096, 333, 64), (1, 24, 4096, 512, 128), (1, 48, 17550, 226, 64)]
 

@@ -295,18 +295,20 @@ def test_attention_fp8_masked_last_tile_tail_columns(hdit, hd, skv):
     """Fixed regression case for the distance between the last PV MFMA and the first read of its result: with a
     masked last key tile in front of the output code, output columns 58, 59, 62, 63 of query rows 32-63 once came
     out wrong.  V is constant per column with e4m3-exact values, so every output element is that constant up to
-    the rounding of the probabilities (2^-8 relative): any wrong register shows as an O(1) error."""
+    the e4m3 rounding of the probabilities (at most 2^-4 relative, averaged over few keys here): a wrong
+    register shows as an O(1) error."""
     print(f"attention fp8 tail columns hd={hd} skv={skv}", flush=True)
     B, H, sq = 1, 2, 128
     q, k = rnd(B, sq, H, hd, seed=31), rnd(B, skv, H, hd, seed=32)
-    col = torch.tensor([1.0, -0.5, 2.0, 0.75, -1.5, 0.25, 3.0, -2.0]).repeat(hd // 8)
+    # absmax 1 maps to 448 = 1.75 * 2^8, so +-1, +-0.5, +-0.25 stay exact in e4m3
+    col = torch.tensor([1.0, -0.5, 0.25, -1.0, 0.5, -0.25, 1.0, -1.0]).repeat(hd // 8)
     v = col.view(1, 1, 1, hd).expand(B, skv, H, hd).contiguous()
     (o,) = hdit.ops.attention([g(q)], [g(k)], [g(v)], fp8=True)
     torch.cuda.synchronize()
-    err = (o.float().cpu() - col.view(1, 1, 1, hd)).abs() / col.abs().view(1, 1, 1, hd)
-    assert err.max().item() < 2.0 ** -6, f"worst at {divmod(int(err.argmax()), hd)}: {err.max().item():.3e}"
+    err = (o.float().cpu() - col.view(1, 1, 1, hd)).abs()
+    assert err.max().item() <= 2.0 ** -4, f"worst at {divmod(int(err.argmax()), hd)}: {err.max().item():.3e}"
     tail = err[:, 32:64][..., [hd - 6, hd - 5, hd - 2, hd - 1]]
-    assert tail.max().item() < 2.0 ** -6
+    assert tail.max().item() <= 2.0 ** -4
 
 
 def test_attention_fp8_two_segments(hdit):

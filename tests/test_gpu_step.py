@@ -157,7 +157,7 @@ def test_conv2d_wrapper_patch_convolution(hdit):
     from hetu_dit_amd import synthetic
     from hetu_dit_amd.layers.conv import hetuDiTConv2dWrapper
 
-    for (cin, cout, p, H, W, bias) in [(16, 256, 2, 32, 48, True), (4, 64, 4, 16, 16, False), (8, 128, 1, 6, 10, True)]:
+    for (cin, cout, p, H, W, bias) in [(16, 256, 2, 32, 48, True), (4, 64, 4, 16, 16, False), (64, 128, 1, 6, 10, True)]:
         print(f"conv wrapper {cin} {cout} {p} {H} {W} {bias}", flush=True)
         conv = nn.Conv2d(cin, cout, p, stride=p, bias=bias)
         synthetic.init_module_(conv, 21)
