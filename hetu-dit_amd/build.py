@@ -20,6 +20,14 @@ HIPCC_FLAGS = [
 ]
 
 
+# Per-file additions.  attention_bf16.hip: its pipelined kernel runs one wave per SIMD with 512 registers, where
+# the compiler would otherwise keep every MFMA accumulator in the AGPR half -- and the softmax (VALU) cannot read
+# those without a copy per score.  In the VGPR form the allocator decides per value.
+EXTRA_FLAGS = {
+    "attention_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
 def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
@@ -30,7 +38,7 @@ def build_library(verbose: bool = False) -> str:
     procs = []
     for src in sources():
         obj = os.path.join(CSRC, os.path.basename(src)[:-4] + ".o")
-        cmd = [hipcc] + HIPCC_FLAGS + ["-c", src, "-o", obj]
+        cmd = [hipcc] + HIPCC_FLAGS + EXTRA_FLAGS.get(os.path.basename(src), []) + ["-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))

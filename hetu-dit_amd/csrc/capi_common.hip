@@ -2,6 +2,8 @@
 // error string, launch check.
 #include <string.h>
 
+#include <atomic>
+
 #include "hdit_common.h"
 
 namespace {
@@ -20,6 +22,18 @@ int check_launch(const char* what) {
   snprintf(buf, sizeof(buf), "%s: %s", what, hipGetErrorString(e));
   set_error(buf);
   return HDIT_ELAUNCH;
+}
+// Compute units of the current device (cached for the first device asked about; 0 if the query fails).
+int num_cus() {
+  static std::atomic<int> cached{0};
+  int n = cached.load(std::memory_order_acquire);
+  if (n == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+      return 0;
+    cached.store(n, std::memory_order_release);
+  }
+  return n;
 }
 }  // namespace hdit_host
 

@@ -70,4 +70,5 @@ __device__ __forceinline__ float silu_f(float x) {
 namespace hdit_host {
 void set_error(const char* msg);
 int check_launch(const char* what);
+int num_cus();
 }  // namespace hdit_host

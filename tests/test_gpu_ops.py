@@ -171,6 +171,28 @@ def test_attention_large_logits_and_scale(hdit):
     assert_parity(o, want, what="attention large logits")
 
 
+@pytest.mark.parametrize("gain", [4.0, 40.0, 400.0])
+@pytest.mark.parametrize("skv", [256, 300, 1000])
+def test_attention_logits_outgrow_the_first_tile(hdit, gain, skv):
+    """The d = 64 kernel fixes its softmax reference after the first keys and starts over with a tracked reference
+    if a row sum overflows.  Keys placed behind the first tile get logits far above everything the first tile
+    holds: a few tens of nats (inside the fixed reference's range), hundreds (overflow, second pass), for every
+    row or only for some, in a full or a masked last tile."""
+    print(f"attention outgrow gain={gain} skv={skv}", flush=True)
+    B, H, hd, sq = 1, 2, 64, 320
+    q, k, v = rnd(B, sq, H, hd, seed=41), rnd(B, skv, H, hd, seed=42), rnd(B, skv, H, hd, seed=43)
+    # keys 130.. of head 0 point along the queries of rows 0..63 (only those rows see the huge logits);
+    # the last key of head 1 points along every query's mean direction
+    k[:, 130:140, 0] = gain * q[:, 0:10, 0] / 8.0
+    k[:, skv - 1, 1] = gain * q[:, :, 1].mean(1) * 2.0
+    q, k = bf16_round(q), bf16_round(k)
+    (o,) = hdit.ops.attention([g(q)], [g(k)], [g(v)])
+    torch.cuda.synchronize()
+    want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
+    for h in range(H):
+        assert_parity(o[:, :, h], want[:, :, h], what=f"attention, logits outgrow the first tile, head {h}")
+
+
 @pytest.mark.parametrize("dim", [64, 1536, 3072, 4096 + 8])
 def test_layernorm_modulate(hdit, dim):
     B, T = 2, 37
