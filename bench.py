@@ -74,7 +74,7 @@ def randomize_(module, device, seed=0):
 
 
 WORKLOADS = ("sd3_1024", "sd3_1024_transformer", "sd3_pipefusion", "sd3_pipefusion_b1", "flux_1024", "cogvideox_5b", "sd3_1024_fp8",
-             "cogvideox_5b_fp8")
+             "cogvideox_5b_fp8", "flux_1024_step", "cogvideox_5b_step")
 
 
 def make_workload(name, dev):
@@ -122,6 +122,35 @@ def make_workload(name, dev):
         step.multi_stream = "eager, the two batch elements as independent block chains on two streams"
         step.set_single_stream = lambda on: setattr(model._runner, "batch_streams", 1 if on else 2)
         return step, desc, gemm, attn, cfg["layers"], "attn_fwd_kernel<64>"
+    if name in ("flux_1024_step", "cogvideox_5b_step"):
+        # the whole block stacks of the two models at the shapes of configs[2] / configs[4]: 19 double + 38 single
+        # Flux blocks (the 1024^2 step BASELINE.md quotes 0.84 s for on the reference's hardware), 42 CogVideoX-5B
+        # blocks; every block one call of its whole-block entry point
+        cfg = synthetic.CONFIGS[name[:-5]]
+        B, Ni, Nt, D = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"]
+        S = Ni + Nt
+        x, e = rnd(B, Ni, D), rnd(B, Nt, D)
+        if name == "flux_1024_step":
+            L2, L1 = 19, 38
+            with torch.device(dev):
+                stack = transformer.FluxTransformerBlocks(L2, L1, D, cfg["heads"], cfg["head_dim"])
+            randomize_(stack, dev)
+            get_runtime_state().max_condition_sequence_length = Nt
+            cos, sin = synthetic.rope_table(synthetic.flux_ids(Nt, *cfg["grid"]), (16, 56, 56))
+            rope, t = (cos.to(dev), sin.to(dev)), rnd(B, D)
+            gemm = 24.0 * S * D * D * B * (L2 + L1)
+            attn = 4.0 * S * S * D * B * (L2 + L1)
+            desc = ("configs[2] as a whole step: Flux-shape, 19 double-stream + 38 single-stream blocks, B1, 4096 image + 512 "
+                    "text tokens, D3072, 24x128 heads")
+            return (lambda: stack(x, e, t, rope)[0]), desc, gemm, attn, L2 + L1, "attn_fwd_pipe_kernel<128>"
+        L = 42
+        with torch.device(dev):
+            stack = transformer.CogVideoXTransformerBlocks(L, D, cfg["heads"], cfg["head_dim"], cfg["temb_dim"])
+        randomize_(stack, dev)
+        cos, sin = synthetic.rope_table(synthetic.cogvideox_positions(*cfg["grid"]), (16, 24, 24))
+        rope, t = (cos.to(dev), sin.to(dev)), rnd(B, cfg["temb_dim"])
+        desc = "configs[4] as a whole step: CogVideoX-5B-shape, 42 blocks, B1, 226 text + 17550 video tokens, D3072, 48x64 heads"
+        return (lambda: stack(x, e, t, rope)[0]), desc, 24.0 * S * D * D * B * L, 4.0 * S * S * D * B * L, L, "attn_fwd_kernel<64>"
     cfg = synthetic.CONFIGS[name]
     B, Ni, Nt, D = cfg["batch"], cfg["n_img"], cfg["n_txt"], cfg["dim"]
     S = Ni + Nt
@@ -185,7 +214,7 @@ def make_workload(name, dev):
         gemm = 24.0 * S * D * D * B * 2
         attn = 4.0 * S * S * D * B * 2
         desc = "configs[2]: Flux-shape, one double-stream + one single-stream block, B1, 4096 image + 512 text tokens, D3072, 24x128 heads"
-        return (lambda: stack(x, e, t, rope)[0]), desc, gemm, attn, 2, "attn_fwd_kernel<128>"
+        return (lambda: stack(x, e, t, rope)[0]), desc, gemm, attn, 2, "attn_fwd_pipe_kernel<128>"
     with torch.device(dev):
         stack = transformer.CogVideoXTransformerBlocks(1, D, cfg["heads"], cfg["head_dim"], cfg["temb_dim"])
     randomize_(stack, dev)

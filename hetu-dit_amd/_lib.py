@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("HDIT_LIBRARY") or os.path.join(HERE, "libhdit.so")
 HDIT_GEMM_MAX_PROBLEMS = 16
 EPI_BIAS, EPI_BIAS_GELU, EPI_GATE_RESIDUAL = 0, 1, 2
 EPI_RESID_F32, EPI_OUT_F32 = 0x10, 0x20
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class GemmProblem(C.Structure):
@@ -138,14 +138,17 @@ class FluxDoubleBlockArgs(C.Structure):
                                                   "temb", "rope_cos", "rope_sin", "hidden_out", "encoder_out", "workspace")
                 + [("workspace_bytes", C.c_int64), ("qk_norm_eps", C.c_float)]
                 + _ints("qk_norm_kind", "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "hidden_f32",
-                        "encoder_f32", "out_f32"))
+                        "encoder_f32", "out_f32", "kv_rows", "kv_row0")
+                + _ptrs("modulation_img", "modulation_txt", "kv_buffer"))
 
 
 class FluxSingleBlockArgs(C.Structure):
     _fields_ = (_ptrs("norm_w", "norm_b", "qkv_w", "qkv_b", "proj_mlp_w", "proj_mlp_b", "proj_out_w", "proj_out_b", "norm_q_w",
                       "norm_k_w", "hidden", "temb", "rope_cos", "rope_sin", "hidden_out", "workspace")
                 + [("workspace_bytes", C.c_int64), ("qk_norm_eps", C.c_float)]
-                + _ints("qk_norm_kind", "batch", "seq", "dim", "heads", "ff_dim", "temb_dim", "hidden_f32", "out_f32"))
+                + _ints("qk_norm_kind", "batch", "seq", "dim", "heads", "ff_dim", "temb_dim", "hidden_f32", "out_f32",
+                        "n_txt", "kv_rows", "kv_row0", "pad_")
+                + _ptrs("modulation", "kv_buffer"))
 
 
 class CogVideoXBlockArgs(C.Structure):
@@ -155,7 +158,8 @@ class CogVideoXBlockArgs(C.Structure):
                       "hidden_out", "encoder_out", "workspace")
                 + [("workspace_bytes", C.c_int64), ("norm_eps", C.c_float), ("qk_norm_eps", C.c_float)]
                 + _ints("qk_norm_kind", "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "hidden_f32",
-                        "encoder_f32", "out_f32", "fp8_attention"))
+                        "encoder_f32", "out_f32", "fp8_attention")
+                + _ptrs("modulation1", "modulation2"))
 
 
 # name -> (restype, argtypes); every symbol include/hdit.h declares

@@ -352,7 +352,7 @@ FluxDoubleWs carve(const hdit_flux_double_block_args* a, void* base) {
   FluxDoubleWs w;
   w.emb_img = (float*)c.take(B * 6 * D * 4), w.emb_txt = (float*)c.take(B * 6 * D * 4);
   w.n_img = c.take(B * Ni * D * 2), w.n_txt = c.take(B * Nt * D * 2);
-  w.qkv_img = c.take(B * Ni * 3 * D * 2), w.qkv_txt = c.take(B * Nt * 3 * D * 2);
+  w.qkv_img = c.take(B * Ni * (a->kv_buffer ? 1 : 3) * D * 2), w.qkv_txt = c.take(B * Nt * 3 * D * 2);  // buffer given: q only
   w.o_img = c.take(B * Ni * D * 2), w.o_txt = c.take(B * Nt * D * 2);
   w.x1_img = (float*)c.take(B * Ni * D * 4), w.x1_txt = (float*)c.take(B * Nt * D * 4);
   w.h_img = c.take(B * Ni * F * 2), w.h_txt = c.take(B * Nt * F * 2);
@@ -369,12 +369,17 @@ int validate(const hdit_flux_double_block_args* a) {
       !w.to_add_out_w || !w.ff_in_w || !w.ff_out_w || !w.ff_context_in_w || !w.ff_context_out_w)
     return HDIT_EINVAL;
   if ((a->rope_cos == nullptr) != (a->rope_sin == nullptr)) return HDIT_EINVAL;
+  if (a->kv_buffer) {
+    if ((((uintptr_t)a->kv_buffer) & 15) || a->kv_rows < a->n_img || a->kv_row0 < 0 || a->kv_row0 + a->n_img > a->kv_rows)
+      return HDIT_EINVAL;
+    if (a->batch + 2 > HDIT_GEMM_MAX_PROBLEMS) return HDIT_EUNSUPPORTED;
+  }
   return HDIT_OK;
 }
 
 struct FluxSingleWs {
   float* emb;
-  unsigned char *n, *qkv, *cat;
+  unsigned char *n, *qkv, *kv_txt, *cat;
   int64_t bytes;
 };
 FluxSingleWs carve(const hdit_flux_single_block_args* a, void* base) {
@@ -383,7 +388,9 @@ FluxSingleWs carve(const hdit_flux_single_block_args* a, void* base) {
   FluxSingleWs w;
   w.emb = (float*)c.take(B * 3 * D * 4);
   w.n = c.take(B * S * D * 2);
-  w.qkv = c.take(B * S * 3 * D * 2);
+  // buffer given: q of all rows [B, S, D], then the text rows' k | v [B, n_txt, 2 D]
+  w.qkv = c.take(a->kv_buffer ? B * S * D * 2 : B * S * 3 * D * 2);
+  w.kv_txt = c.take(a->kv_buffer ? B * (int64_t)a->n_txt * 2 * D * 2 : 0);
   w.cat = c.take(B * S * (D + F) * 2);
   w.bytes = c.off;
   return w;
@@ -395,6 +402,12 @@ int validate(const hdit_flux_single_block_args* a) {
   if (!a->hidden || !a->temb || !a->hidden_out || !a->norm_w || !a->norm_b || !a->qkv_w || !a->proj_mlp_w || !a->proj_out_w)
     return HDIT_EINVAL;
   if ((a->rope_cos == nullptr) != (a->rope_sin == nullptr)) return HDIT_EINVAL;
+  if (a->kv_buffer) {
+    const int n_img = a->seq - a->n_txt;
+    if ((((uintptr_t)a->kv_buffer) & 15) || a->n_txt < 0 || n_img <= 0) return HDIT_EINVAL;
+    if (a->kv_rows < n_img || a->kv_row0 < 0 || a->kv_row0 + n_img > a->kv_rows) return HDIT_EINVAL;
+    if (2 * a->batch + 2 > HDIT_GEMM_MAX_PROBLEMS) return HDIT_EUNSUPPORTED;
+  }
   return HDIT_OK;
 }
 
@@ -468,34 +481,58 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_flux_double(con
   const int B = a->batch, Ni = a->n_img, Nt = a->n_txt, D = a->dim, F = a->ff_dim, H = a->heads, hd = D / H;
   const float eps = 1e-6f;
   const int64_t md = 6 * (int64_t)D;
-  if ((rc = hdit_adaln_gemv(a->temb, w.norm1_w, w.norm1_b, ws.emb_img, B, 6 * D, a->temb_dim, stream))) return rc;
-  if ((rc = hdit_adaln_gemv(a->temb, w.norm1_context_w, w.norm1_context_b, ws.emb_txt, B, 6 * D, a->temb_dim, stream))) return rc;
-  const float *ei = ws.emb_img, *et = ws.emb_txt;  // shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp
+  const float *ei = a->modulation_img, *et = a->modulation_txt;  // shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp
+  if (!ei) {
+    if ((rc = hdit_adaln_gemv(a->temb, w.norm1_w, w.norm1_b, ws.emb_img, B, 6 * D, a->temb_dim, stream))) return rc;
+    ei = ws.emb_img;
+  }
+  if (!et) {
+    if ((rc = hdit_adaln_gemv(a->temb, w.norm1_context_w, w.norm1_context_b, ws.emb_txt, B, 6 * D, a->temb_dim, stream))) return rc;
+    et = ws.emb_txt;
+  }
   hdit_ln_job jobs[2];
   ln_job(jobs[0], a->hidden, a->hidden_f32, ws.n_img, (int64_t)Ni * D, ei, ei + D, md, B, Ni, D);
   ln_job(jobs[1], a->encoder, a->encoder_f32, ws.n_txt, (int64_t)Nt * D, et, et + D, md, B, Nt, D);
   if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, nullptr, nullptr, eps, stream))) return rc;
-  hdit_gemm_problem probs[4];
-  probs[0] = problem(ws.n_img, D, w.qkv_w, w.qkv_b, ws.qkv_img, 3 * D, B * Ni, 3 * D, D, HDIT_EPI_BIAS);
-  probs[1] = problem(ws.n_txt, D, w.add_qkv_w, w.add_qkv_b, ws.qkv_txt, 3 * D, B * Nt, 3 * D, D, HDIT_EPI_BIAS);
-  if ((rc = hdit_gemm_bf16(probs, 2, stream))) return rc;
+  hdit_gemm_problem probs[HDIT_GEMM_MAX_PROBLEMS];
+  const int64_t ld3 = 3 * (int64_t)D, ld2 = 2 * (int64_t)D;
+  // image q | k | v: one packed tensor, or (K/V buffer given) q alone and k | v straight into this call's rows of
+  // the buffer, one problem per batch element (the destinations differ in batch stride)
+  unsigned char *q_img = ws.qkv_img, *k_img, *v_img, *k_new;
+  int64_t ld_q, ld_kv, kv_batch_rows;
+  int kv_len, np = 0;
+  if (a->kv_buffer) {
+    unsigned char* buf = (unsigned char*)a->kv_buffer;
+    const unsigned char* wkv = (const unsigned char*)w.qkv_w + (int64_t)D * D * 2;
+    const unsigned char* bkv = w.qkv_b ? (const unsigned char*)w.qkv_b + (int64_t)D * 2 : nullptr;
+    probs[np++] = problem(ws.n_img, D, w.qkv_w, w.qkv_b, q_img, D, B * Ni, D, D, HDIT_EPI_BIAS);
+    for (int b = 0; b < B; b++)
+      probs[np++] = problem(ws.n_img + (int64_t)b * Ni * D * 2, D, wkv, bkv,
+                            buf + ((int64_t)b * a->kv_rows + a->kv_row0) * ld2 * 2, ld2, Ni, 2 * D, D, HDIT_EPI_BIAS);
+    k_img = buf, v_img = buf + (int64_t)D * 2, k_new = buf + (int64_t)a->kv_row0 * ld2 * 2;
+    ld_q = D, ld_kv = ld2, kv_batch_rows = a->kv_rows, kv_len = a->kv_rows;
+  } else {
+    probs[np++] = problem(ws.n_img, D, w.qkv_w, w.qkv_b, ws.qkv_img, 3 * D, B * Ni, 3 * D, D, HDIT_EPI_BIAS);
+    k_img = ws.qkv_img + (int64_t)D * 2, v_img = ws.qkv_img + (int64_t)2 * D * 2, k_new = k_img;
+    ld_q = ld3, ld_kv = ld3, kv_batch_rows = Ni, kv_len = Ni;
+  }
+  probs[np++] = problem(ws.n_txt, D, w.add_qkv_w, w.add_qkv_b, ws.qkv_txt, 3 * D, B * Nt, 3 * D, D, HDIT_EPI_BIAS);
+  if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
   // per-head RMSNorm on q, k of both streams, then the rotation of the joint [text, image] rows
-  const int64_t ld3 = 3 * (int64_t)D;
-  unsigned char *q_img = ws.qkv_img, *k_img = ws.qkv_img + (int64_t)D * 2, *v_img = ws.qkv_img + (int64_t)2 * D * 2;
   unsigned char *q_txt = ws.qkv_txt, *k_txt = ws.qkv_txt + (int64_t)D * 2, *v_txt = ws.qkv_txt + (int64_t)2 * D * 2;
   const float* cos_i = a->rope_cos ? a->rope_cos + (int64_t)Nt * hd : nullptr;
   const float* sin_i = a->rope_sin ? a->rope_sin + (int64_t)Nt * hd : nullptr;
   hdit_qknorm_job qj[4];
   qk_job(qj[0], q_txt, Nt, ld3, hd, a->norm_added_q_w, nullptr, a->rope_cos, a->rope_sin, Nt, 0, Nt, a->qk_norm_kind);
   qk_job(qj[1], k_txt, Nt, ld3, hd, a->norm_added_k_w, nullptr, a->rope_cos, a->rope_sin, Nt, 0, Nt, a->qk_norm_kind);
-  qk_job(qj[2], q_img, Ni, ld3, hd, a->norm_q_w, nullptr, cos_i, sin_i, Ni, 0, Ni, a->qk_norm_kind);
-  qk_job(qj[3], k_img, Ni, ld3, hd, a->norm_k_w, nullptr, cos_i, sin_i, Ni, 0, Ni, a->qk_norm_kind);
+  qk_job(qj[2], q_img, Ni, ld_q, hd, a->norm_q_w, nullptr, cos_i, sin_i, Ni, 0, Ni, a->qk_norm_kind);
+  qk_job(qj[3], k_new, kv_batch_rows, ld_kv, hd, a->norm_k_w, nullptr, cos_i, sin_i, Ni, 0, Ni, a->qk_norm_kind);
   if ((rc = hdit_qk_norm_rope(qj, 4, B, H, hd, a->qk_norm_eps, stream))) return rc;
   hdit_attn_args at;
   memset(&at, 0, sizeof(at));
-  seg(at.q[0], q_txt, Nt, ld3, hd, Nt), seg(at.q[1], q_img, Ni, ld3, hd, Ni);
-  seg(at.k[0], k_txt, Nt, ld3, hd, Nt), seg(at.k[1], k_img, Ni, ld3, hd, Ni);
-  seg(at.v[0], v_txt, Nt, ld3, hd, Nt), seg(at.v[1], v_img, Ni, ld3, hd, Ni);
+  seg(at.q[0], q_txt, Nt, ld3, hd, Nt), seg(at.q[1], q_img, Ni, ld_q, hd, Ni);
+  seg(at.k[0], k_txt, Nt, ld3, hd, Nt), seg(at.k[1], k_img, kv_batch_rows, ld_kv, hd, kv_len);
+  seg(at.v[0], v_txt, Nt, ld3, hd, Nt), seg(at.v[1], v_img, kv_batch_rows, ld_kv, hd, kv_len);
   seg(at.o[0], ws.o_txt, Nt, D, hd, Nt), seg(at.o[1], ws.o_img, Ni, D, hd, Ni);
   at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
   if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
@@ -530,28 +567,62 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_flux_single(con
   if ((rc = check_workspace(a, ws.bytes))) return rc;
   const int B = a->batch, S = a->seq, D = a->dim, F = a->ff_dim, H = a->heads, hd = D / H;
   const int64_t md = 3 * (int64_t)D, ldc = (int64_t)D + F, ld3 = 3 * (int64_t)D;
-  if ((rc = hdit_adaln_gemv(a->temb, a->norm_w, a->norm_b, ws.emb, B, 3 * D, a->temb_dim, stream))) return rc;
+  const float* emb = a->modulation;  // shift, scale, gate
+  if (!emb) {
+    if ((rc = hdit_adaln_gemv(a->temb, a->norm_w, a->norm_b, ws.emb, B, 3 * D, a->temb_dim, stream))) return rc;
+    emb = ws.emb;
+  }
   hdit_ln_job job;
-  ln_job(job, a->hidden, a->hidden_f32, ws.n, (int64_t)S * D, ws.emb, ws.emb + D, md, B, S, D);  // shift, scale, gate
+  ln_job(job, a->hidden, a->hidden_f32, ws.n, (int64_t)S * D, emb, emb + D, md, B, S, D);
   if ((rc = hdit_layernorm_modulate_jobs(&job, 1, D, nullptr, nullptr, 1e-6f, stream))) return rc;
   // q|k|v and the MLP-in projection share their input: one launch; GELU(MLP) lands beside the attention output
-  hdit_gemm_problem probs[2];
-  probs[0] = problem(ws.n, D, a->qkv_w, a->qkv_b, ws.qkv, ld3, B * S, 3 * D, D, HDIT_EPI_BIAS);
-  probs[1] = problem(ws.n, D, a->proj_mlp_w, a->proj_mlp_b, ws.cat + (int64_t)D * 2, ldc, B * S, F, D, HDIT_EPI_BIAS_GELU);
-  if ((rc = hdit_gemm_bf16(probs, 2, stream))) return rc;
-  unsigned char *q = ws.qkv, *k = ws.qkv + (int64_t)D * 2, *v = ws.qkv + (int64_t)2 * D * 2;
-  hdit_qknorm_job qj[2];
-  qk_job(qj[0], q, S, ld3, hd, a->norm_q_w, nullptr, a->rope_cos, a->rope_sin, S, 0, S, a->qk_norm_kind);
-  qk_job(qj[1], k, S, ld3, hd, a->norm_k_w, nullptr, a->rope_cos, a->rope_sin, S, 0, S, a->qk_norm_kind);
-  if ((rc = hdit_qk_norm_rope(qj, 2, B, H, hd, a->qk_norm_eps, stream))) return rc;
+  hdit_gemm_problem probs[HDIT_GEMM_MAX_PROBLEMS];
+  hdit_qknorm_job qj[3];
   hdit_attn_args at;
   memset(&at, 0, sizeof(at));
-  seg(at.q[0], q, S, ld3, hd, S), seg(at.k[0], k, S, ld3, hd, S), seg(at.v[0], v, S, ld3, hd, S);
+  int np = 0, nj = 0;
+  if (a->kv_buffer) {
+    // patch mode: the queries of all rows in one [B, S, D] tensor, the text rows' k | v in a small tensor of their
+    // own, the image rows' k | v straight into this patch's rows of the layer's buffer (one problem per batch element
+    // and destination: the destinations differ in batch stride)
+    const int Nt = a->n_txt, Ni = S - Nt;
+    const int64_t ld2 = 2 * (int64_t)D;
+    unsigned char* buf = (unsigned char*)a->kv_buffer;
+    const unsigned char* wkv = (const unsigned char*)a->qkv_w + (int64_t)D * D * 2;
+    const unsigned char* bkv = a->qkv_b ? (const unsigned char*)a->qkv_b + (int64_t)D * 2 : nullptr;
+    probs[np++] = problem(ws.n, D, a->qkv_w, a->qkv_b, ws.qkv, D, B * S, D, D, HDIT_EPI_BIAS);
+    for (int b = 0; b < B; b++) {
+      const unsigned char* xb = ws.n + (int64_t)b * S * D * 2;
+      if (Nt > 0)
+        probs[np++] = problem(xb, D, wkv, bkv, ws.kv_txt + (int64_t)b * Nt * ld2 * 2, ld2, Nt, 2 * D, D, HDIT_EPI_BIAS);
+      probs[np++] = problem(xb + (int64_t)Nt * D * 2, D, wkv, bkv, buf + ((int64_t)b * a->kv_rows + a->kv_row0) * ld2 * 2, ld2,
+                            Ni, 2 * D, D, HDIT_EPI_BIAS);
+    }
+    const float* cos_i = a->rope_cos ? a->rope_cos + (int64_t)Nt * hd : nullptr;
+    const float* sin_i = a->rope_sin ? a->rope_sin + (int64_t)Nt * hd : nullptr;
+    qk_job(qj[nj++], ws.qkv, S, D, hd, a->norm_q_w, nullptr, a->rope_cos, a->rope_sin, S, 0, S, a->qk_norm_kind);
+    if (Nt > 0)
+      qk_job(qj[nj++], ws.kv_txt, Nt, ld2, hd, a->norm_k_w, nullptr, a->rope_cos, a->rope_sin, Nt, 0, Nt, a->qk_norm_kind);
+    qk_job(qj[nj++], buf + (int64_t)a->kv_row0 * ld2 * 2, a->kv_rows, ld2, hd, a->norm_k_w, nullptr, cos_i, sin_i, Ni, 0, Ni,
+           a->qk_norm_kind);
+    seg(at.q[0], ws.qkv, S, D, hd, S);
+    seg(at.k[0], ws.kv_txt, Nt, ld2, hd, Nt), seg(at.k[1], buf, a->kv_rows, ld2, hd, a->kv_rows);
+    seg(at.v[0], ws.kv_txt + (int64_t)D * 2, Nt, ld2, hd, Nt), seg(at.v[1], buf + (int64_t)D * 2, a->kv_rows, ld2, hd, a->kv_rows);
+  } else {
+    unsigned char *q = ws.qkv, *k = ws.qkv + (int64_t)D * 2, *v = ws.qkv + (int64_t)2 * D * 2;
+    probs[np++] = problem(ws.n, D, a->qkv_w, a->qkv_b, ws.qkv, ld3, B * S, 3 * D, D, HDIT_EPI_BIAS);
+    qk_job(qj[nj++], q, S, ld3, hd, a->norm_q_w, nullptr, a->rope_cos, a->rope_sin, S, 0, S, a->qk_norm_kind);
+    qk_job(qj[nj++], k, S, ld3, hd, a->norm_k_w, nullptr, a->rope_cos, a->rope_sin, S, 0, S, a->qk_norm_kind);
+    seg(at.q[0], q, S, ld3, hd, S), seg(at.k[0], k, S, ld3, hd, S), seg(at.v[0], v, S, ld3, hd, S);
+  }
+  probs[np++] = problem(ws.n, D, a->proj_mlp_w, a->proj_mlp_b, ws.cat + (int64_t)D * 2, ldc, B * S, F, D, HDIT_EPI_BIAS_GELU);
+  if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
+  if ((rc = hdit_qk_norm_rope(qj, nj, B, H, hd, a->qk_norm_eps, stream))) return rc;
   seg(at.o[0], ws.cat, S, ldc, hd, S);
   at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
   if ((rc = hdit_attn_fwd_bf16(&at, stream))) return rc;
   probs[0] = problem(ws.cat, ldc, a->proj_out_w, a->proj_out_b, a->hidden_out, D, B * S, D, D + F, 0);
-  gated(probs[0], a->hidden, a->hidden_f32, ws.emb + 2 * D, md, S, a->out_f32);
+  gated(probs[0], a->hidden, a->hidden_f32, emb + 2 * D, md, S, a->out_f32);
   return hdit_gemm_bf16(probs, 1, stream);
 }
 
@@ -569,10 +640,16 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_cogvideox(const
   const int sz_h = a->hidden_f32 ? 4 : 2, sz_e = a->encoder_f32 ? 4 : 2, sz_o = a->out_f32 ? 4 : 2;
   // norm1: chunks shift, scale, gate, enc_shift, enc_scale, enc_gate; one affine LayerNorm for both streams,
   // both results written into one joint [text, video] buffer
-  if ((rc = hdit_adaln_gemv(a->temb, a->norm1_w, a->norm1_b, ws.emb1, B, 6 * D, a->temb_dim, stream))) return rc;
-  if ((rc = hdit_adaln_gemv(a->temb, a->norm2_w, a->norm2_b, ws.emb2, B, 6 * D, a->temb_dim, stream))) return rc;
+  const float *e1 = a->modulation1, *e2 = a->modulation2;
+  if (!e1) {
+    if ((rc = hdit_adaln_gemv(a->temb, a->norm1_w, a->norm1_b, ws.emb1, B, 6 * D, a->temb_dim, stream))) return rc;
+    e1 = ws.emb1;
+  }
+  if (!e2) {
+    if ((rc = hdit_adaln_gemv(a->temb, a->norm2_w, a->norm2_b, ws.emb2, B, 6 * D, a->temb_dim, stream))) return rc;
+    e2 = ws.emb2;
+  }
   hdit_ln_job jobs[2];
-  const float* e1 = ws.emb1;
   ln_job(jobs[0], a->encoder, a->encoder_f32, ws.joint, (int64_t)S * D, e1 + 3 * D, e1 + 4 * D, md, B, Nt, D);
   ln_job(jobs[1], a->hidden, a->hidden_f32, ws.joint + (int64_t)Nt * D * 2, (int64_t)S * D, e1, e1 + D, md, B, N, D);
   if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, a->norm1_ln_w, a->norm1_ln_b, a->norm_eps, stream))) return rc;
@@ -607,12 +684,11 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_cogvideox(const
     }
     return hdit_gemm_bf16(probs, np, stream);
   };
-  if ((rc = gated_pair(ws.o, D, a->to_out_w, a->to_out_b, D, a->encoder, sz_e, a->hidden, sz_h, ws.emb1, ws.x1_e, 4, ws.x1_h, 4))) return rc;
-  const float* e2 = ws.emb2;
+  if ((rc = gated_pair(ws.o, D, a->to_out_w, a->to_out_b, D, a->encoder, sz_e, a->hidden, sz_h, e1, ws.x1_e, 4, ws.x1_h, 4))) return rc;
   ln_job(jobs[0], ws.x1_e, 1, ws.joint, (int64_t)S * D, e2 + 3 * D, e2 + 4 * D, md, B, Nt, D);
   ln_job(jobs[1], ws.x1_h, 1, ws.joint + (int64_t)Nt * D * 2, (int64_t)S * D, e2, e2 + D, md, B, N, D);
   if ((rc = hdit_layernorm_modulate_jobs(jobs, 2, D, a->norm2_ln_w, a->norm2_ln_b, a->norm_eps, stream))) return rc;
   probs[0] = problem(ws.joint, D, a->ff_in_w, a->ff_in_b, ws.h, F, B * S, F, D, HDIT_EPI_BIAS_GELU);
   if ((rc = hdit_gemm_bf16(probs, 1, stream))) return rc;
-  return gated_pair(ws.h, F, a->ff_out_w, a->ff_out_b, F, ws.x1_e, 4, ws.x1_h, 4, ws.emb2, a->encoder_out, sz_o, a->hidden_out, sz_o);
+  return gated_pair(ws.h, F, a->ff_out_w, a->ff_out_b, F, ws.x1_e, 4, ws.x1_h, 4, e2, a->encoder_out, sz_o, a->hidden_out, sz_o);
 }

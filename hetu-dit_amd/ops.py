@@ -479,8 +479,27 @@ def _fill_sd3_weights(w, block, ptr):
         setattr(w, prefix + "_out_b", ptr(ff.output_bias.data) if ff.has_output_bias else None)
 
 
-def block_flux_double(block, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None, out_dtype=bf16):
-    """One Flux double-stream block through ``hdit_block_flux_double``; returns ``(encoder, hidden)``."""
+def _kv_buffer_args(a, kv_buffer, kv_row0: int, batch: int, rows: int, dim: int, keep):
+    """``kv_buffer``: contiguous bf16 [batch, kv_rows, 2 dim] K|V buffer of the layer whose rows
+    ``[kv_row0, kv_row0 + rows)`` the call writes."""
+    if kv_buffer is None:
+        return
+    _need(kv_buffer, bf16, "kv_buffer")
+    if kv_buffer.dim() != 3 or tuple(kv_buffer.shape[::2]) != (batch, 2 * dim) or not kv_buffer.is_contiguous():
+        raise ValueError("kv_buffer must be a contiguous bf16 [batch, rows, 2 * dim] tensor")
+    if kv_row0 < 0 or kv_row0 + rows > kv_buffer.shape[1]:
+        raise ValueError("kv_row0 + rows exceeds the K/V buffer")
+    a.kv_buffer, a.kv_rows, a.kv_row0 = kv_buffer.data_ptr(), kv_buffer.shape[1], kv_row0
+    keep.append(kv_buffer)
+
+
+def block_flux_double(block, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None, out_dtype=bf16,
+                      kv_buffer=None, kv_row0: int = 0, modulation_img: Optional[int] = None,
+                      modulation_txt: Optional[int] = None):
+    """One Flux double-stream block through ``hdit_block_flux_double``; returns ``(encoder, hidden)``.
+    ``kv_buffer`` / ``kv_row0``: the image stream's K|V buffer of the layer and the first row this call writes
+    (a pipeline patch attends to all its rows).  ``modulation_*``: device addresses of precomputed f32
+    [batch, 6 dim] adaLN projections (the caller keeps their tensor alive)."""
     attn, m = block.attn, block.attn.module
     B, Ni, D = hidden_states.shape
     Nt = encoder_hidden_states.shape[1]
@@ -504,14 +523,19 @@ def block_flux_double(block, hidden_states, encoder_hidden_states, temb, image_r
     a.hidden_out, a.encoder_out, a.out_f32 = hidden_out.data_ptr(), encoder_out.data_ptr(), int(out_dtype == torch.float32)
     a.batch, a.n_img, a.n_txt, a.dim, a.heads = B, Ni, Nt, D, attn.heads_per_device
     a.ff_dim, a.temb_dim = block.ff.module.net[0].proj.weight.shape[0], temb.shape[1]
+    a.modulation_img, a.modulation_txt = modulation_img, modulation_txt
+    _kv_buffer_args(a, kv_buffer, kv_row0, B, Ni, D, ptr.keep)
     lib = _lib.lib()
     _run_block(a, lib.hdit_block_flux_double_workspace_bytes, lib.hdit_block_flux_double, "hdit_block_flux_double",
                hidden_states.device, ptr.keep)
     return encoder_out, hidden_out
 
 
-def block_flux_single(block, hidden_states, temb, image_rotary_emb=None, out_dtype=bf16):
-    """One Flux single-stream block through ``hdit_block_flux_single`` on the joint [text, image] rows."""
+def block_flux_single(block, hidden_states, temb, image_rotary_emb=None, out_dtype=bf16, kv_buffer=None, kv_row0: int = 0,
+                      n_txt: int = 0, modulation: Optional[int] = None):
+    """One Flux single-stream block through ``hdit_block_flux_single`` on the joint [text, image] rows.
+    ``kv_buffer`` / ``kv_row0`` / ``n_txt``: the layer's K|V buffer for the image rows (the rows behind the first
+    ``n_txt``); ``modulation``: device address of the precomputed f32 [batch, 3 dim] adaLN projection."""
     attn, m = block.attn, block.attn.module
     B, S, D = hidden_states.shape
     _need(temb, bf16, "temb")
@@ -535,14 +559,19 @@ def block_flux_single(block, hidden_states, temb, image_rotary_emb=None, out_dty
     hidden_out = torch.empty(B, S, D, dtype=out_dtype, device=hidden_states.device)
     a.hidden, a.temb, a.hidden_out, a.out_f32 = ptr(hidden_states), ptr(temb.contiguous()), hidden_out.data_ptr(), int(out_dtype == torch.float32)
     a.batch, a.seq, a.dim, a.heads, a.ff_dim, a.temb_dim = B, S, D, attn.heads_per_device, block.mlp_hidden_dim, temb.shape[1]
+    a.modulation, a.n_txt = modulation, n_txt
+    _kv_buffer_args(a, kv_buffer, kv_row0, B, S - n_txt, D, ptr.keep)
     lib = _lib.lib()
     _run_block(a, lib.hdit_block_flux_single_workspace_bytes, lib.hdit_block_flux_single, "hdit_block_flux_single",
                hidden_states.device, ptr.keep)
     return hidden_out
 
 
-def block_cogvideox(block, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None, out_dtype=bf16):
-    """One CogVideoX block through ``hdit_block_cogvideox``; returns ``(hidden, encoder)`` like the block."""
+def block_cogvideox(block, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None, out_dtype=bf16,
+                    modulation1: Optional[int] = None, modulation2: Optional[int] = None):
+    """One CogVideoX block through ``hdit_block_cogvideox``; returns ``(hidden, encoder)`` like the block.
+    ``modulation1`` / ``modulation2``: device addresses of the precomputed f32 [batch, 6 dim] projections of
+    ``norm1`` / ``norm2``."""
     attn, m = block.attn1, block.attn1.module
     B, N, D = hidden_states.shape
     Nt = encoder_hidden_states.shape[1]
@@ -581,6 +610,7 @@ def block_cogvideox(block, hidden_states, encoder_hidden_states, temb, image_rot
     a.batch, a.n_img, a.n_txt, a.dim, a.heads = B, N, Nt, D, attn.heads_per_device
     a.ff_dim, a.temb_dim = ff.module.net[0].proj.weight.shape[0], temb.shape[1]
     a.fp8_attention = int(bool(getattr(attn, "fp8_attention", False)))
+    a.modulation1, a.modulation2 = modulation1, modulation2
     lib = _lib.lib()
     _run_block(a, lib.hdit_block_cogvideox_workspace_bytes, lib.hdit_block_cogvideox, "hdit_block_cogvideox",
                hidden_states.device, ptr.keep)

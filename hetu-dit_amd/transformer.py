@@ -303,7 +303,21 @@ class SD3TransformerBlocks(nn.Module):
         return hidden
 
 
+def _modulation_address(mods, module) -> int:
+    """Device address of ``module``'s [batch, rows] block inside the regrouped stack modulation."""
+    flat, offsets = mods
+    return flat.data_ptr() + 4 * offsets[module]
+
+
 class FluxTransformerBlocks(nn.Module):
+    """The double- and single-stream blocks of the Flux transformer with the reference's loop
+    (``transformer_flux.py:133-201``).  ``use_block_entry_points``: every block is one call of
+    ``hdit_block_flux_double`` / ``hdit_block_flux_single`` -- the launches of the Python blocks on the same
+    operands, so the same bits -- fed from the stack's one adaLN GEMV, its image K|V written straight into the
+    layer's buffer from the cache manager (a fresh one on a full pass, this patch's rows of the persistent one in
+    patch mode).  With a per-launch timer installed, or an fp8 attention switch set on a block, the blocks run
+    kernel by kernel."""
+
     def __init__(self, num_layers: int = 19, num_single_layers: int = 38, dim: int = 3072,
                  num_attention_heads: int = 24, attention_head_dim: int = 128):
         super().__init__()
@@ -315,9 +329,40 @@ class FluxTransformerBlocks(nn.Module):
         )
         self.modulation = StackModulation(list(self.transformer_blocks) + list(self.single_transformer_blocks))
         use_fp32_residual_stream(list(self.transformer_blocks) + list(self.single_transformer_blocks))
+        self.use_block_entry_points = True
+
+    def _entry_points_usable(self) -> bool:
+        if not self.use_block_entry_points or ops.timer_installed():
+            return False
+        blocks = list(self.transformer_blocks) + list(self.single_transformer_blocks)
+        return not any(getattr(b.attn, "fp8_attention", False) for b in blocks)
 
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb):
+        if not self._entry_points_usable():
+            return self._forward_per_kernel(hidden_states, encoder_hidden_states, temb, image_rotary_emb)
+        temb = temb.contiguous()
+        hidden_states, encoder_hidden_states = hidden_states.contiguous(), encoder_hidden_states.contiguous()
+        mods = self.modulation.precompute_by_module(temb)
+        cm = get_cache_manager()
+        B, n_img, dim = hidden_states.shape
+        n_txt = encoder_hidden_states.shape[1]
+        dev = hidden_states.device
+        for block in self.transformer_blocks:
+            buf, start, _ = cm.kv_buffer(block.attn, B, n_img, dim, dev)
+            encoder_hidden_states, hidden_states = ops.block_flux_double(
+                block, hidden_states, encoder_hidden_states, temb, image_rotary_emb, out_dtype=block.stream_dtype,
+                kv_buffer=buf, kv_row0=start, modulation_img=_modulation_address(mods, block.norm1),
+                modulation_txt=_modulation_address(mods, block.norm1_context))
+        hidden_states = torch.cat([encoder_hidden_states, hidden_states], dim=1)
+        for block in self.single_transformer_blocks:
+            buf, start, _ = cm.kv_buffer(block.attn, B, n_img, dim, dev)
+            hidden_states = ops.block_flux_single(
+                block, hidden_states, temb, image_rotary_emb, out_dtype=block.stream_dtype, kv_buffer=buf, kv_row0=start,
+                n_txt=n_txt, modulation=_modulation_address(mods, block.norm))
+        return hidden_states[:, n_txt:, ...], hidden_states[:, :n_txt, ...]
+
+    def _forward_per_kernel(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb):
         self.modulation.precompute(temb)
         for block in self.transformer_blocks:
             encoder_hidden_states, hidden_states = block(
@@ -334,6 +379,10 @@ class FluxTransformerBlocks(nn.Module):
 
 
 class CogVideoXTransformerBlocks(nn.Module):
+    """The blocks of the CogVideoX transformer (``cogvideox_transformer_3d.py:99-127``); with
+    ``use_block_entry_points`` each block is one ``hdit_block_cogvideox`` call fed from the stack's adaLN GEMV
+    (same launches, same bits as the Python block)."""
+
     def __init__(self, num_layers: int = 42, dim: int = 3072, num_attention_heads: int = 48,
                  attention_head_dim: int = 64, time_embed_dim: int = 512):
         super().__init__()
@@ -342,9 +391,19 @@ class CogVideoXTransformerBlocks(nn.Module):
         )
         self.modulation = StackModulation(self.transformer_blocks)
         use_fp32_residual_stream(self.transformer_blocks)
+        self.use_block_entry_points = True
 
     @torch.no_grad()
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None) -> Tuple[torch.Tensor, torch.Tensor]:
+        if self.use_block_entry_points and not ops.timer_installed():
+            temb = temb.contiguous()
+            hidden_states, encoder_hidden_states = hidden_states.contiguous(), encoder_hidden_states.contiguous()
+            mods = self.modulation.precompute_by_module(temb)
+            for block in self.transformer_blocks:
+                hidden_states, encoder_hidden_states = ops.block_cogvideox(
+                    block, hidden_states, encoder_hidden_states, temb, image_rotary_emb, out_dtype=block.stream_dtype,
+                    modulation1=_modulation_address(mods, block.norm1), modulation2=_modulation_address(mods, block.norm2))
+            return hidden_states, encoder_hidden_states
         self.modulation.precompute(temb)
         for block in self.transformer_blocks:
             hidden_states, encoder_hidden_states = block(

@@ -386,9 +386,16 @@ int hdit_block_sd3(const hdit_sd3_block_args* args, void* stream);
  * layers/attention_processor.py:176-192,:284-305) plus the per-head norm weights
  * of q, k of both streams (bf16 [head_dim] or NULL; qk_norm_kind as in
  * hdit_qknorm_job, qk_norm_eps its eps).  rope_cos / rope_sin: f32 [n_txt + n_img,
- * head_dim] over the joint [text, image] rows, or both NULL.  No stale K/V buffer
- * at this level (the Python processor has it).  Tensor conventions and workspace
- * as for hdit_block_sd3. */
+ * head_dim] over this call's joint [text, image] rows, or both NULL.
+ * modulation_img / modulation_txt: optional precomputed linear(silu(temb)) of
+ * norm1 / norm1_context (f32 [batch, 6 dim]); NULL => computed here.  kv_buffer !=
+ * NULL: the image stream's K|V buffer of the layer, bf16 [batch, kv_rows, 2 dim]
+ * (core/resource_manager/cache_manager.py:88-149, the call at
+ * layers/attention_processor.py:908-922): this call projects its image rows' k | v
+ * into rows [kv_row0, kv_row0 + n_img) (k normed and rotated there, in place) and
+ * attention reads the text keys / values followed by all kv_rows -- a pipeline patch
+ * over the stale rows of the other patches; batch <= HDIT_GEMM_MAX_PROBLEMS - 2
+ * then.  Tensor conventions and workspace as for hdit_block_sd3. */
 typedef struct hdit_flux_double_block_args {
   hdit_sd3_block_weights w;
   const void *norm_q_w, *norm_k_w, *norm_added_q_w, *norm_added_k_w;
@@ -405,6 +412,10 @@ typedef struct hdit_flux_double_block_args {
   int32_t qk_norm_kind;
   int32_t batch, n_img, n_txt, dim, heads, ff_dim, temb_dim;
   int32_t hidden_f32, encoder_f32, out_f32;
+  int32_t kv_rows, kv_row0;
+  const float* modulation_img;
+  const float* modulation_txt;
+  void* kv_buffer;
 } hdit_flux_double_block_args;
 
 int64_t hdit_block_flux_double_workspace_bytes(const hdit_flux_double_block_args* args);
@@ -414,7 +425,13 @@ int hdit_block_flux_double(const hdit_flux_double_block_args* args, void* stream
  * transformer_flux.py:194-198) on the joint [text, image] sequence hidden
  * [batch, seq, dim]: adaLN-ZeroSingle (norm_w [3 dim, temb_dim]: shift, scale,
  * gate), q|k|v and proj_mlp in one launch, attention output and GELU(MLP) side by
- * side in one buffer, proj_out [dim, dim + ff_dim] with the gated residual. */
+ * side in one buffer, proj_out [dim, dim + ff_dim] with the gated residual.
+ * modulation: optional precomputed linear(silu(temb)) (f32 [batch, 3 dim]).
+ * kv_buffer != NULL (patch mode, layers/attention_processor.py:908-922): the first
+ * n_txt rows of the sequence are text, the other seq - n_txt rows the image rows
+ * of this pipeline patch; their k | v go into rows [kv_row0, kv_row0 + seq - n_txt)
+ * of the layer's buffer bf16 [batch, kv_rows, 2 dim] and attention reads the text
+ * keys / values followed by all kv_rows; 2 batch + 2 <= HDIT_GEMM_MAX_PROBLEMS. */
 typedef struct hdit_flux_single_block_args {
   const void *norm_w, *norm_b, *qkv_w, *qkv_b, *proj_mlp_w, *proj_mlp_b, *proj_out_w, *proj_out_b, *norm_q_w, *norm_k_w;
   const void* hidden;
@@ -428,6 +445,9 @@ typedef struct hdit_flux_single_block_args {
   int32_t qk_norm_kind;
   int32_t batch, seq, dim, heads, ff_dim, temb_dim;
   int32_t hidden_f32, out_f32;
+  int32_t n_txt, kv_rows, kv_row0, pad_;
+  const float* modulation;
+  void* kv_buffer;
 } hdit_flux_single_block_args;
 
 int64_t hdit_block_flux_single_workspace_bytes(const hdit_flux_single_block_args* args);
@@ -461,6 +481,8 @@ typedef struct hdit_cogvideox_block_args {
   int32_t batch, n_img, n_txt, dim, heads, ff_dim, temb_dim;
   int32_t hidden_f32, encoder_f32, out_f32;
   int32_t fp8_attention;
+  const float* modulation1;  /* optional precomputed linear(silu(temb)) of norm1 / norm2, f32 [batch, 6 dim] */
+  const float* modulation2;
 } hdit_cogvideox_block_args;
 
 int64_t hdit_block_cogvideox_workspace_bytes(const hdit_cogvideox_block_args* args);

@@ -47,7 +47,7 @@ def test_binding_covers_every_declared_symbol():
 
     assert sorted(_lib.SIGNATURES) == declared_symbols()
     lib = _lib.lib()
-    assert lib.hdit_abi_version() == _lib.ABI_VERSION == 3
+    assert lib.hdit_abi_version() == _lib.ABI_VERSION == 4
     assert lib.hdit_last_error() == b""
 
 
@@ -61,6 +61,41 @@ def test_struct_layouts_match_the_header(library):
     assert ctypes.sizeof(_lib.QkNormJob) == 8 + 3 * 8 + 4 * 8 + 4 * 4
     assert ctypes.sizeof(_lib.LnJob) == 4 * 8 + 5 * 8 + 4 * 4
     assert ctypes.sizeof(_lib.Sd3BlockArgs) == 20 * 8 + 9 * 8 + 8 + 14 * 4 + 8 + 2 * 4
+
+
+def test_struct_layouts_against_the_c_compiler(tmp_path):
+    """Every argument struct of include/hdit.h: sizeof and the offset of every field as gcc lays the header out,
+    against the ctypes mirror -- a field added on one side only, or in another order, fails here and not as a
+    misread pointer on the GPU."""
+    import subprocess
+
+    from hetu_dit_amd import _lib
+
+    pairs = {
+        "hdit_gemm_problem": _lib.GemmProblem, "hdit_seq_segment": _lib.SeqSegment, "hdit_attn_args": _lib.AttnArgs,
+        "hdit_qknorm_job": _lib.QkNormJob, "hdit_ln_job": _lib.LnJob, "hdit_sd3_block_weights": _lib.Sd3BlockWeights,
+        "hdit_sd3_block_args": _lib.Sd3BlockArgs, "hdit_flux_double_block_args": _lib.FluxDoubleBlockArgs,
+        "hdit_flux_single_block_args": _lib.FluxSingleBlockArgs, "hdit_cogvideox_block_args": _lib.CogVideoXBlockArgs,
+    }
+    lines = ["#include <stdio.h>", "#include <stddef.h>", f'#include "{HEADER}"', "int main(void) {"]
+    for cname, ct in pairs.items():
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        for fname, ftype in ct._fields_:
+            if fname.endswith("_") or isinstance(ftype, type) and issubclass(ftype, ctypes.Array):
+                continue
+            lines.append(f'  printf("{cname}.{fname} %zu\\n", offsetof({cname}, {fname}));')
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", str(src), "-o", str(exe)], check=True)
+    got = dict(line.split() for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for cname, ct in pairs.items():
+        assert int(got[cname]) == ctypes.sizeof(ct), cname
+        for fname, ftype in ct._fields_:
+            key = f"{cname}.{fname}"
+            if key in got:
+                assert int(got[key]) == getattr(ct, fname).offset, key
 
 
 def test_entry_points_reject_bad_arguments_without_a_gpu(library):

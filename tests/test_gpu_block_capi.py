@@ -231,3 +231,82 @@ def test_block_cogvideox_one_call_matches_python_block(hdit, stream_f32, fp8):
     tol = dict(rel=3e-2, cos=0.999) if fp8 else {}
     assert_parity(hid_c, o_hid, what="hdit_block_cogvideox hidden", **tol)
     assert_parity(enc_c, o_enc, what="hdit_block_cogvideox encoder", **tol)
+
+
+def _flux_stack(seed, layers=2, single_layers=3, D=512, H=4, hd=128):
+    from hetu_dit_amd import synthetic, transformer
+
+    stack = transformer.FluxTransformerBlocks(layers, single_layers, D, H, hd)
+    synthetic.init_module_(stack, seed)
+    return stack.to(DEV)
+
+
+@pytest.mark.parametrize("B", [1, 2])
+def test_flux_stack_through_entry_points_full_and_patches(hdit, B):
+    """``FluxTransformerBlocks`` with every block as one ``hdit_block_flux_double`` / ``_single`` call (modulation
+    from the stack's one GEMV, image K|V written straight into the layers' buffers) against the same stack
+    launched kernel by kernel: a full-sequence pass, then every pipeline patch over the stale buffers
+    (reference layers/attention_processor.py:908-922), bit for bit, outputs and buffers."""
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.cache_manager import get_cache_manager
+    from hetu_dit_amd.runtime_state import get_runtime_state
+
+    Nt, gh, gw, D, P = 24, 16, 8, 512, 4
+    N = gh * gw
+    starts = [gh // P * gw * i for i in range(P + 1)]
+    cos, sin = synthetic.rope_table(synthetic.flux_ids(Nt, gh, gw), (16, 56, 56))
+    stack = _flux_stack(71)
+    x_prev, x_now = synthetic.randn_bf16((B, N, D), 72).to(DEV), synthetic.randn_bf16((B, N, D), 73).to(DEV)
+    e, t = synthetic.randn_bf16((B, Nt, D), 74).to(DEV), synthetic.randn_bf16((B, D), 75).to(DEV)
+    rs = get_runtime_state()
+    rs.set_token_patches(starts)
+    rs.max_condition_sequence_length = Nt
+    cm = get_cache_manager()
+
+    def buffers():
+        return [entry.tensors[0] for entry in cm.cache.values() if entry.tensors[0] is not None]
+
+    def run_step(entry_points: bool):
+        stack.use_block_entry_points = entry_points
+        outs = []
+        rs.set_patched_mode(False)
+        rope = (cos.to(DEV), sin.to(DEV))
+        outs.append([o.clone() for o in stack(x_prev, e, t, rope)])
+        rs.set_patched_mode(True)
+        for p in range(P):
+            rows = torch.cat([torch.arange(Nt), Nt + torch.arange(starts[p], starts[p + 1])])
+            rope = (cos[rows].contiguous().to(DEV), sin[rows].contiguous().to(DEV))
+            outs.append([o.clone() for o in stack(x_now[:, starts[p]:starts[p + 1]].contiguous(), e, t, rope)])
+            rs.next_patch()
+        rs.set_patched_mode(False)
+        torch.cuda.synchronize()
+        return outs, [b.clone() for b in buffers()]
+
+    want, want_buf = run_step(False)
+    got, got_buf = run_step(True)
+    assert len(want_buf) == len(got_buf) == 5
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert torch.equal(g[0], w[0]) and torch.equal(g[1], w[1]), f"pass {i}"
+    # the per-kernel full pass registers strided views of its q|k|v tensors, the entry points contiguous buffers:
+    # compare contents
+    for g, w in zip(got_buf, want_buf):
+        assert torch.equal(g, w)
+
+
+def test_cogvideox_stack_through_entry_points(hdit):
+    from hetu_dit_amd import synthetic, transformer
+
+    B, Nt, grid, D, H, hd, L = 2, 26, (3, 6, 8), 256, 4, 64, 3
+    N = grid[0] * grid[1] * grid[2]
+    cos, sin = synthetic.rope_table(synthetic.cogvideox_positions(*grid), (16, 24, 24))
+    stack = transformer.CogVideoXTransformerBlocks(L, D, H, hd, time_embed_dim=64)
+    synthetic.init_module_(stack, 81)
+    stack = stack.to(DEV)
+    x, e, t = synthetic.randn_bf16((B, N, D), 82).to(DEV), synthetic.randn_bf16((B, Nt, D), 83).to(DEV), synthetic.randn_bf16((B, 64), 84).to(DEV)
+    rope = (cos.to(DEV), sin.to(DEV))
+    stack.use_block_entry_points = False
+    want = [o.clone() for o in stack(x, e, t, rope)]
+    stack.use_block_entry_points = True
+    got = stack(x, e, t, rope)
+    torch.cuda.synchronize()
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
