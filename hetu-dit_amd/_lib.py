@@ -11,6 +11,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("HDIT_LIBRARY") or os.path.join(HERE, "libhdit.so")
 
 HDIT_GEMM_MAX_PROBLEMS = 16
+HDIT_BLOCK_MAX_MULTI = 4
+HDIT_ATTN_MAX_MULTI = 4
 EPI_BIAS, EPI_BIAS_GELU, EPI_GATE_RESIDUAL = 0, 1, 2
 EPI_RESID_F32, EPI_OUT_F32 = 0x10, 0x20
 ABI_VERSION = 4
@@ -168,6 +170,8 @@ SIGNATURES = {
     "hdit_last_error": (C.c_char_p, []),
     "hdit_gemm_bf16": (C.c_int, [C.POINTER(GemmProblem), C.c_int, C.c_void_p]),
     "hdit_attn_fwd_bf16": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p]),
+    "hdit_attn_fwd_bf16_multi": (C.c_int, [C.POINTER(AttnArgs), C.c_int, C.c_void_p]),
+    "hdit_block_sd3_multi": (C.c_int, [C.POINTER(Sd3BlockArgs), C.c_int, C.c_void_p]),
     "hdit_attn_absmax": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p]),
     "hdit_attn_fp8_workspace_bytes": (C.c_int64, [C.POINTER(AttnArgs)]),
     "hdit_attn_fwd_fp8": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p, C.c_void_p, C.c_void_p]),

@@ -59,6 +59,9 @@ struct AttnParams {
 // pipelined: take the software-pipelined kernel (the caller has checked that the problem qualifies).
 int launch_d64(const AttnParams& P, int q_tiles, unsigned grid, bool pipelined, hipStream_t stream);
 int launch_d128(const AttnParams& P, int q_tiles, unsigned grid, bool pipelined, hipStream_t stream);
+// `count` problems of one head dim as one grid of the tracked or of the pipelined kernel
+int launch_multi_d64(const AttnParams* P, const int* q_tiles, const int* nblocks, int count, bool pipelined, hipStream_t stream);
+int launch_multi_d128(const AttnParams* P, const int* q_tiles, const int* nblocks, int count, bool pipelined, hipStream_t stream);
 
 }  // namespace hdit_attn
 
@@ -132,7 +135,8 @@ constexpr float RESCALE_THRESHOLD = 8.0f;
 // The whole kernel for one workgroup: the online softmax with a running reference that follows the column
 // maxima.  Also the second pass of the pipelined d = 64 kernel when its fixed reference overflowed.
 template <int HD>
-__device__ __forceinline__ void attn_tracked_body(const AttnParams& P, int q_tiles, unsigned char* lds) {
+__device__ __forceinline__ void attn_tracked_body(const AttnParams& P, int q_tiles, unsigned char* lds, int block_id,
+                                                  int nblocks) {
   using L = Lds<HD>;
   constexpr int KS = HD / 16;       // k-steps of the S^T MFMA (over head dim)
   constexpr int DB = HD / 32;       // 32-wide d blocks of O^T
@@ -150,9 +154,9 @@ __device__ __forceinline__ void attn_tracked_body(const AttnParams& P, int q_til
   // the partly filled last query tiles (some of their waves have no rows and skip the arithmetic) come after
   // all full ones: workgroups are placed in id order, one per CU first, so when a launch has a few more
   // workgroups than CUs it is the light ones that share a CU with a full one.
-  const int nbh = gridDim.x / q_tiles;
+  const int nbh = nblocks / q_tiles;
   const bool by_xcd = nbh % 8 == 0;
-  const int slot = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int slot = by_xcd ? (block_id >> 3) : block_id;
   const int nbh_loc = by_xcd ? nbh / 8 : nbh;
   int qt = slot % q_tiles, bhl = slot / q_tiles;
   if (q_tiles > 1 && P.sq % BQ != 0) {
@@ -165,7 +169,7 @@ __device__ __forceinline__ void attn_tracked_body(const AttnParams& P, int q_til
       bhl = slot - heavy;
     }
   }
-  const int bh = by_xcd ? bhl * 8 + (int)(blockIdx.x & 7) : bhl;
+  const int bh = by_xcd ? bhl * 8 + (block_id & 7) : bhl;
   const int b = bh / P.heads, h = bh % P.heads;
   const int q0 = qt * BQ + wave * WQ;
   // a wave past the last query row still stages K/V tiles and meets the barriers, but does no arithmetic
@@ -501,7 +505,30 @@ __device__ __forceinline__ void attn_tracked_body(const AttnParams& P, int q_til
 template <int HD>
 __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_kernel(const AttnParams P, int q_tiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  attn_tracked_body<HD>(P, q_tiles, lds);
+  attn_tracked_body<HD>(P, q_tiles, lds, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// Several independent attention problems of one head dim in one grid (the blocks of neighbouring pipeline patches
+// that run side by side): problem i owns the workgroups [start[i], start[i + 1]), each range a multiple of 8 long so
+// that a workgroup's position modulo 8 -- the XCD it lands on -- is the same inside its problem as in the launch.
+constexpr int ATTN_MAX_MULTI = HDIT_ATTN_MAX_MULTI;
+struct AttnMulti {
+  AttnParams p[ATTN_MAX_MULTI];
+  int q_tiles[ATTN_MAX_MULTI];
+  int nblocks[ATTN_MAX_MULTI];   // workgroups that have work (the range may be padded beyond them)
+  int start[ATTN_MAX_MULTI + 1];
+  int count;
+};
+
+template <int HD>
+__global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_multi_kernel(const AttnMulti M) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int i = 0;
+#pragma unroll 1
+  while (i + 1 < M.count && (int)blockIdx.x >= M.start[i + 1]) i++;
+  const int local = (int)blockIdx.x - M.start[i];
+  if (local >= M.nblocks[i]) return;
+  attn_tracked_body<HD>(M.p[i], M.q_tiles[i], lds, local, M.nblocks[i]);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -549,8 +576,7 @@ constexpr int PIPE_MIN_TILES = 3;
 #define SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 
 template <int HD>
-__global__ void __launch_bounds__(256, 1) attn_fwd_pipe_kernel(const AttnParams P, int q_tiles) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+__device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles, unsigned char* lds, int block_id, int nblocks) {
   using PL = PipeLds<HD>;
   constexpr int KS = HD / 16, DB = HD / 32, CPR = HD / 8, NCH = BKV * CPR / 256, RPI = 64 / CPR, ROW = PL::ROW;
   constexpr int PIPE_TILE = PL::TILE, PIPE_V_OFF = PL::V_OFF, PIPE_FLAG_OFF = PL::FLAG_OFF;
@@ -559,9 +585,9 @@ __global__ void __launch_bounds__(256, 1) attn_fwd_pipe_kernel(const AttnParams 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
   // same placement of (batch, head, query tile) on workgroups as the kernel above
-  const int nbh = gridDim.x / q_tiles;
+  const int nbh = nblocks / q_tiles;
   const bool by_xcd = nbh % 8 == 0;
-  const int slot = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int slot = by_xcd ? (block_id >> 3) : block_id;
   const int nbh_loc = by_xcd ? nbh / 8 : nbh;
   int qt = slot % q_tiles, bhl = slot / q_tiles;
   if (q_tiles > 1 && P.sq % BQ != 0) {
@@ -574,7 +600,7 @@ __global__ void __launch_bounds__(256, 1) attn_fwd_pipe_kernel(const AttnParams 
       bhl = slot - heavy;
     }
   }
-  const int bh = by_xcd ? bhl * 8 + (int)(blockIdx.x & 7) : bhl;
+  const int bh = by_xcd ? bhl * 8 + (block_id & 7) : bhl;
   const int b = bh / P.heads, h = bh % P.heads;
   const int q0 = qt * BQ + wave * WQ;
   const bool active = __builtin_amdgcn_readfirstlane(q0 < P.sq);
@@ -702,7 +728,7 @@ __global__ void __launch_bounds__(256, 1) attn_fwd_pipe_kernel(const AttnParams 
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
     __syncthreads();  // the flag barrier
-    if (*(volatile lds_int*)flag) attn_tracked_body<HD>(P, q_tiles, lds);
+    if (*(volatile lds_int*)flag) attn_tracked_body<HD>(P, q_tiles, lds, block_id, nblocks);
     return;
   }
 
@@ -968,7 +994,7 @@ __global__ void __launch_bounds__(256, 1) attn_fwd_pipe_kernel(const AttnParams 
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
     __syncthreads();
     if (*(volatile lds_int*)flag) {
-      attn_tracked_body<HD>(P, q_tiles, lds);
+      attn_tracked_body<HD>(P, q_tiles, lds, block_id, nblocks);
       return;
     }
   }
@@ -993,5 +1019,39 @@ __global__ void __launch_bounds__(256, 1) attn_fwd_pipe_kernel(const AttnParams 
   }
 }
 
+
+template <int HD>
+__global__ void __launch_bounds__(256, 1) attn_fwd_pipe_kernel(const AttnParams P, int q_tiles) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  attn_pipe_body<HD>(P, q_tiles, lds, (int)blockIdx.x, (int)gridDim.x);
+}
+
+template <int HD>
+__global__ void __launch_bounds__(256, 1) attn_fwd_pipe_multi_kernel(const AttnMulti M) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int i = 0;
+#pragma unroll 1
+  while (i + 1 < M.count && (int)blockIdx.x >= M.start[i + 1]) i++;
+  const int local = (int)blockIdx.x - M.start[i];
+  if (local >= M.nblocks[i]) return;
+  attn_pipe_body<HD>(M.p[i], M.q_tiles[i], lds, local, M.nblocks[i]);
+}
+
+// Host side of a multi launch: the table of `count` problems, ranges padded to multiples of 8 workgroups.
+inline int fill_multi(AttnMulti& M, const AttnParams* P, const int* q_tiles, const int* nblocks, int count) {
+  M.count = count;
+  int at = 0;
+  for (int i = 0; i < ATTN_MAX_MULTI; i++) {
+    M.start[i] = at;
+    if (i < count) {
+      M.p[i] = P[i], M.q_tiles[i] = q_tiles[i], M.nblocks[i] = nblocks[i];
+      at += (nblocks[i] + 7) / 8 * 8;
+    } else {
+      M.p[i] = P[0], M.q_tiles[i] = 1, M.nblocks[i] = 0;
+    }
+  }
+  M.start[ATTN_MAX_MULTI] = at;
+  return at;
+}
 
 }  // namespace

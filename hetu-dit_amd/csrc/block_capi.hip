@@ -119,37 +119,45 @@ extern "C" __attribute__((visibility("default"))) int64_t hdit_block_sd3_workspa
   return carve(a, nullptr).bytes;
 }
 
-extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_sd3_block_args* a, void* stream) {
+namespace {
+
+// The launches of one SD3 joint block, stage by stage: what hdit_block_sd3 enqueues in this order, and what
+// hdit_block_sd3_multi merges stage-wise over several independent blocks.
+struct Sd3Plan {
+  const hdit_sd3_block_args* a;
+  Sd3Workspace ws;
+  bool gemv_img, gemv_txt;   // adaLN projections to compute here (no precomputed modulation given)
+  hdit_ln_job ln1[2], ln2[2];
+  int n_ln1, n_ln2;
+  hdit_gemm_problem qkv[HDIT_GEMM_MAX_PROBLEMS], outp[2], ff1[2], ff2[2];
+  int n_qkv, n_out, n_ff1, n_ff2;
+  hdit_attn_args attn;
+};
+
+int plan_sd3(const hdit_sd3_block_args* a, Sd3Plan& pl) {
   int rc = validate(a);
   if (rc != HDIT_OK) return rc;
   if (!a->workspace || (((uintptr_t)a->workspace) & (ALIGN - 1))) return HDIT_EINVAL;
-  const Sd3Workspace ws = carve(a, (unsigned char*)a->workspace);
+  pl.a = a;
+  pl.ws = carve(a, (unsigned char*)a->workspace);
+  const Sd3Workspace& ws = pl.ws;
   if (a->workspace_bytes < ws.bytes) return HDIT_EINVAL;
   const hdit_sd3_block_weights& w = a->w;
   const int B = a->batch, Ni = a->n_img, Nt = a->n_txt, D = a->dim, F = a->ff_dim, H = a->heads, hd = D / H;
   const bool pre_only = a->context_pre_only != 0;
   const bool text_out = !pre_only && !a->skip_text_output;
-  const float eps = 1e-6f;
   const int64_t md = 6 * (int64_t)D;                 // batch stride of the image stream's modulation
   const int64_t mdt = (pre_only ? 2 : 6) * (int64_t)D;
-  const int sz_in = a->hidden_f32 ? 4 : 2, sz_enc = a->encoder_f32 ? 4 : 2;
-  (void)sz_in, (void)sz_enc;
 
   // 1. adaLN projections: linear(silu(temb)) for both streams (a caller that already holds them for this temb --
   //    the projections of all blocks of a stack fit one launch -- passes them in and skips this step)
   const float* emb_img = a->modulation_img;
   const float* emb_txt = a->modulation_txt;
-  if (!emb_img) {
-    if ((rc = hdit_adaln_gemv(a->temb, w.norm1_w, w.norm1_b, ws.emb_img, B, 6 * D, a->temb_dim, stream))) return rc;
-    emb_img = ws.emb_img;
-  }
   const bool reuse_text_kv = a->text_kv_mode == HDIT_TEXT_KV_REUSE;  // the text stream is not touched at all
-  if (!emb_txt && !reuse_text_kv) {
-    if ((rc = hdit_adaln_gemv(a->temb, w.norm1_context_w, w.norm1_context_b, ws.emb_txt, B, (pre_only ? 2 : 6) * D,
-                              a->temb_dim, stream)))
-      return rc;
-    emb_txt = ws.emb_txt;
-  }
+  pl.gemv_img = !emb_img;
+  pl.gemv_txt = !emb_txt && !reuse_text_kv;
+  if (pl.gemv_img) emb_img = ws.emb_img;
+  if (pl.gemv_txt) emb_txt = ws.emb_txt;
   // chunks: shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp; AdaLayerNormContinuous: scale, shift
   const float *sh_a = emb_img, *sc_a = emb_img + D, *g_a = emb_img + 2 * D, *sh_m = emb_img + 3 * D, *sc_m = emb_img + 4 * D,
               *g_m = emb_img + 5 * D;
@@ -164,19 +172,19 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
   }
 
   // 2. norm1 + modulate, both streams in one launch
-  hdit_ln_job jobs[2];
-  memset(jobs, 0, sizeof(jobs));
+  hdit_ln_job* jobs = pl.ln1;
+  memset(pl.ln1, 0, sizeof(pl.ln1));
   jobs[0].x = a->hidden, jobs[0].y = ws.n_img, jobs[0].shift = sh_a, jobs[0].scale = sc_a;
   jobs[0].x_sb = (int64_t)Ni * D, jobs[0].x_st = D, jobs[0].y_sb = (int64_t)Ni * D, jobs[0].y_st = D, jobs[0].mod_stride = md;
   jobs[0].batch = B, jobs[0].tokens = Ni, jobs[0].x_f32 = a->hidden_f32;
   jobs[1].x = a->encoder, jobs[1].y = ws.n_txt, jobs[1].shift = c_sh_a, jobs[1].scale = c_sc_a;
   jobs[1].x_sb = (int64_t)Nt * D, jobs[1].x_st = D, jobs[1].y_sb = (int64_t)Nt * D, jobs[1].y_st = D, jobs[1].mod_stride = mdt;
   jobs[1].batch = B, jobs[1].tokens = Nt, jobs[1].x_f32 = a->encoder_f32;
-  if ((rc = hdit_layernorm_modulate_jobs(jobs, reuse_text_kv ? 1 : 2, D, nullptr, nullptr, eps, stream))) return rc;
+  pl.n_ln1 = reuse_text_kv ? 1 : 2;
 
   // 3. q|k|v of both streams in one grouped launch.  With a stale K/V buffer the image stream's k|v rows go
   //    straight into rows [kv_row0, kv_row0 + n_img) of it, one problem per batch element.
-  hdit_gemm_problem probs[HDIT_GEMM_MAX_PROBLEMS];
+  hdit_gemm_problem* probs = pl.qkv;
   int np = 0;
   const unsigned char* qkv_w = (const unsigned char*)w.qkv_w;
   const unsigned char* qkv_b = (const unsigned char*)w.qkv_b;
@@ -226,10 +234,10 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
     tq_ld = tkv_ld = 3 * (int64_t)D;
     q_txt = ws.qkv_txt, k_txt = ws.qkv_txt + (int64_t)D * 2, v_txt = ws.qkv_txt + (int64_t)2 * D * 2;
   }
-  if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
+  pl.n_qkv = np;
 
   // 4. joint attention over [image, text]; image keys / values come from the stale buffer when there is one
-  hdit_attn_args at;
+  hdit_attn_args& at = pl.attn;
   memset(&at, 0, sizeof(at));
   auto seg = [&](hdit_seq_segment& s, const void* p, int64_t rows_per_batch, int64_t ld, int len) {
     s.ptr = p, s.stride_b = rows_per_batch * ld, s.stride_s = ld, s.stride_h = hd, s.len = len;
@@ -245,12 +253,6 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
     seg(at.o[1], ws.o_txt, Nt, D, Nt);
   }
   at.batch = B, at.heads = H, at.head_dim = hd, at.scale = 0.f;
-  if (a->fp8_attention) {
-    if ((rc = hdit_attn_absmax(&at, ws.absmax, stream))) return rc;
-    if ((rc = hdit_attn_fwd_fp8(&at, ws.absmax, ws.fp8, stream))) return rc;
-  } else if ((rc = hdit_attn_fwd_bf16(&at, stream))) {
-    return rc;
-  }
 
   // 5. out-projections with the gated residual; the stream stays fp32 inside the block
   auto gated = [&](hdit_gemm_problem& p, const void* resid, int resid_f32, const float* gate, int64_t gate_stride, int rows,
@@ -259,17 +261,18 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
     p.resid = resid, p.ldr = p.n, p.gate = gate, p.gate_stride = (int32_t)gate_stride, p.rows_per_batch = rows;
   };
   np = 0;
-  probs[np] = problem(ws.o_img, D, w.to_out_w, w.to_out_b, ws.x1_img, D, B * Ni, D, D, 0);
-  gated(probs[np++], a->hidden, a->hidden_f32, g_a, md, Ni, 1);
+  pl.outp[np] = problem(ws.o_img, D, w.to_out_w, w.to_out_b, ws.x1_img, D, B * Ni, D, D, 0);
+  gated(pl.outp[np++], a->hidden, a->hidden_f32, g_a, md, Ni, 1);
   if (text_out) {
-    probs[np] = problem(ws.o_txt, D, w.to_add_out_w, w.to_add_out_b, ws.x1_txt, D, B * Nt, D, D, 0);
-    gated(probs[np++], a->encoder, a->encoder_f32, c_g_a, mdt, Nt, 1);
+    pl.outp[np] = problem(ws.o_txt, D, w.to_add_out_w, w.to_add_out_b, ws.x1_txt, D, B * Nt, D, D, 0);
+    gated(pl.outp[np++], a->encoder, a->encoder_f32, c_g_a, mdt, Nt, 1);
   }
-  if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
+  pl.n_out = np;
 
   // 6. norm2 + modulate on the fp32 stream
   int nj = 0;
-  memset(jobs, 0, sizeof(jobs));
+  jobs = pl.ln2;
+  memset(pl.ln2, 0, sizeof(pl.ln2));
   jobs[nj].x = ws.x1_img, jobs[nj].y = ws.n_img, jobs[nj].shift = sh_m, jobs[nj].scale = sc_m;
   jobs[nj].x_sb = (int64_t)Ni * D, jobs[nj].x_st = D, jobs[nj].y_sb = (int64_t)Ni * D, jobs[nj].y_st = D, jobs[nj].mod_stride = md;
   jobs[nj].batch = B, jobs[nj].tokens = Ni, jobs[nj].x_f32 = 1;
@@ -280,21 +283,122 @@ extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_
     jobs[nj].batch = B, jobs[nj].tokens = Nt, jobs[nj].x_f32 = 1;
     nj++;
   }
-  if ((rc = hdit_layernorm_modulate_jobs(jobs, nj, D, nullptr, nullptr, eps, stream))) return rc;
+  pl.n_ln2 = nj;
 
   // 7. MLP: bias + GELU-tanh in the first epilogue, gated residual in the second
   np = 0;
-  probs[np++] = problem(ws.n_img, D, w.ff_in_w, w.ff_in_b, ws.h_img, F, B * Ni, F, D, HDIT_EPI_BIAS_GELU);
-  if (text_out) probs[np++] = problem(ws.n_txt, D, w.ff_context_in_w, w.ff_context_in_b, ws.h_txt, F, B * Nt, F, D, HDIT_EPI_BIAS_GELU);
-  if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
+  pl.ff1[np++] = problem(ws.n_img, D, w.ff_in_w, w.ff_in_b, ws.h_img, F, B * Ni, F, D, HDIT_EPI_BIAS_GELU);
+  if (text_out) pl.ff1[np++] = problem(ws.n_txt, D, w.ff_context_in_w, w.ff_context_in_b, ws.h_txt, F, B * Nt, F, D, HDIT_EPI_BIAS_GELU);
+  pl.n_ff1 = np;
   np = 0;
-  probs[np] = problem(ws.h_img, F, w.ff_out_w, w.ff_out_b, a->hidden_out, D, B * Ni, D, F, 0);
-  gated(probs[np++], ws.x1_img, 1, g_m, md, Ni, a->out_f32);
+  pl.ff2[np] = problem(ws.h_img, F, w.ff_out_w, w.ff_out_b, a->hidden_out, D, B * Ni, D, F, 0);
+  gated(pl.ff2[np++], ws.x1_img, 1, g_m, md, Ni, a->out_f32);
   if (text_out) {
-    probs[np] = problem(ws.h_txt, F, w.ff_context_out_w, w.ff_context_out_b, a->encoder_out, D, B * Nt, D, F, 0);
-    gated(probs[np++], ws.x1_txt, 1, c_g_m, mdt, Nt, a->out_f32);
+    pl.ff2[np] = problem(ws.h_txt, F, w.ff_context_out_w, w.ff_context_out_b, a->encoder_out, D, B * Nt, D, F, 0);
+    gated(pl.ff2[np++], ws.x1_txt, 1, c_g_m, mdt, Nt, a->out_f32);
   }
-  return hdit_gemm_bf16(probs, np, stream);
+  pl.n_ff2 = np;
+  return HDIT_OK;
+}
+
+int run_gemvs(const Sd3Plan& pl, void* stream) {
+  const hdit_sd3_block_args* a = pl.a;
+  int rc;
+  if (pl.gemv_img && (rc = hdit_adaln_gemv(a->temb, a->w.norm1_w, a->w.norm1_b, pl.ws.emb_img, a->batch, 6 * a->dim, a->temb_dim, stream)))
+    return rc;
+  if (pl.gemv_txt && (rc = hdit_adaln_gemv(a->temb, a->w.norm1_context_w, a->w.norm1_context_b, pl.ws.emb_txt, a->batch,
+                                           (a->context_pre_only ? 2 : 6) * a->dim, a->temb_dim, stream)))
+    return rc;
+  return HDIT_OK;
+}
+
+int run_attention(const Sd3Plan& pl, void* stream) {
+  int rc;
+  if (pl.a->fp8_attention) {
+    if ((rc = hdit_attn_absmax(&pl.attn, pl.ws.absmax, stream))) return rc;
+    return hdit_attn_fwd_fp8(&pl.attn, pl.ws.absmax, pl.ws.fp8, stream);
+  }
+  return hdit_attn_fwd_bf16(&pl.attn, stream);
+}
+
+// Problems of several plans, one launch per HDIT_GEMM_MAX_PROBLEMS (a launch plans its problems together).
+template <class Get>
+int run_gemm_stage(const Sd3Plan* plans, int count, Get get, void* stream) {
+  hdit_gemm_problem probs[HDIT_GEMM_MAX_PROBLEMS];
+  int np = 0, rc;
+  for (int i = 0; i < count; i++) {
+    int n;
+    const hdit_gemm_problem* p = get(plans[i], n);
+    if (np + n > HDIT_GEMM_MAX_PROBLEMS) {
+      if ((rc = hdit_gemm_bf16(probs, np, stream))) return rc;
+      np = 0;
+    }
+    for (int k = 0; k < n; k++) probs[np++] = p[k];
+  }
+  return np ? hdit_gemm_bf16(probs, np, stream) : HDIT_OK;
+}
+
+template <class Get>
+int run_ln_stage(const Sd3Plan* plans, int count, Get get, int dim, void* stream) {
+  hdit_ln_job jobs[HDIT_LN_MAX_JOBS];
+  int nj = 0, rc;
+  for (int i = 0; i < count; i++) {
+    int n;
+    const hdit_ln_job* j = get(plans[i], n);
+    if (nj + n > HDIT_LN_MAX_JOBS) {
+      if ((rc = hdit_layernorm_modulate_jobs(jobs, nj, dim, nullptr, nullptr, 1e-6f, stream))) return rc;
+      nj = 0;
+    }
+    for (int k = 0; k < n; k++) jobs[nj++] = j[k];
+  }
+  return nj ? hdit_layernorm_modulate_jobs(jobs, nj, dim, nullptr, nullptr, 1e-6f, stream) : HDIT_OK;
+}
+
+// `count` planned blocks, stage by stage: the launches of each stage merged into one
+int run_sd3_plans(const Sd3Plan* plans, int count, void* stream) {
+  int rc;
+  const int D = plans[0].a->dim;
+  for (int i = 0; i < count; i++)
+    if ((rc = run_gemvs(plans[i], stream))) return rc;
+  if ((rc = run_ln_stage(plans, count, [](const Sd3Plan& p, int& n) { n = p.n_ln1; return p.ln1; }, D, stream))) return rc;
+  if ((rc = run_gemm_stage(plans, count, [](const Sd3Plan& p, int& n) { n = p.n_qkv; return p.qkv; }, stream))) return rc;
+  bool any_fp8 = false;
+  for (int i = 0; i < count; i++) any_fp8 |= plans[i].a->fp8_attention != 0;
+  if (count == 1 || any_fp8) {
+    for (int i = 0; i < count; i++)
+      if ((rc = run_attention(plans[i], stream))) return rc;
+  } else {
+    hdit_attn_args at[HDIT_ATTN_MAX_MULTI];
+    for (int first = 0; first < count; first += HDIT_ATTN_MAX_MULTI) {
+      const int n = count - first < HDIT_ATTN_MAX_MULTI ? count - first : HDIT_ATTN_MAX_MULTI;
+      for (int i = 0; i < n; i++) at[i] = plans[first + i].attn;
+      if ((rc = hdit_attn_fwd_bf16_multi(at, n, stream))) return rc;
+    }
+  }
+  if ((rc = run_gemm_stage(plans, count, [](const Sd3Plan& p, int& n) { n = p.n_out; return p.outp; }, stream))) return rc;
+  if ((rc = run_ln_stage(plans, count, [](const Sd3Plan& p, int& n) { n = p.n_ln2; return p.ln2; }, D, stream))) return rc;
+  if ((rc = run_gemm_stage(plans, count, [](const Sd3Plan& p, int& n) { n = p.n_ff1; return p.ff1; }, stream))) return rc;
+  return run_gemm_stage(plans, count, [](const Sd3Plan& p, int& n) { n = p.n_ff2; return p.ff2; }, stream);
+}
+
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int hdit_block_sd3(const hdit_sd3_block_args* a, void* stream) {
+  Sd3Plan pl;
+  const int rc = plan_sd3(a, pl);
+  if (rc != HDIT_OK) return rc;
+  return run_sd3_plans(&pl, 1, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_block_sd3_multi(const hdit_sd3_block_args* args, int count, void* stream) {
+  if (!args || count <= 0 || count > HDIT_BLOCK_MAX_MULTI) return HDIT_EINVAL;
+  static thread_local Sd3Plan plans[HDIT_BLOCK_MAX_MULTI];
+  for (int i = 0; i < count; i++) {
+    const int rc = plan_sd3(&args[i], plans[i]);
+    if (rc != HDIT_OK) return rc;
+    if (args[i].dim != args[0].dim || args[i].heads != args[0].heads) return HDIT_EINVAL;
+  }
+  return run_sd3_plans(plans, count, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------

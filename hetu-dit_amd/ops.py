@@ -361,12 +361,23 @@ class Sd3BlockCall:
         a.context_pre_only = int(bool(block.context_pre_only))
         a.fp8_attention = int(bool(getattr(block.attn, "fp8_attention", False)))
 
-    def __call__(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
-                 out_dtype=bf16, skip_text_output: bool = False, kv_buffer: Optional[torch.Tensor] = None,
-                 kv_row0: int = 0, modulation_img: Optional[int] = None, modulation_txt: Optional[int] = None,
-                 hidden_out: Optional[torch.Tensor] = None, text_kv: Optional[torch.Tensor] = None,
-                 text_kv_mode: int = _lib.TEXT_KV_NONE):
-        """Same contract as ``block_sd3``.  ``modulation_img`` / ``modulation_txt``: device addresses of the f32
+    def __call__(self, *args, **kwargs):
+        """Fill the argument struct (``prepare``) and launch the block on the current stream."""
+        encoder_out, hidden_out, ws = self.prepare(*args, **kwargs)
+        check(_lib.lib().hdit_block_sd3(C.byref(self.args), _stream()), "hdit_block_sd3")
+        # stream-ordered reuse: the workspace may be freed as soon as the launches are queued
+        del ws
+        return encoder_out, hidden_out
+
+    def prepare(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
+                out_dtype=bf16, skip_text_output: bool = False, kv_buffer: Optional[torch.Tensor] = None,
+                kv_row0: int = 0, modulation_img: Optional[int] = None, modulation_txt: Optional[int] = None,
+                hidden_out: Optional[torch.Tensor] = None, text_kv: Optional[torch.Tensor] = None,
+                text_kv_mode: int = _lib.TEXT_KV_NONE):
+        """Fills ``self.args`` for one call without launching; returns ``(encoder_out_or_None, hidden_out,
+        workspace tensor)`` -- the caller launches (``hdit_block_sd3`` or, with other blocks' structs,
+        ``sd3_blocks_launch``) and keeps the workspace alive until then.
+        Same contract as ``block_sd3``.  ``modulation_img`` / ``modulation_txt``: device addresses of the f32
         [batch, 6 dim] (text stream of a ``context_pre_only`` block: [batch, 2 dim]) adaLN projections of this
         block for this ``temb`` (the caller keeps their tensor alive), or None to have the call compute them.
         ``hidden_out``: a contiguous [batch, n_img, dim] tensor of ``out_dtype`` to write the image stream to.
@@ -417,10 +428,17 @@ class Sd3BlockCall:
             self._ws_bytes[key] = nbytes
         ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)
         a.workspace, a.workspace_bytes = (ws.data_ptr() + 255) // 256 * 256, nbytes
-        check(lib.hdit_block_sd3(C.byref(a), _stream()), "hdit_block_sd3")
-        # stream-ordered reuse: these may be freed by the caller as soon as the launches are queued
-        del ws
-        return encoder_out, hidden_out
+        return encoder_out, hidden_out, ws
+
+
+def sd3_blocks_launch(calls: Sequence["Sd3BlockCall"]):
+    """The prepared calls -- blocks that do not depend on each other -- as one ``hdit_block_sd3_multi`` call per
+    ``HDIT_BLOCK_MAX_MULTI``: every stage of the blocks (normalise, q|k|v, attention, ...) is one merged launch."""
+    lib = _lib.lib()
+    for first in range(0, len(calls), _lib.HDIT_BLOCK_MAX_MULTI):
+        chunk = calls[first : first + _lib.HDIT_BLOCK_MAX_MULTI]
+        arr = (_lib.Sd3BlockArgs * len(chunk))(*(c.args for c in chunk))
+        check(lib.hdit_block_sd3_multi(arr, len(chunk), _stream()), "hdit_block_sd3_multi")
 
 
 class _ArgFiller:

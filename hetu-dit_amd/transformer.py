@@ -71,6 +71,7 @@ class SD3TransformerBlocks(nn.Module):
         self.use_block_entry_points = True
         self.batch_streams = 2
         self.reuse_text_kv = True  # patch mode: later patches take the text keys / values the first patch projected
+        self.group_fronts = True   # forward_patches on one stream: one merged call per front of independent blocks
         self._block_calls: Optional[List[ops.Sd3BlockCall]] = None
         # per block: (k|v buffer of the text stream, the text states and temb it was projected from, with their
         # in-place modification counters) -- patch mode
@@ -99,9 +100,11 @@ class SD3TransformerBlocks(nn.Module):
         return self._block_calls
 
     def _run_block(self, i: int, calls, mods, hidden, encoder, temb, skip_text_output: bool = False,
-                   kv_buffer=None, kv_row0: int = 0, batch0: int = 0, hidden_out=None, patch: Optional[int] = None):
+                   kv_buffer=None, kv_row0: int = 0, batch0: int = 0, hidden_out=None, patch: Optional[int] = None,
+                   defer: Optional[list] = None):
         """Block i on the current stream: ``(encoder_out_or_None, hidden_out)``.  ``batch0``: index of the
         first batch element of ``hidden`` within the ``temb`` the modulation ``mods`` was computed for.
+        ``defer``: a list -- the call is prepared and appended to it instead of launched (``_launch_front``).
         ``patch``: index of the pipeline patch in patch mode.  The later patches of a step are fed the text states
         the first one stored (``transformer_sd3.py:131-146``), so the text stream's keys and values are the same
         numbers for all of them: the first patch's call leaves them in a buffer and the later ones take them from
@@ -129,13 +132,18 @@ class SD3TransformerBlocks(nn.Module):
         dim = hidden.shape[2]
         rows_txt = (2 if block.context_pre_only else 6) * dim
         base = flat.data_ptr()
-        return calls[i](
-            hidden, encoder, temb, out_dtype=block.stream_dtype, skip_text_output=skip_text_output,
-            kv_buffer=kv_buffer, kv_row0=kv_row0,
+        kwargs = dict(
+            out_dtype=block.stream_dtype, skip_text_output=skip_text_output, kv_buffer=kv_buffer, kv_row0=kv_row0,
             modulation_img=base + 4 * (offsets[block.norm1] + batch0 * 6 * dim),
             modulation_txt=base + 4 * (offsets[block.norm1_context] + batch0 * rows_txt),
             hidden_out=hidden_out, text_kv=text_kv, text_kv_mode=text_kv_mode,
         )
+        if defer is None:
+            return calls[i](hidden, encoder, temb, **kwargs)
+        # the struct is filled, the launch is the caller's (merged with the other blocks of its front)
+        encoder_out, hidden_new, ws = calls[i].prepare(hidden, encoder, temb, **kwargs)
+        defer.append((calls[i], ws))
+        return encoder_out, hidden_new
 
     def _kv_buffer(self, i: int, hidden: torch.Tensor):
         """``(buffer, first row)``: the K|V buffer block i's image stream writes into, from the cache manager --
@@ -244,7 +252,8 @@ class SD3TransformerBlocks(nn.Module):
             raise ValueError("num_streams must be at least 1")
         main = torch.cuda.current_stream()
         if num_streams > 1 and torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("forward_patches with several streams cannot be captured into a graph")
+            raise RuntimeError("forward_patches with several streams cannot be captured into a graph "
+                               "(num_streams=1 can: its fronts are merged launches on the caller's stream)")
         calls = self._entry_point_calls()
         if calls is not None and not self._persistent_buffers_contiguous():
             calls = None
@@ -257,6 +266,8 @@ class SD3TransformerBlocks(nn.Module):
             encoder_hidden_states, temb = encoder_hidden_states.contiguous(), temb.contiguous()
             mods = self.modulation.precompute_by_module(temb)
         device = hidden[0].device
+        if num_streams == 1 and calls is not None and self.group_fronts:
+            return self._forward_patches_grouped(calls, mods, hidden, encoder_hidden_states, temb)
         streams = [main] if num_streams == 1 else side_streams(device, min(num_streams, P))
         start = torch.cuda.Event()
         start.record(main)
@@ -300,6 +311,40 @@ class SD3TransformerBlocks(nn.Module):
                 main.wait_event(joined)
         for h in hidden:
             h.record_stream(main)  # allocated on a side stream, read by the caller on its own
+        return hidden
+
+    def _forward_patches_grouped(self, calls, mods, hidden, encoder_hidden_states, temb):
+        """``forward_patches`` on ONE stream: the blocks (patch p, layer l) of a front p + l = const do not depend on
+        each other, so every front is one ``hdit_block_sd3_multi`` call -- each stage of its up to four blocks
+        one merged launch (one grouped q|k|v GEMM of 4 x 198 tiles, one attention grid of 4 x 192 workgroups, ...)
+        instead of four patch-sized launches that each fill a fraction of the GPU.  No side stream, no event, every
+        allocation on the caller's stream: the pass can be recorded into a HIP graph.  Same operands and kernels
+        per block as the sequential pass, so the same bits."""
+        rs = get_runtime_state()
+        P, L = len(hidden), len(self.transformer_blocks)
+        cache = self.encoder_hidden_states_cache
+        try:
+            for front in range(L + P - 1):
+                group = []
+                for p in range(P):
+                    i = front - p
+                    if not 0 <= i < L:
+                        continue
+                    rs.pipeline_patch_idx = p
+                    kv = self._kv_buffer(i, hidden[p])
+                    if p == 0:
+                        cache[i] = encoder_hidden_states
+                        encoder_hidden_states, hidden[0] = self._run_block(
+                            i, calls, mods, hidden[0], encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1], patch=0,
+                            defer=group)
+                    else:
+                        _, hidden[p] = self._run_block(
+                            i, calls, mods, hidden[p], cache[i], temb, skip_text_output=True, kv_buffer=kv[0],
+                            kv_row0=kv[1], patch=p, defer=group)
+                ops.sd3_blocks_launch([c for c, _ in group])
+                del group  # the workspaces: stream-ordered reuse once the launches are queued
+        finally:
+            rs.pipeline_patch_idx = 0
         return hidden
 
 

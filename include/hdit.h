@@ -143,6 +143,15 @@ typedef struct hdit_attn_args {
 
 int hdit_attn_fwd_bf16(const hdit_attn_args* args, void* stream);
 
+/* `count` (<= HDIT_ATTN_MAX_MULTI) independent attention problems of one head dim
+ * as ONE launch.  No single call site in the reference: the blocks (patch p, layer
+ * l) with p + l constant of a PipeFusion step
+ * (model_executor/pipelines/pipeline_stable_diffusion_3.py:1549-1644 runs them one
+ * after the other) are independent, and each alone leaves most of the GPU idle.
+ * Results are those of `count` hdit_attn_fwd_bf16 calls, bit for bit. */
+#define HDIT_ATTN_MAX_MULTI 4
+int hdit_attn_fwd_bf16_multi(const hdit_attn_args* args, int count, void* stream);
+
 /* Same contract on the fp8-e4m3 (OCP) MFMA path: Q, K, V are quantised with one
  * absmax scale per (batch, head) taken from `absmax` (f32 [3, batch, heads]:
  * q, k, v; written by hdit_attn_absmax), P is re-quantised per tile.  K and V
@@ -190,7 +199,7 @@ int hdit_layernorm_modulate(const void* x, void* y, const float* shift, const fl
 /* The same for up to HDIT_LN_MAX_JOBS tensors of one width in one launch (the
  * image and the text stream of a joint block: norm1 + norm1_context, or
  * norm2 + norm2_context, of the blocks cited above). */
-#define HDIT_LN_MAX_JOBS 4
+#define HDIT_LN_MAX_JOBS 8
 typedef struct hdit_ln_job {
   const void* x;      /* bf16 [batch, tokens, dim], or f32 with x_f32 */
   void* y;            /* bf16 [batch, tokens, dim] */
@@ -378,6 +387,22 @@ typedef struct hdit_sd3_block_args {
 
 int64_t hdit_block_sd3_workspace_bytes(const hdit_sd3_block_args* args);
 int hdit_block_sd3(const hdit_sd3_block_args* args, void* stream);
+
+/* `count` (<= HDIT_BLOCK_MAX_MULTI) SD3 joint blocks that do not depend on each
+ * other (one width and head count; each with its own workspace, K/V buffer and
+ * outputs), run stage by stage with the launches of a stage merged: one
+ * normalise launch, one grouped q|k|v GEMM, one attention launch
+ * (hdit_attn_fwd_bf16_multi), ... for all of them.  These are the blocks (patch p,
+ * layer l) with p + l constant of a PipeFusion step: the loop of
+ * model_executor/pipelines/pipeline_stable_diffusion_3.py:1549-1644 runs patch after
+ * patch through models/transformers/transformer_sd3.py:107-152, but block l of
+ * patch p only needs block l of patch p - 1 and block l - 1 of its own patch, so
+ * the blocks on a diagonal are independent, and a patch-sized launch alone fills
+ * a fraction of the GPU.  Every output and K/V buffer is what `count`
+ * hdit_block_sd3 calls in array order produce, bit for bit.  Everything is
+ * validated before anything is enqueued. */
+#define HDIT_BLOCK_MAX_MULTI 4
+int hdit_block_sd3_multi(const hdit_sd3_block_args* args, int count, void* stream);
 
 /* The Flux double-stream block (diffusers FluxTransformerBlock, called at
  * models/transformers/transformer_flux.py:160-165) as one call.  Weights as in

@@ -118,3 +118,67 @@ def test_pipefusion_patch_graph_replay_from_restored_buffers(hdit):
         assert torch.equal(out, want), f"replay {i} differs from the eager result"
         step()  # eager passes in between move the buffers on
         torch.cuda.synchronize()
+
+
+def test_pipefusion_grouped_fronts_graph_replay(hdit):
+    """``forward_patches(num_streams=1)``: every front of independent (patch, layer) blocks is one merged
+    ``hdit_block_sd3_multi`` call on the caller's stream, so the whole PipeFusion step can be recorded into a graph.
+    Replays (from restored K/V buffers, with eager passes in between) reproduce the eager sequential pass."""
+    from hetu_dit_amd import synthetic, transformer
+    from hetu_dit_amd.cache_manager import get_cache_manager
+    from hetu_dit_amd.runtime_state import get_runtime_state
+
+    B, Ni, Nt, D, H, P, L = 2, 1024, 77, 256, 4, 4, 6
+    with torch.device(DEV):
+        stack = transformer.SD3TransformerBlocks(L, D, H, 64)
+    synthetic.init_module_(stack, 21)
+    e, t = dev_randn((B, Nt, D), 22), dev_randn((B, D), 23)
+    rs = get_runtime_state()
+    rs.set_token_patches([Ni // P * i for i in range(P + 1)])
+    rs.set_patched_mode(False)
+    stack(dev_randn((B, Ni, D), 24), e, t)  # fills the K/V buffers
+    rs.set_patched_mode(True)
+    xs = [dev_randn((B, Ni // P, D), 25 + p) for p in range(P)]
+
+    def sequential():
+        outs = []
+        for p in range(P):
+            outs.append(stack(xs[p], e, t))
+            rs.next_patch()
+        return outs
+
+    def grouped():
+        return stack.forward_patches(xs, e, t, num_streams=1)
+
+    def buffers():
+        return [b for entry in get_cache_manager().cache.values() for b in entry.tensors if b is not None]
+
+    grouped()
+    torch.cuda.synchronize()
+    saved = [b.clone() for b in buffers()]
+
+    def restore():
+        for b, s0 in zip(buffers(), saved):
+            b.copy_(s0)
+
+    want = [o.clone() for o in sequential()]
+    want_buf = [b.clone() for b in buffers()]
+    restore()
+    got = grouped()
+    torch.cuda.synchronize()
+    for p in range(P):
+        assert torch.equal(got[p], want[p]), f"eager grouped pass, patch {p}"
+    assert all(torch.equal(a, b) for a, b in zip(buffers(), want_buf))
+    restore()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = grouped()
+    for i in range(3):
+        restore()
+        graph.replay()
+        torch.cuda.synchronize()
+        for p in range(P):
+            assert torch.equal(outs[p], want[p]), f"replay {i}, patch {p}"
+        assert all(torch.equal(a, b) for a, b in zip(buffers(), want_buf)), f"replay {i}: K/V buffers"
+        sequential()  # eager passes in between move the buffers on
+        torch.cuda.synchronize()

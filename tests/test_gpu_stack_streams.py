@@ -63,7 +63,9 @@ def run_step_sequence(stack, B, Ni, Nt, D, P, entry_points, batch_streams, patch
                 seen.append(stack(xs[p], e, t).clone())
                 rs.next_patch()
         else:
-            seen += [o.clone() for o in stack.forward_patches(xs, e, t, num_streams=patch_streams)]
+            stack.group_fronts = patch_streams > 0  # -1: one stream, one call per block
+            seen += [o.clone() for o in stack.forward_patches(xs, e, t, num_streams=abs(patch_streams))]
+            stack.group_fronts = True
         assert rs.pipeline_patch_idx == 0
         torch.cuda.synchronize()
         seen += [b.clone() for b in buffers()]
@@ -83,7 +85,8 @@ def test_entry_point_blocks_lanes_and_overlapped_patches_give_the_same_bits(hdit
     forms = [
         ("entry points, one stream", True, 1, 0),
         ("entry points, batch lanes", True, 2, 0),
-        ("entry points, three batch lanes, patches on one stream through forward_patches", True, 3, 1),
+        ("entry points, three batch lanes, patches on one stream through forward_patches (merged fronts)", True, 3, 1),
+        ("entry points, patches on one stream through forward_patches, fronts not merged", True, 1, -1),
         ("entry points, batch lanes, patches on two streams", True, 2, 2),
         ("entry points, patches on three streams", True, 1, 3),
         ("kernel by kernel, patches on two streams", False, 1, 2),
