@@ -548,7 +548,7 @@ __global__ void __launch_bounds__(256, (HD == 64 ? 2 : 1)) attn_fwd_multi_kernel
 //   segment D   P.V steps 1, 2 of tile t (8)                                                      |  keys 48-63
 //
 // For the block to have no branch the reference of the online softmax is fixed after the first tile (its column
-// maxima plus a margin: p = 2^(s - m) may then grow to 2^PIPE_LIMIT_LOG2 and shrink to nothing without any loss
+// maxima plus a margin: p = 2^(s - m) may then grow to PIPE_LIMIT and shrink to nothing without any loss
 // of relative precision in fp32 / bf16): no maxima, no rescale in the loop.  A row whose sum ends at or above
 // the limit (infinity and NaN included) makes the whole workgroup run the tracked kernel above from the start.
 // K tiles are staged one tile ahead of V tiles (the scores run half a tile ahead of P.V), in rings of four LDS slots
@@ -690,14 +690,8 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles,
     dma_v(t + PIPE_LEAD - 1, wave_dst + PIPE_V_OFF + ((t + PIPE_LEAD - 1) & PIPE_MASK) * PIPE_TILE);
   };
   auto stage_end = [&]() {
-#ifdef PIPE_X_NODMA
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-#else
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(2 * NCH * (PIPE_LEAD - 2)));
-#endif
-#ifndef PIPE_X_NOBAR
     __syncthreads();
-#endif
   };
 
   // ---- prologue: flag, a zero V tile in the last slot (the lagged P.V of iteration 0 multiplies it by P = 0),
@@ -827,30 +821,14 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles,
   // exponentials, packs and row sums of the 16 keys of step u: accumulator entries 8*(u%2) .. of key block u/2
   auto chunk = [&](const f32x16 (&sc)[2], int u) __attribute__((always_inline)) {
     const int hh = u & 1;
-#ifdef PIPE_X_NOVALU
-    if (u >= 0) {
-#pragma unroll
-      for (int qb = 0; qb < 2; qb++) {
-        i32x4 pk;
-#pragma unroll
-        for (int e = 0; e < 4; e++) pk[e] = __float_as_int(sc[qb][hh * 8 + 2 * e]);
-        pf[qb][u] = __builtin_bit_cast(bf16x8, pk);
-      }
-      return;
-    }
-#endif
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
       i32x4 pk;
       float rs = l_run[qb];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-#ifdef PIPE_NOEXP
-        const float p0 = sc[qb][hh * 8 + 2 * e], p1 = sc[qb][hh * 8 + 2 * e + 1];
-#else
         const float p0 = __builtin_amdgcn_exp2f(sc[qb][hh * 8 + 2 * e]);
         const float p1 = __builtin_amdgcn_exp2f(sc[qb][hh * 8 + 2 * e + 1]);
-#endif
         const uint32_t pp = hdit::pack2(p0, p1);
         pk[e] = (int)pp;
         rs = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pp), ones2, rs, false);
@@ -908,10 +886,8 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles,
   };
   for (int t = 0; t < nb; t++) {
     const unsigned S = (unsigned)(t & PIPE_MASK) * PIPE_TILE, SN = (unsigned)((t + 1) & PIPE_MASK) * PIPE_TILE;  // ring slots of tiles t, t+1
-#ifndef PIPE_X_NODMA
     dma_k(t + PIPE_LEAD, wave_dst + (unsigned)((t + PIPE_LEAD) & PIPE_MASK) * PIPE_TILE);
     dma_v(t + PIPE_LEAD - 1, wave_dst + PIPE_V_OFF + (unsigned)((t + PIPE_LEAD - 1) & PIPE_MASK) * PIPE_TILE);
-#endif
     __builtin_amdgcn_sched_barrier(0);
     // fragment reads in the order the MFMAs consume them
     bf16x8 k1[KS], k0n[KS], vf[3][DB];
@@ -985,11 +961,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles,
 
   // ---- did the fixed reference hold?
   {
-#if defined(PIPE_X_NODMA) || defined(PIPE_X_NOBAR) || defined(PIPE_X_NOVALU)
-    const bool bad = false;  // timing experiments compute garbage
-#else
     const bool bad = !(l_run[0] < PIPE_LIMIT) || !(l_run[1] < PIPE_LIMIT);
-#endif
     if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) *flag = 1;
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
     __syncthreads();
