@@ -298,81 +298,96 @@ struct QkJobs {
   hdit_qknorm_job j[4];
 };
 
-template <int HD>
+// A thread works on chunk c of NH heads of one row (heads h, h + heads/NH, ...): the cos / sin values of the chunk,
+// which are the same for every head of a row and four times the bytes of the chunk itself, are fetched once per
+// NH head vectors, and NH loads are in flight per lane.
+template <int HD, int NH>
 __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkJobs jobs, int batch, int heads, float eps) {
   constexpr int LPH = HD / 8;  // lanes per head vector
   const hdit_qknorm_job& job = jobs.j[blockIdx.y];
-  const int64_t vec = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPH;
-  const int c = threadIdx.x % LPH;
-  const int64_t nvec = (int64_t)batch * job.seq * heads;
-  if (vec >= nvec) return;
-  const int h = (int)(vec % heads);
-  const int64_t bs = vec / heads;
-  const int s = (int)(bs % job.seq);
-  const int b = (int)(bs / job.seq);
-  __bf16* p = (__bf16*)job.x + b * job.stride_b + s * job.stride_s + h * job.stride_h + c * 8;
-  float f[8];
-  unpack8(*(const i32x4*)p, f);
-  if (job.norm_kind == 1) {
-    float q = 0.f;
+  const int hs = heads / NH;   // heads per pass over a row
+  const int per_row = hs * LPH;
+  const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = tid / per_row;
+  if (row >= (int64_t)batch * job.seq) return;
+  const int rem = (int)(tid - row * per_row);
+  const int h0 = rem / LPH;
+  const int c = rem % LPH;  // = threadIdx.x % LPH (per_row and 256 are multiples of LPH): a head's lanes sit side by side in one wave
+  const int s = (int)(row % job.seq);
+  const int b = (int)(row / job.seq);
+  __bf16* p = (__bf16*)job.x + b * job.stride_b + s * job.stride_s + h0 * job.stride_h + c * 8;
+  const int64_t hstep = (int64_t)hs * job.stride_h;
+  i32x4 raw[NH];
 #pragma unroll
-    for (int e = 0; e < 8; e++) q += f[e] * f[e];
-#pragma unroll
-    for (int off = LPH / 2; off > 0; off >>= 1) q += __shfl_xor(q, off, 64);
-    float r = rsqrtf(q * (1.0f / HD) + eps);
-#pragma unroll
-    for (int e = 0; e < 8; e++) f[e] *= r;
-  } else if (job.norm_kind == 2) {
-    float sm = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; e++) sm += f[e];
-#pragma unroll
-    for (int off = LPH / 2; off > 0; off >>= 1) sm += __shfl_xor(sm, off, 64);
-    float mean = sm * (1.0f / HD);
-    float q = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-      f[e] -= mean;
-      q += f[e] * f[e];
-    }
-#pragma unroll
-    for (int off = LPH / 2; off > 0; off >>= 1) q += __shfl_xor(q, off, 64);
-    float r = rsqrtf(q * (1.0f / HD) + eps);
-#pragma unroll
-    for (int e = 0; e < 8; e++) f[e] *= r;
-  }
-  if (job.norm_kind != 0) {
-    if (job.weight) {
-      float w[8];
-      unpack8(*(const i32x4*)((const __bf16*)job.weight + c * 8), w);
-#pragma unroll
-      for (int e = 0; e < 8; e++) f[e] *= w[e];
-    }
-    if (job.bias) {
-      float w[8];
-      unpack8(*(const i32x4*)((const __bf16*)job.bias + c * 8), w);
-#pragma unroll
-      for (int e = 0; e < 8; e++) f[e] += w[e];
-    }
-  }
+  for (int n = 0; n < NH; n++) raw[n] = *(const i32x4*)(p + n * hstep);
   const int rr = s - job.rope_row0;
-  if (job.cos_table && rr >= 0 && rr < job.rope_rows) {
+  const bool rope = job.cos_table && rr >= 0 && rr < job.rope_rows;
+  float cs[8], sn[8];
+  if (rope) {
     const float* cp = job.cos_table + (int64_t)rr * HD + c * 8;
     const float* sp = job.sin_table + (int64_t)rr * HD + c * 8;
-    f32x4 c0 = *(const f32x4*)cp, c1 = *(const f32x4*)(cp + 4);
-    f32x4 s0 = *(const f32x4*)sp, s1 = *(const f32x4*)(sp + 4);
-    float cs[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-    float sn[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-    float o[8];
+    const f32x4 c0 = *(const f32x4*)cp, c1 = *(const f32x4*)(cp + 4);
+    const f32x4 s0 = *(const f32x4*)sp, s1 = *(const f32x4*)(sp + 4);
 #pragma unroll
-    for (int e = 0; e < 8; e += 2) {
-      o[e] = f[e] * cs[e] - f[e + 1] * sn[e];
-      o[e + 1] = f[e + 1] * cs[e + 1] + f[e] * sn[e + 1];
-    }
-#pragma unroll
-    for (int e = 0; e < 8; e++) f[e] = o[e];
+    for (int e = 0; e < 4; e++) cs[e] = c0[e], cs[e + 4] = c1[e], sn[e] = s0[e], sn[e + 4] = s1[e];
   }
-  *(i32x4*)p = pack8(f);
+  float w[8], wb[8];
+  if (job.norm_kind != 0 && job.weight) unpack8(*(const i32x4*)((const __bf16*)job.weight + c * 8), w);
+  if (job.norm_kind != 0 && job.bias) unpack8(*(const i32x4*)((const __bf16*)job.bias + c * 8), wb);
+#pragma unroll
+  for (int n = 0; n < NH; n++) {
+    float f[8];
+    unpack8(raw[n], f);
+    if (job.norm_kind == 1) {
+      float q = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) q += f[e] * f[e];
+#pragma unroll
+      for (int off = LPH / 2; off > 0; off >>= 1) q += __shfl_xor(q, off, 64);
+      float r = rsqrtf(q * (1.0f / HD) + eps);
+#pragma unroll
+      for (int e = 0; e < 8; e++) f[e] *= r;
+    } else if (job.norm_kind == 2) {
+      float sm = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) sm += f[e];
+#pragma unroll
+      for (int off = LPH / 2; off > 0; off >>= 1) sm += __shfl_xor(sm, off, 64);
+      float mean = sm * (1.0f / HD);
+      float q = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        f[e] -= mean;
+        q += f[e] * f[e];
+      }
+#pragma unroll
+      for (int off = LPH / 2; off > 0; off >>= 1) q += __shfl_xor(q, off, 64);
+      float r = rsqrtf(q * (1.0f / HD) + eps);
+#pragma unroll
+      for (int e = 0; e < 8; e++) f[e] *= r;
+    }
+    if (job.norm_kind != 0) {
+      if (job.weight) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) f[e] *= w[e];
+      }
+      if (job.bias) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) f[e] += wb[e];
+      }
+    }
+    if (rope) {
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        o[e] = f[e] * cs[e] - f[e + 1] * sn[e];
+        o[e + 1] = f[e + 1] * cs[e + 1] + f[e] * sn[e + 1];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e++) f[e] = o[e];
+    }
+    *(i32x4*)(p + n * hstep) = pack8(f);
+  }
 }
 
 __global__ void __launch_bounds__(256) copy_rows_kernel(const __bf16* __restrict__ src, __bf16* __restrict__ dst,
@@ -534,13 +549,22 @@ extern "C" __attribute__((visibility("default"))) int hdit_qk_norm_rope(const hd
     if (nv > max_vec) max_vec = nv;
   }
   if (max_vec == 0) return HDIT_OK;
-  int lph = head_dim / 8;
-  int64_t threads = max_vec * lph;
+  const int lph = head_dim / 8;
+  const int nh = heads % 4 == 0 ? 4 : heads % 2 == 0 ? 2 : 1;  // head vectors per thread
+  const int64_t threads = max_vec / nh * lph;
   dim3 grid((unsigned)((threads + 255) / 256), count), block(256);
-  if (head_dim == 64)
-    hipLaunchKernelGGL(qk_norm_rope_kernel<64>, grid, block, 0, (hipStream_t)stream, tab, batch, heads, eps);
-  else
-    hipLaunchKernelGGL(qk_norm_rope_kernel<128>, grid, block, 0, (hipStream_t)stream, tab, batch, heads, eps);
+#define QK_LAUNCH(HD, NH) \
+  hipLaunchKernelGGL((qk_norm_rope_kernel<HD, NH>), grid, block, 0, (hipStream_t)stream, tab, batch, heads, eps)
+  if (head_dim == 64) {
+    if (nh == 4) QK_LAUNCH(64, 4);
+    else if (nh == 2) QK_LAUNCH(64, 2);
+    else QK_LAUNCH(64, 1);
+  } else {
+    if (nh == 4) QK_LAUNCH(128, 4);
+    else if (nh == 2) QK_LAUNCH(128, 2);
+    else QK_LAUNCH(128, 1);
+  }
+#undef QK_LAUNCH
   return hdit_host::check_launch("hdit_qk_norm_rope");
 }
 
