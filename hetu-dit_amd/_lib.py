@@ -15,7 +15,7 @@ HDIT_BLOCK_MAX_MULTI = 4
 HDIT_ATTN_MAX_MULTI = 4
 EPI_BIAS, EPI_BIAS_GELU, EPI_GATE_RESIDUAL = 0, 1, 2
 EPI_RESID_F32, EPI_OUT_F32 = 0x10, 0x20
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class GemmProblem(C.Structure):
@@ -95,6 +95,14 @@ class LnJob(C.Structure):
         ("tokens", C.c_int32),
         ("x_f32", C.c_int32),
         ("pad_", C.c_int32),
+        ("delta_y", C.c_void_p),
+        ("delta_gate", C.c_void_p),
+        ("x_out", C.c_void_p),
+        ("d_sb", C.c_int64),
+        ("d_st", C.c_int64),
+        ("gate_stride", C.c_int64),
+        ("xo_sb", C.c_int64),
+        ("xo_st", C.c_int64),
     ]
 
 
@@ -121,7 +129,10 @@ class Sd3BlockArgs(C.Structure):
     ] + [(n, C.c_int32) for n in (
         "batch", "n_img", "n_txt", "dim", "heads", "ff_dim", "temb_dim", "kv_rows", "kv_row0", "hidden_f32",
         "encoder_f32", "out_f32", "context_pre_only", "skip_text_output")] + [
-        ("text_kv", C.c_void_p), ("text_kv_mode", C.c_int32), ("fp8_attention", C.c_int32)]
+        ("text_kv", C.c_void_p), ("text_kv_mode", C.c_int32), ("fp8_attention", C.c_int32),
+        ("pending_img", C.c_void_p), ("pending_img_gate", C.c_void_p), ("pending_txt", C.c_void_p),
+        ("pending_txt_gate", C.c_void_p), ("pending_img_gate_stride", C.c_int64), ("pending_txt_gate_stride", C.c_int64),
+        ("defer_img", C.c_void_p), ("defer_txt", C.c_void_p), ("lazy_residual", C.c_int32), ("pad_", C.c_int32)]
 
 
 TEXT_KV_NONE, TEXT_KV_STORE, TEXT_KV_REUSE = 0, 1, 2

@@ -98,6 +98,13 @@ int validate(const hdit_sd3_block_args* a) {
   if (a->text_kv_mode == HDIT_TEXT_KV_REUSE && !a->skip_text_output) return HDIT_EINVAL;
   if (a->fp8_attention != 0 && a->fp8_attention != 1) return HDIT_EINVAL;
   if (a->fp8_attention && fp8_attention_bytes(a) < 0) return HDIT_EINVAL;
+  // updates owed to the fp32 streams, and the ones this block leaves to its successor
+  if (a->pending_img && (!a->hidden_f32 || !a->pending_img_gate || (((uintptr_t)a->pending_img) & 15))) return HDIT_EINVAL;
+  if (a->pending_txt && (!a->encoder_f32 || !a->pending_txt_gate || (((uintptr_t)a->pending_txt) & 15))) return HDIT_EINVAL;
+  if (a->lazy_residual != 0 && a->lazy_residual != 1) return HDIT_EINVAL;
+  if (a->defer_img && (!a->out_f32 || !a->modulation_img || (((uintptr_t)a->defer_img) & 15))) return HDIT_EINVAL;
+  if (a->defer_txt && (!text_out || !a->out_f32 || !a->modulation_txt || (((uintptr_t)a->defer_txt) & 15)))
+    return HDIT_EINVAL;
   return HDIT_OK;
 }
 
@@ -181,6 +188,30 @@ int plan_sd3(const hdit_sd3_block_args* a, Sd3Plan& pl) {
   jobs[1].x_sb = (int64_t)Nt * D, jobs[1].x_st = D, jobs[1].y_sb = (int64_t)Nt * D, jobs[1].y_st = D, jobs[1].mod_stride = mdt;
   jobs[1].batch = B, jobs[1].tokens = Nt, jobs[1].x_f32 = a->encoder_f32;
   pl.n_ln1 = reuse_text_kv ? 1 : 2;
+  // The fp32 streams inside the block.  A stream that arrives in fp32 takes its gated residuals in the
+  // normalisation that reads it next (hdit_ln_job.delta_y) instead of in the projection's epilogue: the out-projection
+  // and, with defer_img / defer_txt, the MLP's second projection write only bf16(A W^T + bias).  `st_*` is where the
+  // updated stream lives: the block's output when the MLP's residual is left to the next block (the output is then
+  // the stream after the attention residual), the workspace otherwise.
+  const bool lazy_img = a->lazy_residual && a->hidden_f32 != 0, lazy_txt = a->lazy_residual && a->encoder_f32 != 0 && text_out;
+  float* st_img = a->defer_img ? (float*)a->hidden_out : ws.x1_img;
+  float* st_txt = a->defer_txt ? (float*)a->encoder_out : ws.x1_txt;
+  const void* x0_img = a->hidden;
+  const void* x0_txt = a->encoder;
+  if (a->pending_img) {
+    jobs[0].delta_y = a->pending_img, jobs[0].delta_gate = a->pending_img_gate, jobs[0].gate_stride = a->pending_img_gate_stride;
+    jobs[0].d_sb = (int64_t)Ni * D, jobs[0].d_st = D;
+    jobs[0].x_out = st_img, jobs[0].xo_sb = (int64_t)Ni * D, jobs[0].xo_st = D;
+    x0_img = st_img;
+  }
+  if (a->pending_txt && !reuse_text_kv) {
+    jobs[1].delta_y = a->pending_txt, jobs[1].delta_gate = a->pending_txt_gate, jobs[1].gate_stride = a->pending_txt_gate_stride;
+    jobs[1].d_sb = (int64_t)Nt * D, jobs[1].d_st = D;
+    if (text_out) {  // a stream without an output (context_pre_only, patches after the first) is only normalised
+      jobs[1].x_out = st_txt, jobs[1].xo_sb = (int64_t)Nt * D, jobs[1].xo_st = D;
+      x0_txt = st_txt;
+    }
+  }
 
   // 3. q|k|v of both streams in one grouped launch.  With a stale K/V buffer the image stream's k|v rows go
   //    straight into rows [kv_row0, kv_row0 + n_img) of it, one problem per batch element.
@@ -261,11 +292,20 @@ int plan_sd3(const hdit_sd3_block_args* a, Sd3Plan& pl) {
     p.resid = resid, p.ldr = p.n, p.gate = gate, p.gate_stride = (int32_t)gate_stride, p.rows_per_batch = rows;
   };
   np = 0;
-  pl.outp[np] = problem(ws.o_img, D, w.to_out_w, w.to_out_b, ws.x1_img, D, B * Ni, D, D, 0);
-  gated(pl.outp[np++], a->hidden, a->hidden_f32, g_a, md, Ni, 1);
+  // the projected attention output of a lazily updated stream goes where that stream's q (|k|v) was: dead since the attention
+  if (lazy_img) {
+    pl.outp[np++] = problem(ws.o_img, D, w.to_out_w, w.to_out_b, ws.qkv_img, D, B * Ni, D, D, HDIT_EPI_BIAS);
+  } else {
+    pl.outp[np] = problem(ws.o_img, D, w.to_out_w, w.to_out_b, st_img, D, B * Ni, D, D, 0);
+    gated(pl.outp[np++], a->hidden, a->hidden_f32, g_a, md, Ni, 1);
+  }
   if (text_out) {
-    pl.outp[np] = problem(ws.o_txt, D, w.to_add_out_w, w.to_add_out_b, ws.x1_txt, D, B * Nt, D, D, 0);
-    gated(pl.outp[np++], a->encoder, a->encoder_f32, c_g_a, mdt, Nt, 1);
+    if (lazy_txt) {
+      pl.outp[np++] = problem(ws.o_txt, D, w.to_add_out_w, w.to_add_out_b, ws.qkv_txt, D, B * Nt, D, D, HDIT_EPI_BIAS);
+    } else {
+      pl.outp[np] = problem(ws.o_txt, D, w.to_add_out_w, w.to_add_out_b, st_txt, D, B * Nt, D, D, 0);
+      gated(pl.outp[np++], a->encoder, a->encoder_f32, c_g_a, mdt, Nt, 1);
+    }
   }
   pl.n_out = np;
 
@@ -273,14 +313,24 @@ int plan_sd3(const hdit_sd3_block_args* a, Sd3Plan& pl) {
   int nj = 0;
   jobs = pl.ln2;
   memset(pl.ln2, 0, sizeof(pl.ln2));
-  jobs[nj].x = ws.x1_img, jobs[nj].y = ws.n_img, jobs[nj].shift = sh_m, jobs[nj].scale = sc_m;
+  jobs[nj].x = lazy_img ? x0_img : st_img, jobs[nj].y = ws.n_img, jobs[nj].shift = sh_m, jobs[nj].scale = sc_m;
   jobs[nj].x_sb = (int64_t)Ni * D, jobs[nj].x_st = D, jobs[nj].y_sb = (int64_t)Ni * D, jobs[nj].y_st = D, jobs[nj].mod_stride = md;
   jobs[nj].batch = B, jobs[nj].tokens = Ni, jobs[nj].x_f32 = 1;
+  if (lazy_img) {
+    jobs[nj].delta_y = ws.qkv_img, jobs[nj].delta_gate = g_a, jobs[nj].gate_stride = md;
+    jobs[nj].d_sb = (int64_t)Ni * D, jobs[nj].d_st = D;
+    jobs[nj].x_out = st_img, jobs[nj].xo_sb = (int64_t)Ni * D, jobs[nj].xo_st = D;
+  }
   nj++;
   if (text_out) {
-    jobs[nj].x = ws.x1_txt, jobs[nj].y = ws.n_txt, jobs[nj].shift = c_sh_m, jobs[nj].scale = c_sc_m;
+    jobs[nj].x = lazy_txt ? x0_txt : st_txt, jobs[nj].y = ws.n_txt, jobs[nj].shift = c_sh_m, jobs[nj].scale = c_sc_m;
     jobs[nj].x_sb = (int64_t)Nt * D, jobs[nj].x_st = D, jobs[nj].y_sb = (int64_t)Nt * D, jobs[nj].y_st = D, jobs[nj].mod_stride = mdt;
     jobs[nj].batch = B, jobs[nj].tokens = Nt, jobs[nj].x_f32 = 1;
+    if (lazy_txt) {
+      jobs[nj].delta_y = ws.qkv_txt, jobs[nj].delta_gate = c_g_a, jobs[nj].gate_stride = mdt;
+      jobs[nj].d_sb = (int64_t)Nt * D, jobs[nj].d_st = D;
+      jobs[nj].x_out = st_txt, jobs[nj].xo_sb = (int64_t)Nt * D, jobs[nj].xo_st = D;
+    }
     nj++;
   }
   pl.n_ln2 = nj;
@@ -291,11 +341,19 @@ int plan_sd3(const hdit_sd3_block_args* a, Sd3Plan& pl) {
   if (text_out) pl.ff1[np++] = problem(ws.n_txt, D, w.ff_context_in_w, w.ff_context_in_b, ws.h_txt, F, B * Nt, F, D, HDIT_EPI_BIAS_GELU);
   pl.n_ff1 = np;
   np = 0;
-  pl.ff2[np] = problem(ws.h_img, F, w.ff_out_w, w.ff_out_b, a->hidden_out, D, B * Ni, D, F, 0);
-  gated(pl.ff2[np++], ws.x1_img, 1, g_m, md, Ni, a->out_f32);
+  if (a->defer_img) {
+    pl.ff2[np++] = problem(ws.h_img, F, w.ff_out_w, w.ff_out_b, a->defer_img, D, B * Ni, D, F, HDIT_EPI_BIAS);
+  } else {
+    pl.ff2[np] = problem(ws.h_img, F, w.ff_out_w, w.ff_out_b, a->hidden_out, D, B * Ni, D, F, 0);
+    gated(pl.ff2[np++], st_img, 1, g_m, md, Ni, a->out_f32);
+  }
   if (text_out) {
-    pl.ff2[np] = problem(ws.h_txt, F, w.ff_context_out_w, w.ff_context_out_b, a->encoder_out, D, B * Nt, D, F, 0);
-    gated(pl.ff2[np++], ws.x1_txt, 1, c_g_m, mdt, Nt, a->out_f32);
+    if (a->defer_txt) {
+      pl.ff2[np++] = problem(ws.h_txt, F, w.ff_context_out_w, w.ff_context_out_b, a->defer_txt, D, B * Nt, D, F, HDIT_EPI_BIAS);
+    } else {
+      pl.ff2[np] = problem(ws.h_txt, F, w.ff_context_out_w, w.ff_context_out_b, a->encoder_out, D, B * Nt, D, F, 0);
+      gated(pl.ff2[np++], st_txt, 1, c_g_m, mdt, Nt, a->out_f32);
+    }
   }
   pl.n_ff2 = np;
   return HDIT_OK;

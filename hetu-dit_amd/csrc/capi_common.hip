@@ -37,7 +37,7 @@ int num_cus() {
 }
 }  // namespace hdit_host
 
-extern "C" __attribute__((visibility("default"))) int hdit_abi_version(void) { return 4; }
+extern "C" __attribute__((visibility("default"))) int hdit_abi_version(void) { return 5; }
 extern "C" __attribute__((visibility("default"))) const char* hdit_last_error(void) { return g_err; }
 
 namespace {

@@ -1,6 +1,8 @@
 // Bandwidth-bound glue kernels for gfx950: every tensor is touched once, with
 // 16-byte accesses laid out so that a wave reads/writes contiguous 1 KiB runs,
 // statistics in fp32, wave64 cross-lane reductions.
+#include <cstring>
+
 #include "hdit_common.h"
 
 namespace {
@@ -31,11 +33,16 @@ struct LnJobs {
 // takes 16.6 us this way against 18.5 us, the time of a plain copy of the same bytes.
 // Rows of up to 64 floats per lane are held to 128 registers (four waves per SIMD): left alone, the compiler hoists
 // every LDS read of the modulation above the reductions and the wide kernels drop to three waves per SIMD.
-template <int NCH, bool XF32>
+//
+// DELTA (fp32 stream only): a job may carry a pending update of the stream, x' = x + gate[b, :] * delta_y (the gated
+// residual of the projection that ran before this normalisation, whose GEMM wrote only delta_y = bf16(A.W^T + bias)).
+// It is applied here, in the registers the row is read into anyway, and x' is written back as the new stream: the
+// GEMM's epilogue then has no read-modify-write of the fp32 stream, which four waves per CU cannot keep HBM busy with.
+template <int NCH, bool XF32, bool DELTA>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NCH * (XF32 ? 4 : 8) <= 64 ? 4 : 2)))
-ln_modulate_kernel(const LnJobs jobs, const __bf16* __restrict__ lw,
-                                                          const __bf16* __restrict__ lb, int dim, float eps) {
-  extern __shared__ __attribute__((aligned(16))) float lmod[];  // scale[dim] | shift[dim] of this batch element
+ln_modulate_kernel(const LnJobs jobs, const __bf16* __restrict__ lw, const __bf16* __restrict__ lb, int dim, float eps) {
+  static_assert(XF32 || !DELTA, "the pending update exists for the fp32 stream only");
+  extern __shared__ __attribute__((aligned(16))) float lmod[];  // scale[dim] | shift[dim] (| gate[dim]) of this batch element
   // which job this workgroup belongs to (a launch normalises up to HDIT_LN_MAX_JOBS tensors, e.g. the
   // image and the text stream of a joint block)
   int ji = 0;
@@ -52,25 +59,41 @@ ln_modulate_kernel(const LnJobs jobs, const __bf16* __restrict__ lw,
   const bool live = t < job.tokens;
   const float* __restrict__ shift = job.shift ? job.shift + (int64_t)b * job.mod_stride : nullptr;
   const float* __restrict__ scale = job.scale ? job.scale + (int64_t)b * job.mod_stride : nullptr;
+  const bool has_delta = DELTA && job.delta_y != nullptr;
+  const float* __restrict__ dgate = has_delta ? job.delta_gate + (int64_t)b * job.gate_stride : nullptr;
   const int nchunks = dim / EPC;
   const int nvec = dim >> 2;  // f32x4 pieces of a modulation vector
   constexpr int MV = (NCH * 64 * (EPC / 4) + 255) / 256;
-  f32x4 mreg[2][MV];
+  f32x4 mreg[DELTA ? 3 : 2][MV];
 #pragma unroll
   for (int k = 0; k < MV; k++) {
     const int i = (int)threadIdx.x + k * 256;
     if (i < nvec) {
       if (scale) mreg[0][k] = *(const f32x4*)(scale + i * 4);
       if (shift) mreg[1][k] = *(const f32x4*)(shift + i * 4);
+      if constexpr (DELTA) {
+        if (has_delta) mreg[2][k] = *(const f32x4*)(dgate + i * 4);
+      }
     }
   }
   i32x4 raw[NCH];
+  i32x2 draw[DELTA ? NCH : 1];
   if (live) {
     const unsigned char* xr = (const unsigned char*)job.x + ((int64_t)b * job.x_sb + (int64_t)t * job.x_st) * XB;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
       const int c = lane + i * 64;
       if (c < nchunks) raw[i] = *(const i32x4*)(xr + c * 16);
+    }
+    if constexpr (DELTA) {
+      if (has_delta) {
+        const __bf16* dr = (const __bf16*)job.delta_y + (int64_t)b * job.d_sb + (int64_t)t * job.d_st;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+          const int c = lane + i * 64;
+          if (c < nchunks) draw[i] = *(const i32x2*)(dr + c * 4);
+        }
+      }
     }
   }
 #pragma unroll
@@ -79,10 +102,34 @@ ln_modulate_kernel(const LnJobs jobs, const __bf16* __restrict__ lw,
     if (i < nvec) {
       if (scale) *(f32x4*)(lmod + i * 4) = mreg[0][k];
       if (shift) *(f32x4*)(lmod + dim + i * 4) = mreg[1][k];
+      if constexpr (DELTA) {
+        if (has_delta) *(f32x4*)(lmod + 2 * dim + i * 4) = mreg[2][k];
+      }
     }
   }
   __syncthreads();
   if (!live) return;
+  if constexpr (DELTA) {
+    if (has_delta) {
+      // x' = fma(gate, delta, x), the operation of the GEMM's gated-residual epilogue, bit for bit
+      float* xo = job.x_out ? (float*)job.x_out + (int64_t)b * job.xo_sb + (int64_t)t * job.xo_st : nullptr;
+#pragma unroll
+      for (int i = 0; i < NCH; i++) {
+        const int c = lane + i * 64;
+        if (c < nchunks) {
+          const f32x4 g = *(const f32x4*)(lmod + 2 * dim + c * 4);
+          const float d[4] = {__uint_as_float((uint32_t)draw[i][0] << 16), __uint_as_float((uint32_t)draw[i][0] & 0xffff0000u),
+                              __uint_as_float((uint32_t)draw[i][1] << 16), __uint_as_float((uint32_t)draw[i][1] & 0xffff0000u)};
+          f32x4 v;
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(g[e], d[e], __int_as_float(raw[i][e]));
+#pragma unroll
+          for (int e = 0; e < 4; e++) raw[i][e] = __float_as_int(v[e]);
+          if (xo) *(f32x4*)(xo + c * 4) = v;
+        }
+      }
+    }
+  }
   // EPC bf16 values (an affine weight or bias) at element offset c * EPC
   auto load_bf16 = [&](const __bf16* p, int c, float (&w)[EPC]) {
     if constexpr (XF32) {
@@ -419,6 +466,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate_jo
     LnJobs tab;
     tab.count = 0;
     int64_t blocks = 0;
+    bool any_delta = false;
     for (int i = 0; i < count; i++) {
       const hdit_ln_job& j = jobs[i];
       if (j.batch < 0 || j.tokens < 0) return HDIT_EINVAL;
@@ -428,6 +476,15 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate_jo
       if (!j.x || !j.y) return HDIT_EINVAL;
       if (j.x_sb % 8 || j.x_st % 8 || j.y_sb % 8 || j.y_st % 8 || j.mod_stride % 4) return HDIT_EINVAL;
       if (!aligned16(j.x) || !aligned16(j.y) || !aligned16(j.shift) || !aligned16(j.scale)) return HDIT_EINVAL;
+      if (j.delta_y) {
+        // a pending update of the fp32 stream: x' = x + gate * delta_y, optionally written back
+        if (!f32 || !j.delta_gate) return HDIT_EINVAL;
+        if (j.d_sb % 8 || j.d_st % 8 || j.gate_stride % 4 || j.xo_sb % 4 || j.xo_st % 4) return HDIT_EINVAL;
+        if (!aligned16(j.delta_y) || !aligned16(j.delta_gate) || !aligned16(j.x_out)) return HDIT_EINVAL;
+        any_delta = true;
+      } else if (j.x_out || j.delta_gate) {
+        return HDIT_EINVAL;
+      }
       tab.block_start[tab.count] = (int)blocks;
       tab.j[tab.count++] = j;
       blocks += (int64_t)j.batch * ((j.tokens + 3) / 4);  // four rows of one batch element per workgroup
@@ -438,15 +495,18 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate_jo
     dim3 grid((unsigned)blocks), block(256);
     if (f32 && dim > 4096) return HDIT_EUNSUPPORTED;  // a row of the fp32 stream is held in registers: 16 chunks per lane
     const int nch = (dim / (f32 ? 4 : 8) + 63) / 64;
-    const size_t lds_bytes = (size_t)dim * 8;  // scale | shift of one batch element, fp32
+    const size_t lds_bytes = (size_t)dim * (any_delta ? 12 : 8);  // scale | shift (| gate) of one batch element, fp32
 #define LN_LAUNCH(N)                                                                                                  \
   do {                                                                                                                \
-    if (f32)                                                                                                          \
-      hipLaunchKernelGGL((ln_modulate_kernel<N, true>), grid, block, lds_bytes, s, tab, (const __bf16*)ln_weight,             \
-                         (const __bf16*)ln_bias, dim, eps);                                                           \
+    if (f32 && any_delta)                                                                                             \
+      hipLaunchKernelGGL((ln_modulate_kernel<N, true, true>), grid, block, lds_bytes, s, tab,                         \
+                         (const __bf16*)ln_weight, (const __bf16*)ln_bias, dim, eps);                                 \
+    else if (f32)                                                                                                     \
+      hipLaunchKernelGGL((ln_modulate_kernel<N, true, false>), grid, block, lds_bytes, s, tab,                        \
+                         (const __bf16*)ln_weight, (const __bf16*)ln_bias, dim, eps);                                 \
     else                                                                                                              \
-      hipLaunchKernelGGL((ln_modulate_kernel<N, false>), grid, block, lds_bytes, s, tab, (const __bf16*)ln_weight,            \
-                         (const __bf16*)ln_bias, dim, eps);                                                           \
+      hipLaunchKernelGGL((ln_modulate_kernel<N, false, false>), grid, block, lds_bytes, s, tab,                       \
+                         (const __bf16*)ln_weight, (const __bf16*)ln_bias, dim, eps);                                 \
   } while (0)
     if (nch <= 1) LN_LAUNCH(1);
     else if (nch <= 2) LN_LAUNCH(2);
@@ -468,6 +528,7 @@ extern "C" __attribute__((visibility("default"))) int hdit_layernorm_modulate(co
                                        int64_t x_sb, int64_t x_st, int64_t y_sb, int64_t y_st, int64_t mod_stride,
                                        float eps, void* stream) {
   hdit_ln_job j;
+  memset(&j, 0, sizeof(j));
   j.x = x, j.y = y, j.shift = shift, j.scale = scale;
   j.batch = batch, j.tokens = tokens;
   j.x_f32 = 0, j.pad_ = 0;

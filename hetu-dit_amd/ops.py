@@ -364,16 +364,21 @@ class Sd3BlockCall:
     def __call__(self, *args, **kwargs):
         """Fill the argument struct (``prepare``) and launch the block on the current stream."""
         encoder_out, hidden_out, ws = self.prepare(*args, **kwargs)
-        check(_lib.lib().hdit_block_sd3(C.byref(self.args), _stream()), "hdit_block_sd3")
+        self.launch()
         # stream-ordered reuse: the workspace may be freed as soon as the launches are queued
         del ws
         return encoder_out, hidden_out
+
+    def launch(self):
+        """Enqueue the block described by ``self.args`` (filled by ``prepare``) on the current stream."""
+        check(_lib.lib().hdit_block_sd3(C.byref(self.args), _stream()), "hdit_block_sd3")
 
     def prepare(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
                 out_dtype=bf16, skip_text_output: bool = False, kv_buffer: Optional[torch.Tensor] = None,
                 kv_row0: int = 0, modulation_img: Optional[int] = None, modulation_txt: Optional[int] = None,
                 hidden_out: Optional[torch.Tensor] = None, text_kv: Optional[torch.Tensor] = None,
-                text_kv_mode: int = _lib.TEXT_KV_NONE):
+                text_kv_mode: int = _lib.TEXT_KV_NONE, pending_img=None, pending_txt=None, defer: bool = False,
+                lazy: bool = False):
         """Fills ``self.args`` for one call without launching; returns ``(encoder_out_or_None, hidden_out,
         workspace tensor)`` -- the caller launches (``hdit_block_sd3`` or, with other blocks' structs,
         ``sd3_blocks_launch``) and keeps the workspace alive until then.
@@ -382,7 +387,12 @@ class Sd3BlockCall:
         block for this ``temb`` (the caller keeps their tensor alive), or None to have the call compute them.
         ``hidden_out``: a contiguous [batch, n_img, dim] tensor of ``out_dtype`` to write the image stream to.
         ``text_kv`` / ``text_kv_mode``: bf16 [batch, n_txt, 2 dim] buffer of the text stream's keys | values that
-        this call fills (``TEXT_KV_STORE``) or, with ``skip_text_output``, takes as they are (``TEXT_KV_REUSE``)."""
+        this call fills (``TEXT_KV_STORE``) or, with ``skip_text_output``, takes as they are (``TEXT_KV_REUSE``).
+        ``pending_img`` / ``pending_txt``: ``(y, gate address, gate batch stride)`` -- an update ``gate * y`` the
+        previous block of the chain left owing to the f32 stream it hands over; this block's first normalisation
+        adds it.  ``defer`` (f32 output, modulation given): the MLP residuals of this block are left owing in the
+        same way; ``self.deferred`` is then ``(pending_img, pending_txt_or_None)`` for the next block.  ``lazy``:
+        inside the block the attention residual of an f32 stream is added by norm2 rather than by the out-projection."""
         a = self.args
         B, Ni, D = hidden_states.shape
         Nt = encoder_hidden_states.shape[1]
@@ -418,6 +428,28 @@ class Sd3BlockCall:
             a.text_kv, a.text_kv_mode = text_kv.data_ptr(), text_kv_mode
         else:
             a.text_kv, a.text_kv_mode = None, _lib.TEXT_KV_NONE
+        for name, pend, rows, f32 in (("img", pending_img, Ni, a.hidden_f32), ("txt", pending_txt, Nt, a.encoder_f32)):
+            if pend is None:
+                setattr(a, f"pending_{name}", None), setattr(a, f"pending_{name}_gate", None)
+                setattr(a, f"pending_{name}_gate_stride", 0)
+                continue
+            y, gate, stride = pend
+            if not f32 or y.dtype != bf16 or tuple(y.shape) != (B, rows, D) or not y.is_contiguous():
+                raise ValueError("a pending update is a contiguous bf16 tensor of the shape of its f32 stream")
+            setattr(a, f"pending_{name}", y.data_ptr()), setattr(a, f"pending_{name}_gate", gate)
+            setattr(a, f"pending_{name}_gate_stride", stride)
+        self._pending = (pending_img, pending_txt)
+        self.deferred = None
+        a.defer_img = a.defer_txt = None
+        a.lazy_residual = int(bool(defer or lazy))
+        if defer:
+            if out_dtype != torch.float32 or modulation_img is None or (text_out and modulation_txt is None):
+                raise ValueError("residuals can only be left to the next block on an f32 stream with the modulation given")
+            d_img = torch.empty(B, Ni, D, dtype=bf16, device=dev)
+            d_txt = torch.empty(B, Nt, D, dtype=bf16, device=dev) if text_out else None
+            a.defer_img, a.defer_txt = d_img.data_ptr(), (d_txt.data_ptr() if text_out else None)
+            # gate_mlp is the sixth chunk of a stream's modulation
+            self.deferred = ((d_img, modulation_img + 4 * 5 * D, 6 * D), (d_txt, modulation_txt + 4 * 5 * D, 6 * D) if text_out else None)
         lib = _lib.lib()
         key = (B, Ni, Nt, bool(skip_text_output), a.kv_rows, text_kv_mode, a.fp8_attention)
         nbytes = self._ws_bytes.get(key)
@@ -690,8 +722,9 @@ def layernorm_modulate(x, shift=None, scale=None, eps: float = 1e-6, ln_weight=N
 def layernorm_modulate_many(items, eps: float = 1e-6, ln_weight=None, ln_bias=None):
     """LayerNorm + modulate of several tensors of one width in one launch.
 
-    ``items`` is a list of ``(x, shift, scale)`` or ``(x, shift, scale, out)``;
-    returns the outputs in order."""
+    ``items`` is a list of ``(x, shift, scale)``, ``(x, shift, scale, out)`` or ``(x, shift, scale, out, delta)``
+    with ``delta = (y bf16 like x, gate f32 [batch, dim], x_out f32 like x or None)``: the f32 stream ``x`` is
+    first updated to ``x + gate * y`` (and written to ``x_out``, which may be ``x``).  Returns the outputs in order."""
     jobs = (_lib.LnJob * len(items))()
     outs, keep, D0, nbytes = [], [], None, 0.0
     for i, it in enumerate(items):
@@ -716,6 +749,23 @@ def layernorm_modulate_many(items, eps: float = 1e-6, ln_weight=None, ln_bias=No
         j.x, j.y, j.shift, j.scale = x.data_ptr(), out.data_ptr(), sh, sc
         j.x_sb, j.x_st, j.y_sb, j.y_st, j.mod_stride = xsb, xst, ysb, yst, (st1 or st2 or 0)
         j.batch, j.tokens, j.x_f32 = B, T, int(x_f32)
+        if len(it) > 4 and it[4] is not None:
+            dy, gate, x_out = it[4]
+            if not x_f32:
+                raise ValueError("a pending update needs the f32 stream")
+            Bd, Td, Dd, dsb, dst = _as3d(dy, "delta y")
+            g, gst = _mod(gate, B, D, "delta gate")
+            if (Bd, Td, Dd) != (B, T, D):
+                raise ValueError("delta y must have the shape of x")
+            j.delta_y, j.delta_gate, j.d_sb, j.d_st, j.gate_stride = dy.data_ptr(), g, dsb, dst, gst
+            if x_out is not None:
+                Bx, Tx, Dx, xosb, xost = _as3d(x_out, "x_out", torch.float32)
+                if (Bx, Tx, Dx) != (B, T, D):
+                    raise ValueError("x_out must have the shape of x")
+                j.x_out, j.xo_sb, j.xo_st = x_out.data_ptr(), xosb, xost
+                nbytes += 4.0 * B * T * D
+            nbytes += 2.0 * B * T * D
+            keep.append((dy, gate, x_out))
         outs.append(out)
         keep.append((x, shift, scale, out))
         nbytes += (6.0 if x_f32 else 4.0) * B * T * D

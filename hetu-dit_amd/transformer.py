@@ -9,6 +9,7 @@ blocks" with each model family's call convention and patch-mode rules.
   ``cat([text, image])``, single blocks on the joint sequence, split.
 * CogVideoX (``cogvideox_transformer_3d.py:99-127``).
 """
+import os
 import warnings
 from typing import List, Optional, Tuple
 
@@ -37,6 +38,21 @@ def side_streams(device: torch.device, count: int) -> List["torch.cuda.Stream"]:
     while len(have) < min(count, MAX_SIDE_STREAMS):
         have.append(torch.cuda.Stream(device=device))  # default priority, like the caller's stream
     return have[: min(count, MAX_SIDE_STREAMS)]
+
+
+class _Chain:
+    """What one chain of SD3 blocks (a full pass, one batch lane, one pipeline patch) carries from a block to the
+    next besides the streams: the gated MLP residual the block did not add itself.  ``img`` / ``txt``: ``(y bf16
+    [batch, rows, dim], address of the f32 gate, its batch stride)`` or None -- the stream a block hands over is
+    then short of ``gate * y``, and the next block's first normalisation, which reads the stream anyway, adds it
+    (``hdit_sd3_block_args.pending_*`` / ``defer_*``).  The GEMM that produced ``y`` is spared the
+    read-modify-write of the f32 stream in its epilogue."""
+
+    __slots__ = ("img", "txt")
+
+    def __init__(self):
+        self.img = None
+        self.txt = None
 
 
 class SD3TransformerBlocks(nn.Module):
@@ -72,6 +88,11 @@ class SD3TransformerBlocks(nn.Module):
         self.batch_streams = 2
         self.reuse_text_kv = True  # patch mode: later patches take the text keys / values the first patch projected
         self.group_fronts = True   # forward_patches on one stream: one merged call per front of independent blocks
+        # entry-point passes: a block leaves its MLP residual to the next block's norm1 (HDIT_DEFER_RESIDUALS=0: fused
+        # into the GEMM epilogue as in a block called on its own)
+        self.defer_residuals = os.environ.get("HDIT_DEFER_RESIDUALS", "1") != "0"
+        # patch mode: the pending text update that goes with encoder_hidden_states_cache[i]
+        self._text_pending: List[Optional[tuple]] = [None] * num_layers
         self._block_calls: Optional[List[ops.Sd3BlockCall]] = None
         # per block: (k|v buffer of the text stream, the text states and temb it was projected from, with their
         # in-place modification counters) -- patch mode
@@ -101,8 +122,10 @@ class SD3TransformerBlocks(nn.Module):
 
     def _run_block(self, i: int, calls, mods, hidden, encoder, temb, skip_text_output: bool = False,
                    kv_buffer=None, kv_row0: int = 0, batch0: int = 0, hidden_out=None, patch: Optional[int] = None,
-                   defer: Optional[list] = None):
-        """Block i on the current stream: ``(encoder_out_or_None, hidden_out)``.  ``batch0``: index of the
+                   defer: Optional[list] = None, chain: Optional["_Chain"] = None):
+        """Block i on the current stream: ``(encoder_out_or_None, hidden_out)``.  ``chain``: the gated residuals
+        the previous block of this chain of blocks left to this one's first normalisation (``_Chain``); updated
+        with what this block leaves to the next.  ``batch0``: index of the
         first batch element of ``hidden`` within the ``temb`` the modulation ``mods`` was computed for.
         ``defer``: a list -- the call is prepared and appended to it instead of launched (``_launch_front``).
         ``patch``: index of the pipeline patch in patch mode.  The later patches of a step are fed the text states
@@ -138,11 +161,25 @@ class SD3TransformerBlocks(nn.Module):
             modulation_txt=base + 4 * (offsets[block.norm1_context] + batch0 * rows_txt),
             hidden_out=hidden_out, text_kv=text_kv, text_kv_mode=text_kv_mode,
         )
-        if defer is None:
-            return calls[i](hidden, encoder, temb, **kwargs)
-        # the struct is filled, the launch is the caller's (merged with the other blocks of its front)
+        if chain is not None:
+            kwargs["pending_img"] = chain.img
+            kwargs["pending_txt"] = chain.txt
+            # every block but the last leaves its MLP residuals to the next block's first normalisation
+            kwargs["defer"] = self.defer_residuals and i + 1 < len(self.transformer_blocks) \
+                and block.stream_dtype == torch.float32
+            kwargs["lazy"] = self.defer_residuals
         encoder_out, hidden_new, ws = calls[i].prepare(hidden, encoder, temb, **kwargs)
-        defer.append((calls[i], ws))
+        if chain is not None:
+            left = calls[i].deferred
+            chain.img = left[0] if left is not None else None
+            if not skip_text_output:  # a call that drops its text output leaves the text stream's state alone
+                chain.txt = left[1] if left is not None else None
+        if defer is None:
+            calls[i].launch()
+            del ws  # stream-ordered reuse: the workspace may be freed as soon as the launches are queued
+        else:
+            # the struct is filled, the launch is the caller's (merged with the other blocks of its front)
+            defer.append((calls[i], ws))
         return encoder_out, hidden_new
 
     def _kv_buffer(self, i: int, hidden: torch.Tensor):
@@ -181,20 +218,26 @@ class SD3TransformerBlocks(nn.Module):
             lanes = min(self.batch_streams, hidden_states.shape[0])
             if not rs.patch_mode and lanes > 1 and not torch.cuda.is_current_stream_capturing():
                 return self._forward_batch_lanes(calls, mods, hidden_states, encoder_hidden_states, temb, lanes)
+        chain = _Chain() if calls is not None else None
         for i in range(len(self.transformer_blocks)):
             kv = self._kv_buffer(i, hidden_states) if calls is not None else (None, 0)
             if rs.patch_mode and rs.pipeline_patch_idx == 0:
                 self.encoder_hidden_states_cache[i] = encoder_hidden_states
+                self._text_pending[i] = chain.txt if chain is not None else None
                 encoder_hidden_states, hidden_states = self._run_block(
-                    i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1], patch=0)
+                    i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1], patch=0,
+                    chain=chain)
             elif rs.patch_mode:
                 # the text output of these calls is dropped: the block does not compute it
+                if chain is not None:
+                    chain.txt = self._text_pending[i]
                 _, hidden_states = self._run_block(
                     i, calls, mods, hidden_states, self.encoder_hidden_states_cache[i], temb, skip_text_output=True,
-                    kv_buffer=kv[0], kv_row0=kv[1], patch=rs.pipeline_patch_idx)
+                    kv_buffer=kv[0], kv_row0=kv[1], patch=rs.pipeline_patch_idx, chain=chain)
             else:
                 encoder_hidden_states, hidden_states = self._run_block(
-                    i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1])
+                    i, calls, mods, hidden_states, encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1],
+                    chain=chain)
         return hidden_states
 
     def _forward_batch_lanes(self, calls, mods, hidden_states, encoder_hidden_states, temb, lanes: int):
@@ -213,14 +256,17 @@ class SD3TransformerBlocks(nn.Module):
         for k, s in enumerate(streams):
             s.wait_event(start)
             b0, b1 = bounds[k], bounds[k + 1]
-            state.append([hidden_states[b0:b1], encoder_hidden_states[b0:b1], temb[b0:b1]])
+            # no residual chain here: with a second chain of blocks in flight the read-modify-write of a fused
+            # gated epilogue runs under the other chain's MFMAs, and moving it into the normalisation kernels
+            # only lengthens those (measured: 19.85 ms fused, 20.18 ms deferred for the SD3 step on two streams)
+            state.append([hidden_states[b0:b1], encoder_hidden_states[b0:b1], temb[b0:b1], None])
         for i in range(L):
             for k, s in enumerate(streams):
                 b0, b1 = bounds[k], bounds[k + 1]
-                h, e, t = state[k]
+                h, e, t, chain = state[k]
                 with torch.cuda.stream(s):
                     e, h = self._run_block(i, calls, mods, h, e, t, kv_buffer=kv[i][b0:b1], batch0=b0,
-                                           hidden_out=out[b0:b1] if i == L - 1 else None)
+                                           hidden_out=out[b0:b1] if i == L - 1 else None, chain=chain)
                 state[k][0], state[k][1] = h, e
         for s in streams:
             done = torch.cuda.Event()
@@ -276,6 +322,8 @@ class SD3TransformerBlocks(nn.Module):
                 s.wait_event(start)
         events = self._patch_events
         cache = self.encoder_hidden_states_cache
+        # residual chains only where the patches run one after the other (see _forward_batch_lanes)
+        chains = [_Chain() for _ in range(P)] if calls is not None and len(streams) == 1 else [None] * P
         try:
             for front in range(L + P - 1):  # launches are issued along the diagonal, the order they can start in
                 for p in range(P):
@@ -290,13 +338,16 @@ class SD3TransformerBlocks(nn.Module):
                         kv = self._kv_buffer(i, hidden[p]) if calls is not None else (None, 0)
                         if p == 0:
                             cache[i] = encoder_hidden_states
+                            self._text_pending[i] = chains[0].txt if chains[0] is not None else None
                             encoder_hidden_states, hidden[0] = self._run_block(
                                 i, calls, mods, hidden[0], encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1],
-                                patch=0)
+                                patch=0, chain=chains[0])
                         else:
+                            if chains[p] is not None:
+                                chains[p].txt = self._text_pending[i]
                             _, hidden[p] = self._run_block(
                                 i, calls, mods, hidden[p], cache[i], temb, skip_text_output=True,
-                                kv_buffer=kv[0], kv_row0=kv[1], patch=p)
+                                kv_buffer=kv[0], kv_row0=kv[1], patch=p, chain=chains[p])
                         if P > 1 and len(streams) > 1:
                             done = events.get((p, i))
                             if done is None:
@@ -323,6 +374,7 @@ class SD3TransformerBlocks(nn.Module):
         rs = get_runtime_state()
         P, L = len(hidden), len(self.transformer_blocks)
         cache = self.encoder_hidden_states_cache
+        chains = [_Chain() for _ in range(P)]
         try:
             for front in range(L + P - 1):
                 group = []
@@ -334,13 +386,15 @@ class SD3TransformerBlocks(nn.Module):
                     kv = self._kv_buffer(i, hidden[p])
                     if p == 0:
                         cache[i] = encoder_hidden_states
+                        self._text_pending[i] = chains[0].txt
                         encoder_hidden_states, hidden[0] = self._run_block(
                             i, calls, mods, hidden[0], encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1], patch=0,
-                            defer=group)
+                            defer=group, chain=chains[0])
                     else:
+                        chains[p].txt = self._text_pending[i]
                         _, hidden[p] = self._run_block(
                             i, calls, mods, hidden[p], cache[i], temb, skip_text_output=True, kv_buffer=kv[0],
-                            kv_row0=kv[1], patch=p, defer=group)
+                            kv_row0=kv[1], patch=p, defer=group, chain=chains[p])
                 ops.sd3_blocks_launch([c for c, _ in group])
                 del group  # the workspaces: stream-ordered reuse once the launches are queued
         finally:

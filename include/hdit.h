@@ -209,6 +209,17 @@ typedef struct hdit_ln_job {
   int32_t batch, tokens;
   int32_t x_f32; /* != 0: x is f32 [batch, tokens, dim] (strides in f32 elements): the fp32 residual stream */
   int32_t pad_;
+  /* Optional pending update of the fp32 stream (x_f32 only; all NULL / 0 otherwise), applied before the
+   * statistics: x' = x + delta_gate[b, :] * delta_y -- the gated residual `hidden_states + gate * attn_output`
+   * (or `+ gate * ff_output`) of the blocks cited above, when the projection's GEMM wrote only
+   * delta_y = bf16(A W^T + bias) and left the addition to the normalisation that reads the stream next.
+   * delta_y bf16 [batch, tokens, dim] (strides d_sb, d_st), delta_gate f32 (batch stride gate_stride);
+   * x_out != NULL: x' is written there as f32 (strides xo_sb, xo_st; may be x itself).  The result is
+   * fma(gate, delta_y, x) per element, what HDIT_EPI_GATE_RESIDUAL computes. */
+  const void* delta_y;
+  const float* delta_gate;
+  void* x_out;
+  int64_t d_sb, d_st, gate_stride, xo_sb, xo_st;
 } hdit_ln_job;
 
 int hdit_layernorm_modulate_jobs(const hdit_ln_job* jobs, int count, int dim, const void* ln_weight,
@@ -379,6 +390,25 @@ typedef struct hdit_sd3_block_args {
   void* text_kv;
   int32_t text_kv_mode;
   int32_t fp8_attention;
+  /* Gated residuals left to the next normalisation (fp32 streams only; all optional).
+   * pending_img / pending_txt: bf16 [batch, n_img | n_txt, dim], an update still owed to `hidden` / `encoder`:
+   * the stream this block works on is hidden + pending_img_gate[b, :] * pending_img (gate f32, batch stride
+   * pending_*_gate_stride) -- applied inside norm1 / norm1_context.  defer_img / defer_txt (need out_f32 and
+   * modulation_img / modulation_txt): the MLP's output projection writes bf16(A W^T + bias) there instead of
+   * adding it; hidden_out / encoder_out then hold the stream after the attention residual, and the caller passes
+   * (defer_*, modulation_* + 5 dim, 6 dim) as the next block's pending_*.  The sums are the ones the fused epilogue
+   * makes, fma(gate, y, x) in fp32, so a stack run this way returns the same bits. */
+  const void* pending_img;
+  const float* pending_img_gate;
+  const void* pending_txt;
+  const float* pending_txt_gate;
+  int64_t pending_img_gate_stride, pending_txt_gate_stride;
+  void* defer_img;
+  void* defer_txt;
+  /* != 0: inside the block, too, the attention residual of a stream that arrives in f32 is added by norm2
+   * (the out-projection writes bf16(A W^T + bias)) instead of in the out-projection's epilogue; same bits. */
+  int32_t lazy_residual;
+  int32_t pad_;
 } hdit_sd3_block_args;
 
 #define HDIT_TEXT_KV_NONE 0

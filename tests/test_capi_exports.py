@@ -47,7 +47,7 @@ def test_binding_covers_every_declared_symbol():
 
     assert sorted(_lib.SIGNATURES) == declared_symbols()
     lib = _lib.lib()
-    assert lib.hdit_abi_version() == _lib.ABI_VERSION == 4
+    assert lib.hdit_abi_version() == _lib.ABI_VERSION == 5
     assert lib.hdit_last_error() == b""
 
 
@@ -59,8 +59,8 @@ def test_struct_layouts_match_the_header(library):
     assert ctypes.sizeof(_lib.SeqSegment) == 8 + 3 * 8 + 2 * 4
     assert ctypes.sizeof(_lib.AttnArgs) == 8 * ctypes.sizeof(_lib.SeqSegment) + 4 * 4
     assert ctypes.sizeof(_lib.QkNormJob) == 8 + 3 * 8 + 4 * 8 + 4 * 4
-    assert ctypes.sizeof(_lib.LnJob) == 4 * 8 + 5 * 8 + 4 * 4
-    assert ctypes.sizeof(_lib.Sd3BlockArgs) == 20 * 8 + 9 * 8 + 8 + 14 * 4 + 8 + 2 * 4
+    assert ctypes.sizeof(_lib.LnJob) == 4 * 8 + 5 * 8 + 4 * 4 + 3 * 8 + 5 * 8
+    assert ctypes.sizeof(_lib.Sd3BlockArgs) == 20 * 8 + 9 * 8 + 8 + 14 * 4 + 8 + 2 * 4 + 8 * 8 + 2 * 4
 
 
 def test_struct_layouts_against_the_c_compiler(tmp_path):

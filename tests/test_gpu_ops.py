@@ -529,6 +529,47 @@ def test_gemm_fp32_flags_only_with_gate_residual(hdit):
         ops.gemm_problem(a, w, torch.empty(64, 64, dtype=torch.float32, device=DEV))
 
 
+@pytest.mark.parametrize("D", [256, 1536, 3072, 4096])
+def test_layernorm_modulate_applies_a_pending_update(hdit, D):
+    """``hdit_ln_job.delta_y``: the fp32 stream is first updated to fma(gate, y, x) -- the operation of the GEMM's
+    gated-residual epilogue -- written back, and normalised.  Checked against the GEMM epilogue itself (identity
+    weight, so the epilogue's product is y exactly), against float64, and against the plain kernel run on the
+    updated stream; in place, out of place, next to a job without an update, and without a write-back."""
+    print(f"ln pending update D={D}", flush=True)
+    ops = hdit.ops
+    B, T = 2, 41
+    gen = torch.Generator().manual_seed(81)
+    x = (torch.randn(B, T, D, generator=gen) * 3 + 0.5).to(DEV)
+    y = g(rnd(B, T, D, seed=82))
+    gate = torch.randn(B, D, generator=gen).to(DEV)
+    sh, sc = torch.randn(B, D, generator=gen).to(DEV), (torch.randn(B, D, generator=gen) * 0.1).to(DEV)
+    other = (torch.randn(B, 7, D, generator=gen)).to(DEV)
+    # what the fused epilogue computes: C = resid + gate * bf16(A . I^T) with A = y
+    eye = torch.eye(D, device=DEV, dtype=torch.bfloat16)
+    fused = torch.empty(B * T, D, device=DEV)
+    ops.gemm_launch([ops.gemm_problem(y.view(-1, D), eye, fused, None, ops.EPI_GATE_RESIDUAL, x.view(-1, D), gate, T)])
+    x_new = torch.empty_like(x)
+    out, out_other = ops.layernorm_modulate_many([(x, sh, sc, None, (y, gate, x_new)), (other, sh, sc)])
+    plain = ops.layernorm_modulate(x_new, sh, sc)
+    plain_other = ops.layernorm_modulate(other, sh, sc)
+    torch.cuda.synchronize()
+    assert torch.equal(x_new.view(-1, D), fused), "the update is not the gated epilogue's"
+    exact = (x.double() + gate.double()[:, None, :] * y.double()).float()
+    assert (x_new - exact).abs().max().item() <= 1e-6 * exact.abs().max().item()
+    assert torch.equal(out, plain) and torch.equal(out_other, plain_other)
+    # no write-back: same normalised rows, stream untouched
+    keep = x.clone()
+    (out2,) = ops.layernorm_modulate_many([(x, sh, sc, None, (y, gate, None))])
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out) and torch.equal(x, keep)
+    # in place
+    (out3,) = ops.layernorm_modulate_many([(x, sh, sc, None, (y, gate, x))])
+    torch.cuda.synchronize()
+    assert torch.equal(out3, out) and torch.equal(x, x_new)
+    with pytest.raises(ValueError):  # only the fp32 stream takes an update
+        ops.layernorm_modulate_many([(y, sh, sc, None, (y, gate, None))])
+
+
 @pytest.mark.parametrize("D", [256, 1536, 3072, 4096, 264])
 @pytest.mark.parametrize("affine", [False, True])
 def test_layernorm_modulate_fp32_rows(hdit, D, affine):

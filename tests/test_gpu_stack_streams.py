@@ -82,8 +82,12 @@ def test_entry_point_blocks_lanes_and_overlapped_patches_give_the_same_bits(hdit
     for block in stack.transformer_blocks:
         block.attn.fp8_attention = fp8  # the attention of every form on the fp8-e4m3 path
     want = run_step_sequence(stack, B, Ni, Nt, D, P, entry_points=False, batch_streams=1, patch_streams=0)
+    # on one stream the entry-point passes leave every gated residual to the normalisation that reads the stream next
+    # (stack.defer_residuals); batch lanes and patches on several streams keep them in the GEMM epilogues
     forms = [
         ("entry points, one stream", True, 1, 0),
+        ("entry points, one stream, residuals fused into the GEMM epilogues", True, 1, 0, False),
+        ("entry points, merged fronts, residuals fused into the GEMM epilogues", True, 1, 1, False),
         ("entry points, batch lanes", True, 2, 0),
         ("entry points, three batch lanes, patches on one stream through forward_patches (merged fronts)", True, 3, 1),
         ("entry points, patches on one stream through forward_patches, fronts not merged", True, 1, -1),
@@ -91,9 +95,11 @@ def test_entry_point_blocks_lanes_and_overlapped_patches_give_the_same_bits(hdit
         ("entry points, patches on three streams", True, 1, 3),
         ("kernel by kernel, patches on two streams", False, 1, 2),
     ]
-    for name, entry_points, batch_streams, patch_streams in forms:
+    for name, entry_points, batch_streams, patch_streams, *rest in forms:
         reset_runtime_state()  # the full pass of every form replaces the K/V buffers of the one before
+        stack.defer_residuals = rest[0] if rest else True
         got = run_step_sequence(stack, B, Ni, Nt, D, P, entry_points, batch_streams, patch_streams)
+        stack.defer_residuals = True
         assert len(got) == len(want)
         for i, (a, b) in enumerate(zip(got, want)):
             assert a.shape == b.shape and torch.equal(a, b), f"{name}: item {i} differs"
