@@ -167,11 +167,17 @@ class JointTransformerBlock(nn.Module):
 
     @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
-                skip_text_output: bool = False):
+                skip_text_output: bool = False, pending=None, defer: bool = False):
         """``skip_text_output``: the caller drops this block's text output (the SD3 block loop does for every
         pipeline patch after the first, ``transformer_sd3.py:131-146``), so the text stream stops after its
         q|k|v projection -- no out-projection, ``norm2_context`` or ``ff_context`` -- and ``None`` is returned
-        for it.  The image output is unchanged bit for bit."""
+        for it.  The image output is unchanged bit for bit.
+
+        ``pending`` / ``defer`` (block stacks, f32 streams): the launches of ``hdit_block_sd3`` with
+        ``lazy_residual`` -- see ``_forward_lazy``."""
+        if pending is not None or defer:
+            return self._forward_lazy(hidden_states, encoder_hidden_states, temb, skip_text_output,
+                                      pending or (None, None), defer)
         eps = 1e-6
         sh_a, sc_a, g_a, sh_m, sc_m, g_m = _adaln(self.norm1, temb)
         if self.context_pre_only:
@@ -192,6 +198,86 @@ class JointTransformerBlock(nn.Module):
         hidden, encoder = _mlp_both_streams(self.ff, _rows2d(n2), hidden, g_m, self.ff_context, _rows2d(nc2), encoder,
                                             c_g_m, out_dtype=self.stream_dtype)
         return encoder, hidden
+
+
+    def _forward_lazy(self, hidden_states, encoder_hidden_states, temb, skip_text_output, pending, defer):
+        """The block with its gated residuals taken out of the GEMM epilogues: a projection writes
+        ``y = bf16(A W^T + bias)`` and the normalisation that reads the f32 stream next adds ``gate * y`` (and
+        writes the updated stream), which spares the GEMM the read-modify-write of the stream.  ``pending``:
+        ``(img, txt)``, each ``(y, gate)`` or None -- the MLP residual the previous block left to this block's
+        norm1.  ``defer``: this block leaves its own MLP residuals the same way; ``self.deferred`` is then the
+        ``pending`` of the next block and the returned streams are the ones after the attention residual.  A
+        stream that arrives in bf16 (the first block of a stack) keeps the fused epilogue for its attention
+        residual.  Sums are fma(gate, y, x) in fp32 wherever they are made, so the bits are the ones of
+        ``forward`` without these arguments."""
+        eps = 1e-6
+        f32 = torch.float32
+        pre_only = self.context_pre_only
+        text_out = not pre_only and not skip_text_output
+        sh_a, sc_a, g_a, sh_m, sc_m, g_m = _adaln(self.norm1, temb)
+        if pre_only:
+            c_sc_a, c_sh_a = _adaln(self.norm1_context, temb)  # AdaLayerNormContinuous: scale first
+            c_g_a = c_sh_m = c_sc_m = c_g_m = None
+        else:
+            c_sh_a, c_sc_a, c_g_a, c_sh_m, c_sc_m, c_g_m = _adaln(self.norm1_context, temb)
+        pend_img, pend_txt = pending
+
+        def first_norm(x, shift, scale, pend, keep):
+            """norm1 item of one stream; returns (item, the stream the rest of the block works on)."""
+            if pend is None:
+                return (x, shift, scale), x
+            x0 = torch.empty_like(x) if keep else None
+            return (x, shift, scale, None, (pend[0], pend[1], x0)), x0
+
+        item_i, x0_img = first_norm(hidden_states, sh_a, sc_a, pend_img, True)
+        item_t, x0_txt = first_norm(encoder_hidden_states, c_sh_a, c_sc_a, pend_txt, text_out)
+        n, nc = ops.layernorm_modulate_many([item_i, item_t], eps)
+        kwargs = {"skip_text_queries": True} if skip_text_output and not pre_only else {}
+        o_img, o_txt = self.attn.processor(self.attn, n, encoder_hidden_states=nc, **kwargs)
+        lazy_img = x0_img.dtype == f32
+        lazy_txt = text_out and x0_txt.dtype == f32
+        problems, outs = self.attn.out_proj_problems(
+            o_img, o_txt, None if lazy_img else x0_img, None if lazy_img else g_a,
+            None if lazy_txt else x0_txt, None if lazy_txt else c_g_a, skip_txt=not text_out)
+        ops.gemm_launch(problems)
+        # norm2 (+ the attention residual of the lazily updated streams)
+        items = [(x0_img, sh_m, sc_m, None, (outs[0], g_a, x0_img if x0_img is not hidden_states else torch.empty_like(x0_img)))
+                 if lazy_img else (outs[0], sh_m, sc_m)]
+        if text_out:
+            items.append((x0_txt, c_sh_m, c_sc_m, None,
+                          (outs[1], c_g_a, x0_txt if x0_txt is not encoder_hidden_states else torch.empty_like(x0_txt)))
+                         if lazy_txt else (outs[1], c_sh_m, c_sc_m))
+        normed = ops.layernorm_modulate_many(items, eps)
+        x1_img = items[0][4][2] if lazy_img else outs[0]
+        x1_txt = (items[1][4][2] if lazy_txt else outs[1]) if text_out else None
+        # MLP
+        p_in, h = self.ff.in_problem(_rows2d(normed[0]))
+        probs = [p_in]
+        if text_out:
+            pc_in, hc = self.ff_context.in_problem(_rows2d(normed[1]))
+            probs.append(pc_in)
+        ops.gemm_launch(probs)
+        self.deferred = None
+        if defer:
+            if self.stream_dtype != f32:
+                raise ValueError("residuals can only be left to the next block on an f32 stream")
+            y_img = torch.empty(x1_img.shape, dtype=torch.bfloat16, device=x1_img.device)
+            probs = [self.ff.out_problem(h, _rows2d(y_img))]
+            y_txt = None
+            if text_out:
+                y_txt = torch.empty(x1_txt.shape, dtype=torch.bfloat16, device=x1_txt.device)
+                probs.append(self.ff_context.out_problem(hc, _rows2d(y_txt)))
+            ops.gemm_launch(probs)
+            self.deferred = ((y_img, g_m), (y_txt, c_g_m) if text_out else None)
+            return x1_txt, x1_img
+        out = _stream_out(x1_img, self.stream_dtype)
+        probs = [self.ff.out_problem(h, _rows2d(out), _rows2d(x1_img), g_m, rows_per_batch=x1_img.shape[1])]
+        out_c = None
+        if text_out:
+            out_c = _stream_out(x1_txt, self.stream_dtype)
+            probs.append(self.ff_context.out_problem(hc, _rows2d(out_c), _rows2d(x1_txt), c_g_m, rows_per_batch=x1_txt.shape[1]))
+        ops.gemm_launch(probs)
+        return out_c, out
 
 
 class FluxTransformerBlock(nn.Module):

@@ -54,6 +54,12 @@ class _Chain:
         self.img = None
         self.txt = None
 
+    def take(self, left, skipped_text_output: bool):
+        """``left``: what the block that just ran left owing, ``(img, txt_or_None)`` or None."""
+        self.img = left[0] if left is not None else None
+        if not skipped_text_output:  # a call that drops its text output leaves the text stream's state alone
+            self.txt = left[1] if left is not None else None
+
 
 class SD3TransformerBlocks(nn.Module):
     """The 24 joint blocks of the SD3 transformer with the reference's block loop.
@@ -133,9 +139,16 @@ class SD3TransformerBlocks(nn.Module):
         numbers for all of them: the first patch's call leaves them in a buffer and the later ones take them from
         there -- as long as they really come with the same text states and the same ``temb``."""
         block = self.transformer_blocks[i]
+        # every block but the last leaves its MLP residuals to the next block's first normalisation
+        leave = chain is not None and i + 1 < len(self.transformer_blocks) and block.stream_dtype == torch.float32
         if calls is None:
-            return block(hidden_states=hidden, encoder_hidden_states=encoder, temb=temb,
-                         skip_text_output=skip_text_output)
+            if chain is None:
+                return block(hidden_states=hidden, encoder_hidden_states=encoder, temb=temb,
+                             skip_text_output=skip_text_output)
+            out = block(hidden_states=hidden, encoder_hidden_states=encoder, temb=temb,
+                        skip_text_output=skip_text_output, pending=(chain.img, chain.txt), defer=leave)
+            chain.take(block.deferred, skip_text_output)
+            return out
         text_kv, text_kv_mode = None, _lib.TEXT_KV_NONE
         if not self.reuse_text_kv:
             pass
@@ -162,18 +175,10 @@ class SD3TransformerBlocks(nn.Module):
             hidden_out=hidden_out, text_kv=text_kv, text_kv_mode=text_kv_mode,
         )
         if chain is not None:
-            kwargs["pending_img"] = chain.img
-            kwargs["pending_txt"] = chain.txt
-            # every block but the last leaves its MLP residuals to the next block's first normalisation
-            kwargs["defer"] = self.defer_residuals and i + 1 < len(self.transformer_blocks) \
-                and block.stream_dtype == torch.float32
-            kwargs["lazy"] = self.defer_residuals
+            kwargs.update(pending_img=chain.img, pending_txt=chain.txt, defer=leave, lazy=True)
         encoder_out, hidden_new, ws = calls[i].prepare(hidden, encoder, temb, **kwargs)
         if chain is not None:
-            left = calls[i].deferred
-            chain.img = left[0] if left is not None else None
-            if not skip_text_output:  # a call that drops its text output leaves the text stream's state alone
-                chain.txt = left[1] if left is not None else None
+            chain.take(calls[i].deferred, skip_text_output)
         if defer is None:
             calls[i].launch()
             del ws  # stream-ordered reuse: the workspace may be freed as soon as the launches are queued
@@ -218,7 +223,7 @@ class SD3TransformerBlocks(nn.Module):
             lanes = min(self.batch_streams, hidden_states.shape[0])
             if not rs.patch_mode and lanes > 1 and not torch.cuda.is_current_stream_capturing():
                 return self._forward_batch_lanes(calls, mods, hidden_states, encoder_hidden_states, temb, lanes)
-        chain = _Chain() if calls is not None else None
+        chain = _Chain() if self.defer_residuals else None
         for i in range(len(self.transformer_blocks)):
             kv = self._kv_buffer(i, hidden_states) if calls is not None else (None, 0)
             if rs.patch_mode and rs.pipeline_patch_idx == 0:
@@ -323,7 +328,7 @@ class SD3TransformerBlocks(nn.Module):
         events = self._patch_events
         cache = self.encoder_hidden_states_cache
         # residual chains only where the patches run one after the other (see _forward_batch_lanes)
-        chains = [_Chain() for _ in range(P)] if calls is not None and len(streams) == 1 else [None] * P
+        chains = [_Chain() for _ in range(P)] if self.defer_residuals and len(streams) == 1 else [None] * P
         try:
             for front in range(L + P - 1):  # launches are issued along the diagonal, the order they can start in
                 for p in range(P):
@@ -374,7 +379,7 @@ class SD3TransformerBlocks(nn.Module):
         rs = get_runtime_state()
         P, L = len(hidden), len(self.transformer_blocks)
         cache = self.encoder_hidden_states_cache
-        chains = [_Chain() for _ in range(P)]
+        chains = [_Chain() if self.defer_residuals else None for _ in range(P)]
         try:
             for front in range(L + P - 1):
                 group = []
@@ -386,12 +391,13 @@ class SD3TransformerBlocks(nn.Module):
                     kv = self._kv_buffer(i, hidden[p])
                     if p == 0:
                         cache[i] = encoder_hidden_states
-                        self._text_pending[i] = chains[0].txt
+                        self._text_pending[i] = chains[0].txt if chains[0] is not None else None
                         encoder_hidden_states, hidden[0] = self._run_block(
                             i, calls, mods, hidden[0], encoder_hidden_states, temb, kv_buffer=kv[0], kv_row0=kv[1], patch=0,
                             defer=group, chain=chains[0])
                     else:
-                        chains[p].txt = self._text_pending[i]
+                        if chains[p] is not None:
+                            chains[p].txt = self._text_pending[i]
                         _, hidden[p] = self._run_block(
                             i, calls, mods, hidden[p], cache[i], temb, skip_text_output=True, kv_buffer=kv[0],
                             kv_row0=kv[1], patch=p, defer=group, chain=chains[p])
