@@ -500,11 +500,13 @@ def main():
             "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": gemm_traffic if headline else None,
             "traffic_note": "from profiles/sd3_1024_step_hbm_traffic.txt: rocprofv3 FETCH_SIZE and WRITE_SIZE, each scaled "
                             "by what the counter reads for a 256 MiB copy, mean over the step's hdit_gemm_bf16 calls; "
-                            "algorithmic operand + residual + result bytes average 177.9 MB per call (activations of both streams, both weight sets, fp32 residual stream)",
+                            "algorithmic operand + result bytes average 137.5 MB per call (activations of both streams, both weight sets; "
+                            "on one stream the gated residuals of the fp32 stream are added by the normalisation kernels, "
+                            "not by the GEMM epilogues)",
             "launches_per_step": n_g // 3, "avg_launch_us": round(ms_g / max(n_g, 1) * 1e3, 2),
             "flops_per_launch": round(fl_g / max(n_g, 1), 1),
-            "measured_in": "three instrumented passes after the timed ones: kernel by kernel on one stream, HIP events "
-                           "around every launch (a launch alone on the GPU); the rocprofv3 trace of `bench.py --single-stream "
+            "measured_in": "three instrumented passes after the timed ones: kernel by kernel on one stream (the launches of "
+                           "the single-stream form), HIP events around every launch (a launch alone on the GPU); the rocprofv3 trace of `bench.py --single-stream "
                            "--no-graph` is profiles/<workload>_kernel_stats.txt, that of this command "
                            "profiles/<workload>_two_streams_kernel_stats.txt",
         },
