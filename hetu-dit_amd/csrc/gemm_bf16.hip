@@ -123,6 +123,16 @@ __device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, uns
                : "m0");
 }
 
+// The same with the LDS address given as a uniform base plus a uniform offset: the sum is formed in M0 itself, one
+// scalar instruction less per request than adding first and moving the result (a slab is 16 requests per wave).
+__device__ __forceinline__ void lds_dma16_sum(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform,
+                                              unsigned lds_off_uniform) {
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr_uniform), "v"(voff), "s"(base_uniform), "s"(lds_off_uniform)
+               : "m0", "scc");
+}
+
 // One wave-wide 4-byte direct-to-LDS load: lane l's dword at base + voff lands at LDS byte address lds_addr + 4*l.
 // Used only to pull cache lines towards the CU ahead of time; what lands in LDS is never read.
 __device__ __forceinline__ void lds_touch4(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
@@ -205,13 +215,13 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     G[i] = *(const i32x4*)(base + p_off[i]);
   };
   // direct-to-LDS request i of the slab at the cursor: A rows into A slot `slot`, B rows into B slot `slot`
+  const unsigned wave_lds = lds_base_addr + wave * 8 * ROW_BYTES;
   auto dma_a = [&](int slot, int i) {
-    lds_dma16(p_abase + (size_t)p_kt * ROW_BYTES, p_off[i],
-              lds_base_addr + slot * C::A_BYTES + i * (NW * 8 * ROW_BYTES) + wave * 8 * ROW_BYTES);
+    lds_dma16_sum(p_abase + (size_t)p_kt * ROW_BYTES, p_off[i], wave_lds + slot * C::A_BYTES, i * (NW * 8 * ROW_BYTES));
   };
   auto dma_b = [&](int slot, int i) {
-    lds_dma16(p_bbase + (size_t)p_kt * ROW_BYTES, p_off[C::A_LOADS + i],
-              lds_base_addr + C::B_OFF + slot * C::B_BYTES + i * (NW * 8 * ROW_BYTES) + wave * 8 * ROW_BYTES);
+    lds_dma16_sum(p_bbase + (size_t)p_kt * ROW_BYTES, p_off[C::A_LOADS + i], wave_lds + C::B_OFF + slot * C::B_BYTES,
+                  i * (NW * 8 * ROW_BYTES));
   };
   auto l_store = [&](int stage, int i) {
     const int tile_off = i < C::A_LOADS ? i * (NW * 8 * ROW_BYTES) : C::A_BYTES + (i - C::A_LOADS) * (NW * 8 * ROW_BYTES);
