@@ -156,6 +156,63 @@ def test_block_sd3_one_call_with_fp8_attention(hdit):
     assert_parity(enc_c, want_e, rel=3e-2, cos=0.999, what="fp8 block encoder")
 
 
+def test_block_sd3_residuals_left_to_the_next_normalisation(hdit):
+    """``lazy_residual`` / ``defer_*`` / ``pending_*``: a chain of three blocks (the last ``context_pre_only``)
+    in which every gated residual of the f32 streams is added by the normalisation that reads the stream next
+    returns the bits of the chain with the residuals fused into the GEMM epilogues; and what the entry point
+    refuses."""
+    from hetu_dit_amd import _lib, synthetic
+    from hetu_dit_amd.blocks import StackModulation
+
+    B, N, Nt, D, H = 2, 300, 45, 512, 8
+    blks = [make_block(i == 2, 10 + i, D, H)[0] for i in range(3)]
+    for b in blks[:2]:
+        b.stream_dtype = torch.float32
+    x, e, t = (synthetic.randn_bf16(s, k).to(DEV) for s, k in (((B, N, D), 5), ((B, Nt, D), 6), ((B, D), 7)))
+    mods = StackModulation(torch.nn.ModuleList(blks)).precompute_by_module(t)
+    flat, offsets = mods
+    calls = [hdit.ops.Sd3BlockCall(b) for b in blks]
+
+    def chain(lazy):
+        h, enc, pend = x, e, (None, None)
+        for i, (b, call) in enumerate(zip(blks, calls)):
+            addr = lambda m: flat.data_ptr() + 4 * offsets[m]
+            enc, h = call(h, enc, t, out_dtype=b.stream_dtype, modulation_img=addr(b.norm1),
+                          modulation_txt=addr(b.norm1_context), pending_img=pend[0], pending_txt=pend[1],
+                          defer=lazy and i < 2, lazy=lazy)
+            pend = call.deferred if call.deferred is not None else (None, None)
+            assert (call.deferred is not None) == (lazy and i < 2)
+        return h
+
+    fused, lazy = chain(False).clone(), chain(True).clone()
+    torch.cuda.synchronize()
+    assert fused.dtype == torch.bfloat16 and torch.equal(fused, lazy)
+    # refusals: nothing may be left owing on a bf16 output, without the modulation, or owed to a bf16 stream
+    lib = _lib.lib()
+    call = calls[0]
+    call.prepare(x.float(), e.float(), t, out_dtype=torch.float32, modulation_img=flat.data_ptr() + 4 * offsets[blks[0].norm1],
+                 modulation_txt=flat.data_ptr() + 4 * offsets[blks[0].norm1_context], defer=True, lazy=True)
+    a = call.args
+    assert lib.hdit_block_sd3_workspace_bytes(C.byref(a)) > 0
+    keep = a.modulation_img
+    a.modulation_img = None
+    assert lib.hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
+    a.modulation_img = keep
+    a.out_f32 = 0
+    assert lib.hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
+    a.out_f32 = 1
+    a.pending_img, a.pending_img_gate, a.hidden_f32 = a.defer_img, a.modulation_img, 0
+    assert lib.hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
+    a.hidden_f32 = 1
+    a.pending_img_gate = None
+    assert lib.hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
+    a.pending_img = None
+    a.lazy_residual = 2
+    assert lib.hdit_block_sd3_workspace_bytes(C.byref(a)) == -1
+    with pytest.raises(ValueError):  # the binding refuses the same before the library sees it
+        call.prepare(x.float(), e.float(), t, out_dtype=torch.bfloat16, modulation_img=keep, modulation_txt=keep, defer=True)
+
+
 def test_block_sd3_refuses_bad_arguments(hdit):
     from hetu_dit_amd import _lib
 
