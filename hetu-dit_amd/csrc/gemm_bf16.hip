@@ -456,6 +456,12 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     auto epilogue = [&](auto mode_tag) {
       constexpr int MODE = decltype(mode_tag)::value;
       constexpr bool GATED = MODE == HDIT_EPI_GATE_RESIDUAL;
+      // The lane-dependent addresses of the epilogue are recomputed per tile from an opaque copy of the lane id:
+      // otherwise the compiler hoists some fifty of them out of the tile loop and, the main loop having no registers
+      // to spare, spills them around it -- reloads that wait for every operand request in flight.
+      int lane_e = lane;
+      asm volatile("" : "+v"(lane_e));
+      const int l32 = lane_e & 31, lh = lane_e >> 5;
       // all addressing below is a uniform base plus a 32-bit byte offset per lane (checked on the host)
       unsigned char* __restrict__ Cb = (unsigned char*)pr.c;
       const unsigned char* __restrict__ Rb = (const unsigned char*)pr.resid;
@@ -469,8 +475,8 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
       // per 32-row block, done as two halves of 4.  The residual rows and the gate columns are requested one
       // block ahead, before the stores in front of them: vector memory operations retire in order, so a load
       // placed behind stores would wait for the stores' round trip.
-      const int rchunk = lane & 15;
-      const int wr_row = lane >> 4;
+      const int rchunk = lane_e & 15;
+      const int wr_row = lane_e >> 4;
       const int wr_n = ncol0 + rchunk * 8;
       const int wr_nc = min(wr_n, N - 8);
       const bool wr_ok = rchunk < 4 * TN && wr_n < N;
@@ -518,9 +524,17 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
         prefetch_gate(0);
       }
 
+      typedef __attribute__((address_space(3))) i32x4 lds_i32x4;
 #pragma unroll
       for (int i = 0; i < TM; i++) {
         const int mrow0 = tc.m0 + wm0 + i * 32;
+        // Staging addresses: the XOR swizzle only touches bits 4-7, which are zero in the 256-byte aligned row
+        // base, so slot (chunk ^ (row & 15)) of a row is (row base + ((row & 15) << 4)) ^ (chunk << 4): one register
+        // and one v_xor per access, made opaque per block so that the sixteen write and eight read addresses are not
+        // computed ahead and spilled.
+        unsigned wa = lds_address(epi) + l32 * 256 + ((l32 & 15) << 4);
+        unsigned ra = lds_address(epi) + wr_row * 256 + ((rchunk ^ wr_row) << 4);
+        asm volatile("" : "+v"(wa), "+v"(ra));
 #pragma unroll
         for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -544,7 +558,7 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
 #pragma unroll
               for (int e = 0; e < 8; e++) v[e] = hdit::gelu_tanh_f(v[e]);
             }
-            *(i32x4*)(epi + l32 * 256 + ((chunk ^ (l32 & 15)) << 4)) = hdit::pack8(v);
+            *(lds_i32x4*)(uintptr_t)(wa ^ (unsigned)(chunk << 4)) = hdit::pack8(v);
           }
           SCHED_FENCE();  // keeps the scheduler from pulling whole accumulator tiles into VGPRs at once
         }
@@ -556,7 +570,8 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
           for (int q = 0; q < 4; q++) {
             const int it = half * 4 + q;
             const int r = it * 4 + wr_row;
-            i32x4 val = *(const i32x4*)(epi + r * 256 + ((rchunk ^ (r & 15)) << 4));
+            // row r = 4 it + wr_row: slot rchunk ^ (r & 15) = (rchunk ^ wr_row) ^ 4 (it & 3)
+            i32x4 val = *(const lds_i32x4*)(uintptr_t)((ra ^ (unsigned)(((it & 3) * 4) << 4)) + it * 1024);
             if (GATED) {
               f32x4 g0 = gte0, g1 = gte1;
               if (straddle) {  // rows of this block belong to different batch elements: fetch the gate per row
