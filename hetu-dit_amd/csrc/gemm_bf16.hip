@@ -133,15 +133,6 @@ __device__ __forceinline__ void lds_dma16_sum(const unsigned char* base_uniform,
                : "m0", "scc");
 }
 
-// One wave-wide 4-byte direct-to-LDS load: lane l's dword at base + voff lands at LDS byte address lds_addr + 4*l.
-// Used only to pull cache lines towards the CU ahead of time; what lands in LDS is never read.
-__device__ __forceinline__ void lds_touch4(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-               :
-               : "s"(lds_addr_uniform), "v"(voff), "s"(base_uniform)
-               : "m0");
-}
-
 __device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
   return (unsigned)(uintptr_t)((const __attribute__((address_space(3))) unsigned char*)p);
 }
@@ -389,8 +380,6 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     constexpr int CPA = (C::A_LOADS + 2) / 3;  // A requests per k-step (k-steps 0..2 of a slab)
 
     if constexpr (C::DMA) {
-      const bool gated = (pr.epilogue & HDIT_EPI_MODE_MASK) == HDIT_EPI_GATE_RESIDUAL;
-      const int touch_kt = KT >= 2 ? KT - 2 : 0;
       for (int kt = 0; kt < KT; kt++) {
         const unsigned char* ab = lds + sa * C::A_BYTES;
         const unsigned char* bb = lds + C::B_OFF + sb * C::B_BYTES;
@@ -406,28 +395,6 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
         const int sb_req = sb;  // the B slot this slab vacates takes the B rows of the slab after next
         sa = sa == C::A_SLOTS - 1 ? 0 : sa + 1;
         sb ^= 1;
-        if (gated && kt == touch_kt) {
-          // Gated residual: the epilogue reads this wave's (32*TM) x (32*TN) piece of the residual, a tensor last
-          // written hundreds of microseconds ago, i.e. from HBM, and can only keep one 32-row block of requests
-          // in flight.  Touch every cache line of the piece now, two slabs before the epilogue, so that those
-          // requests find the lines in L2.  The dwords go to the first 256 bytes of this wave's share of the B
-          // slot just vacated; the wave's own B request for that share is issued below, returns later (a wave's
-          // loads return in order) and overwrites them.
-          const int esz = (pr.epilogue & HDIT_EPI_RESID_F32) ? 4 : 2;
-          const int seg_bytes = min(C::WN, pr.n - (tc.n0 + wn0)) * esz;  // bytes of the piece per row
-          if (seg_bytes > 0) {
-            const int ppr = (seg_bytes + 127) >> 7;  // 128-byte pieces per row
-            const unsigned char* rb = (const unsigned char*)pr.resid;
-            const unsigned dst = lds_base_addr + C::B_OFF + sb_req * C::B_BYTES + wave * 8 * ROW_BYTES;
-            const int total = C::WM * ppr;
-#pragma unroll 1
-            for (int idx = lane; idx < total; idx += 64) {
-              const int r = idx / ppr, piece = idx - r * ppr;
-              const int mm = min(tc.m0 + wm0 + r, pr.m - 1);
-              lds_touch4(rb, (unsigned)((mm * (int)pr.ldr + tc.n0 + wn0) * esz + min(piece * 128, seg_bytes - 4)), dst);
-            }
-          }
-        }
         k_step_dma(1, lds + sa * C::A_BYTES, lds + C::B_OFF + sb * C::B_BYTES, 0, 1, 0, C::B_LOADS, sb_req);
         p_advance();
       }
