@@ -81,8 +81,15 @@ struct Cfg {
   static constexpr int A_SLOTS = 3, B_SLOTS = 2;
   static constexpr int B_OFF = A_SLOTS * A_BYTES;
   static constexpr int DMA_BYTES = A_SLOTS * A_BYTES + B_SLOTS * B_BYTES;
+  // RING: the 128x128 shape takes its slabs the same way into a ring of four stages (A then B, 32 KiB each),
+  // requested three slabs ahead: its slabs are short (16 MFMAs per wave), and only a lead of several of them
+  // covers the latency of operands that come from HBM.  The epilogue windows alias the stage the tile's last slab
+  // vacated.
+  static constexpr bool RING = TM == 2 && TN == 2;
+  static constexpr int NS = RING ? 4 : 2;
+  static constexpr bool DIRECT = DMA || RING;
   static constexpr bool BIAS_IN_LDS = !DMA || DMA_BYTES + NW * 1024 <= 160 * 1024;
-  static constexpr int BIAS_OFF = DMA ? DMA_BYTES : 2 * STAGE_BYTES;  // one 1 KiB bias slot per wave
+  static constexpr int BIAS_OFF = DMA ? DMA_BYTES : NS * STAGE_BYTES;  // one 1 KiB bias slot per wave
   static constexpr int LDS_BYTES = BIAS_OFF + (BIAS_IN_LDS ? NW * 1024 : 0);
   static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
   static_assert(DMA ? NW * EPI_WAVE_BYTES <= A_BYTES : NW * EPI_WAVE_BYTES <= STAGE_BYTES,
@@ -116,8 +123,12 @@ __device__ __forceinline__ TileCoord locate(const GemmTable& tab, int lid) {
 // lds_addr + 16*l.  Only used for the bias slots.  Inline assembly, so the compiler's wait-count
 // insertion does not see it: an extra operation in flight only makes the waits it computes for its own
 // loads stricter than needed.
+// Every direct-to-LDS request is issued at agent scope (sc1), which the CU's L1 never serves.  The kernels wait
+// for "all but the newest n" requests and rely on completion in issue order; a request that hits in L1 completes
+// ahead of older misses (measured: a ragged tile, whose out-of-range lanes all read the problem's last row, then
+// multiplied a slab that had not landed).  From L2, hits and misses complete in issue order.
 __device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
                :
                : "s"(lds_addr_uniform), "v"(voff), "s"(base_uniform)
                : "m0");
@@ -127,7 +138,7 @@ __device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, uns
 // scalar instruction less per request than adding first and moving the result (a slab is 16 requests per wave).
 __device__ __forceinline__ void lds_dma16_sum(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform,
                                               unsigned lds_off_uniform) {
-  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
                :
                : "s"(lds_addr_uniform), "v"(voff), "s"(base_uniform), "s"(lds_off_uniform)
                : "m0", "scc");
@@ -172,7 +183,7 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
   const int st_off = st_row * ROW_BYTES + ((ld_chunk ^ ((st_row >> 1) & 7)) << 4);
   // A direct-to-LDS request lands lane l at byte 16*l of the wave's 1 KiB (row l/8, position l%8), so the
   // swizzle is applied on the source side: position c' of row r receives chunk c' ^ ((r>>1)&7).
-  const int src_chunk = C::DMA ? (ld_chunk ^ ((st_row >> 1) & 7)) : ld_chunk;
+  const int src_chunk = C::DIRECT ? (ld_chunk ^ ((st_row >> 1) & 7)) : ld_chunk;
   const unsigned lds_base_addr = __builtin_amdgcn_readfirstlane(lds_address(lds));
   int p_lid = lid;
   bool p_valid = true;
@@ -180,7 +191,7 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
   const unsigned char* p_abase = nullptr;
   const unsigned char* p_bbase = nullptr;
   unsigned p_off[C::LOADS];
-  i32x4 G[C::DMA ? 1 : C::LOADS];  // the slab in flight between global memory and LDS (register-staged shapes)
+  i32x4 G[C::DIRECT ? 1 : C::LOADS];  // the slab in flight between global memory and LDS (register-staged shapes)
   auto p_setup = [&]() {
     const TileCoord tc = locate<C>(tab, p_lid);
     const hdit_gemm_problem& pr = tab.p[tc.pi];
@@ -213,6 +224,14 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
   auto dma_b = [&](int slot, int i) {
     lds_dma16_sum(p_bbase + (size_t)p_kt * ROW_BYTES, p_off[C::A_LOADS + i], wave_lds + C::B_OFF + slot * C::B_BYTES,
                   i * (NW * 8 * ROW_BYTES));
+  };
+  // ring shapes: request i (A rows, then B rows) of the slab at the cursor into stage `slot`
+  auto dma_ring = [&](int slot, int i) {
+    if (i < C::A_LOADS)
+      lds_dma16_sum(p_abase + (size_t)p_kt * ROW_BYTES, p_off[i], wave_lds + slot * C::STAGE_BYTES, i * (NW * 8 * ROW_BYTES));
+    else
+      lds_dma16_sum(p_bbase + (size_t)p_kt * ROW_BYTES, p_off[i], wave_lds + slot * C::STAGE_BYTES,
+                    C::A_BYTES + (i - C::A_LOADS) * (NW * 8 * ROW_BYTES));
   };
   auto l_store = [&](int stage, int i) {
     const int tile_off = i < C::A_LOADS ? i * (NW * 8 * ROW_BYTES) : C::A_BYTES + (i - C::A_LOADS) * (NW * 8 * ROW_BYTES);
@@ -276,6 +295,17 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(C::LOADS));
     __syncthreads();
     read_frags2(lds, lds + C::B_OFF, 0, 0);
+  } else if constexpr (C::RING) {
+    // slabs 0 .. NS-2 into stages 0 .. NS-2; slab 0 has landed before the first fragment read
+#pragma unroll
+    for (int s = 0; s < C::NS - 1; s++) {
+#pragma unroll
+      for (int i = 0; i < C::LOADS; i++) dma_ring(s, i);
+      p_advance();
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((C::NS - 2) * C::LOADS));
+    __syncthreads();
+    read_frags(lds, 0, 0);
   } else {
 #pragma unroll
     for (int i = 0; i < C::LOADS; i++) g_load(i);
@@ -371,7 +401,8 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
           for (int j = 0; j < C::LOADS; j++)
             if (j < n && RD_MFMA + (j * SLOTS) / (n > 0 ? n : 1) == t) {
               if (kind == 0) dma_a(slot, first + j);
-              else dma_b(slot, first + j);
+              else if (kind == 1) dma_b(slot, first + j);
+              else dma_ring(slot, first + j);
             }
           SCHED_FENCE();
         }
@@ -398,6 +429,25 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
         k_step_dma(1, lds + sa * C::A_BYTES, lds + C::B_OFF + sb * C::B_BYTES, 0, 1, 0, C::B_LOADS, sb_req);
         p_advance();
       }
+    } else if constexpr (C::RING) {
+      constexpr int RQ = C::LOADS / 4;  // requests per k-step
+      static_assert(C::LOADS % 4 == 0, "ring requests are dealt evenly to the four k-steps");
+      for (int kt = 0; kt < KT; kt++) {
+        const unsigned char* sbase = lds + stage * C::STAGE_BYTES;
+        // the slab NS-1 ahead goes to the stage the previous slab vacated
+        const int rq = stage == 0 ? C::NS - 1 : stage - 1;
+        k_step_dma(0, sbase, sbase + C::A_BYTES, 1, 2, 0, RQ, rq);
+        k_step_dma(1, sbase, sbase + C::A_BYTES, 2, 2, RQ, 2 * RQ, rq);
+        k_step_dma(0, sbase, sbase + C::A_BYTES, 3, 2, 2 * RQ, 3 * RQ, rq);
+        // ---- turn over: the next slab has landed -- everything but the slab after it (NS-3 whole slabs in
+        // general) and the requests just issued
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm((C::NS - 3) * C::LOADS + 3 * RQ) & 0xf0ff);  // and lgkmcnt(0)
+        __syncthreads();
+        stage = stage == C::NS - 1 ? 0 : stage + 1;
+        const unsigned char* nbase = lds + stage * C::STAGE_BYTES;
+        k_step_dma(1, nbase, nbase + C::A_BYTES, 0, 2, 3 * RQ, C::LOADS, rq);
+        p_advance();
+      }
     } else
     for (int kt = 0; kt < KT; kt++) {
       const unsigned char* sbase = lds + stage * C::STAGE_BYTES;
@@ -414,7 +464,9 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     }
     // staging window of this wave: inside the stage (the A slot) the tile's last slab vacated
     unsigned char* epi = lds + wave * EPI_WAVE_BYTES +
-                         (C::DMA ? (sa == 0 ? C::A_SLOTS - 1 : sa - 1) * C::A_BYTES : (stage ^ 1) * C::STAGE_BYTES);
+                         (C::DMA    ? (sa == 0 ? C::A_SLOTS - 1 : sa - 1) * C::A_BYTES
+                          : C::RING ? (stage == 0 ? C::NS - 1 : stage - 1) * C::STAGE_BYTES
+                                    : (stage ^ 1) * C::STAGE_BYTES);
 
     // ---- epilogue ---------------------------------------------------------
     // register-staged shapes: the bias copy is only known to have landed after the second slab's loads
@@ -610,7 +662,7 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     if (lid >= xcd_end) break;
   }
   // requests past the end of the stream are still in flight: nothing may land in LDS after this returns
-  if constexpr (C::DMA) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+  if constexpr (C::DIRECT) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 }
 
 template <class C>

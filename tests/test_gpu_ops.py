@@ -35,6 +35,31 @@ def test_gemm_bias(hdit, m, n, k, cfg):
         hdit._lib.lib().hdit_gemm_force_config(-1)
 
 
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("m", [666, 154, 40])
+def test_gemm_ragged_tile_with_operands_out_of_the_caches(hdit, m, cfg):
+    """The out-of-range rows of a ragged tile all read the problem's last row.  Served from the CU's L1, such
+    requests complete ahead of older ones that miss, which the "all but the newest n" waits of the direct-to-LDS
+    pipelines cannot tolerate: with operands that come from HBM the tile then multiplied slabs that had not landed.
+    The requests are issued at agent scope for that reason; this is the case that showed it."""
+    print(f"gemm ragged cold m={m} cfg={cfg}", flush=True)
+    n, k = 1536, 1536
+    lib = hdit._lib.lib()
+    lib.hdit_gemm_force_config(cfg)
+    try:
+        flush = torch.empty(1 << 28, dtype=torch.int32, device=DEV)  # 1 GiB: four times the last-level cache
+        for rep in range(3):
+            a, w, b = rnd(m, k, seed=rep), rnd(n, k, scale=0.05, seed=10 + rep), rnd(n, seed=20 + rep)
+            ga, gw, gb = g(a), g(w), g(b)
+            flush.fill_(rep)
+            torch.cuda.synchronize()
+            out = hdit.ops.linear(ga, gw, gb)
+            torch.cuda.synchronize()
+            assert_parity(out, O.linear(a, w, b), what=f"gemm ragged cold rep {rep}")
+    finally:
+        lib.hdit_gemm_force_config(-1)
+
+
 def test_gemm_gelu_and_gate_residual_grouped(hdit):
     B, T1, T2, D, F = 2, 320, 77, 256, 512
     x1, x2 = rnd(B, T1, D), rnd(B, T2, D)
@@ -137,6 +162,27 @@ def test_attention_single_segment(hdit, hd, sq, skv):
     torch.cuda.synchronize()
     want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
     assert_parity(o, want, what="attention")
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("skv", [1000, 2049])
+def test_attention_clamped_last_tile_with_operands_out_of_the_caches(hdit, hd, skv):
+    """The rows past the end of the last K/V tile all read the last row, and tiles requested past the end read the
+    last tile again: requests that could be served from the CU's L1 and then complete ahead of older ones, which the
+    pipelined kernel's partial waits cannot tolerate.  Operands come from HBM here (caches flushed), the case in
+    which the same pattern made the GEMM multiply slabs that had not landed."""
+    print(f"attention clamped cold hd={hd} skv={skv}", flush=True)
+    B, H, sq = 1, 4, 512
+    flush = torch.empty(1 << 28, dtype=torch.int32, device=DEV)
+    for rep in range(2):
+        q, k, v = rnd(B, sq, H, hd, seed=rep), rnd(B, skv, H, hd, seed=10 + rep), rnd(B, skv, H, hd, seed=20 + rep)
+        gq, gk, gv = g(q), g(k), g(v)
+        flush.fill_(rep)
+        torch.cuda.synchronize()
+        (o,) = hdit.ops.attention([gq], [gk], [gv])
+        torch.cuda.synchronize()
+        want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
+        assert_parity(o, want, what=f"attention clamped cold rep {rep}")
 
 
 def test_attention_two_segments_strided(hdit):
