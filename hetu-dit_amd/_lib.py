@@ -275,3 +275,22 @@ def check(rc: int, what: str):
         if rc in (-3, -4):
             detail = ": " + lib().hdit_last_error().decode()
         raise HditError(f"{what} failed with {_CODES.get(rc, rc)}{detail}")
+
+
+def eager_only(fn):
+    """Mark ``fn`` as opaque to ``torch.compile``: it reaches the C ABI through ``ctypes`` (raw pointers, the current
+    stream's handle), which Dynamo cannot trace.  A compiled caller -- the reference compiles ``transformer.forward``
+    when ``use_torch_compile`` is set (``base_pipeline.py:274-279``) -- breaks the graph here and runs ``fn`` as
+    written; everything else it traces is unaffected.  The disabled function sits behind a plain forwarding function:
+    ``torch.compile`` of a bound method whose function is itself the disabled wrapper loses ``self``."""
+    import functools
+
+    import torch
+
+    opaque = torch.compiler.disable(fn)
+
+    @functools.wraps(fn)
+    def call(*args, **kwargs):
+        return opaque(*args, **kwargs)
+
+    return call

@@ -25,6 +25,7 @@ import torch
 from torch import nn
 
 from . import ops
+from ._lib import eager_only
 from .base_model import wrap_layer
 from .layers.attention_processor import _PackedProjection, _rows2d, hetuDiTAttentionWrapper
 from .layers.feedforward import hetuDiTFeedForwardWrapper
@@ -166,6 +167,7 @@ class JointTransformerBlock(nn.Module):
             self.ff_context = None
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
                 skip_text_output: bool = False, pending=None, defer: bool = False):
         """``skip_text_output``: the caller drops this block's text output (the SD3 block loop does for every
@@ -298,6 +300,7 @@ class FluxTransformerBlock(nn.Module):
         self.ff_context = _wrap(FeedForward(dim))
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None):
         eps = 1e-6
         sh_a, sc_a, g_a, sh_m, sc_m, g_m = _adaln(self.norm1, temb)
@@ -331,6 +334,7 @@ class FluxSingleTransformerBlock(nn.Module):
         )
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states, temb, image_rotary_emb=None):
         B, S, D = hidden_states.shape
         sh, sc, g = _adaln(self.norm, temb)
@@ -391,6 +395,7 @@ class CogVideoXBlock(nn.Module):
         return probs
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None):
         hidden_states = hidden_states.contiguous()
         encoder_hidden_states = encoder_hidden_states.contiguous()

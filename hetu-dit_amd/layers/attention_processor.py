@@ -18,6 +18,7 @@ import torch
 from torch import nn
 
 from .. import ops
+from .._lib import eager_only
 from ..cache_manager import get_cache_manager
 from ..parallel_state import (
     get_pipeline_parallel_world_size,
@@ -296,6 +297,7 @@ class hetuDiTJointAttnProcessor2_0(JointAttnProcessor2_0):
         super().__init__()
         self.use_long_ctx_attn_kvcache = HAS_LONG_CTX_ATTN and get_sequence_parallel_world_size() > 1
 
+    @eager_only
     def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, *args,
                  skip_text_queries: bool = False, **kwargs):
         """``skip_text_queries``: the caller drops the text rows of the attention output (the SD3 block loop
@@ -365,6 +367,7 @@ class hetuDiTFluxAttnProcessor2_0(FluxAttnProcessor2_0):
         super().__init__()
         self.use_long_ctx_attn_kvcache = HAS_LONG_CTX_ATTN and get_sequence_parallel_world_size() > 1
 
+    @eager_only
     def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, image_rotary_emb=None,
                  *args, out=None, extra_problems=None, **kwargs):
         """``image_rotary_emb`` = (cos, sin) f32 [S_call, head_dim] over this call's
@@ -487,6 +490,7 @@ class hetuDiTCogVideoXAttnProcessor2_0(CogVideoXAttnProcessor2_0):
         super().__init__()
         self.use_long_ctx_attn_kvcache = HAS_LONG_CTX_ATTN and get_sequence_parallel_world_size() > 1
 
+    @eager_only
     def __call__(self, attn, hidden_states, encoder_hidden_states, attention_mask=None, image_rotary_emb=None,
                  *args, joint_input: Optional[torch.Tensor] = None, **kwargs):
         """``joint_input``: optionally the already-assembled [B, S, D] joint rows

@@ -6,8 +6,15 @@ from abc import ABCMeta, abstractmethod
 
 import torch.nn as nn
 
+from .._lib import eager_only
+
 
 class hetuDiTDiffusionLayerBaseWrapper(nn.Module, metaclass=ABCMeta):
+    def __init_subclass__(cls, **kwargs):
+        super().__init_subclass__(**kwargs)
+        if "forward" in cls.__dict__ and not getattr(cls.__dict__["forward"], "__isabstractmethod__", False):
+            cls.forward = eager_only(cls.__dict__["forward"])  # the wrappers launch kernels through ctypes
+
     def __init__(self, module: nn.Module):
         super().__init__()
         self.module = module

@@ -17,6 +17,7 @@ import torch
 from torch import nn
 
 from . import _lib, ops
+from ._lib import eager_only
 from .blocks import (CogVideoXBlock, FluxSingleTransformerBlock, FluxTransformerBlock, JointTransformerBlock,
                      StackModulation, use_fp32_residual_stream)
 from .cache_manager import get_cache_manager
@@ -208,6 +209,7 @@ class SD3TransformerBlocks(nn.Module):
 
     # -- the reference's block loop -----------------------------------------------------------------------
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states, encoder_hidden_states, temb):
         rs = get_runtime_state()
         calls = self._entry_point_calls()
@@ -280,6 +282,7 @@ class SD3TransformerBlocks(nn.Module):
         return out
 
     @torch.no_grad()
+    @eager_only
     def forward_patches(self, hidden_states_patches: List[torch.Tensor], encoder_hidden_states: torch.Tensor,
                         temb: torch.Tensor, num_streams: int = 2) -> List[torch.Tensor]:
         """One PipeFusion step of this stage: every patch through every block, the same kernels on the same
@@ -443,6 +446,7 @@ class FluxTransformerBlocks(nn.Module):
         return not any(getattr(b.attn, "fp8_attention", False) for b in blocks)
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb):
         if not self._entry_points_usable():
             return self._forward_per_kernel(hidden_states, encoder_hidden_states, temb, image_rotary_emb)
@@ -499,6 +503,7 @@ class CogVideoXTransformerBlocks(nn.Module):
         self.use_block_entry_points = True
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None) -> Tuple[torch.Tensor, torch.Tensor]:
         if self.use_block_entry_points and not ops.timer_installed():
             temb = temb.contiguous()

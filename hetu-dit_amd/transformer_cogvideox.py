@@ -6,6 +6,7 @@ import torch
 from torch import nn
 
 from . import ops
+from ._lib import eager_only
 from .blocks import _adaln
 from .layers.embeddings import hetuDiTCogVideoXPatchEmbedWrapper, project
 from .layers.modules import AdaLayerNorm, CogVideoXPatchEmbed, TimestepEmbedding
@@ -35,6 +36,7 @@ class CogVideoXTransformer3DModel(nn.Module):
         return project(ops.silu(project(t_proj, self.time_embedding.linear_1)), self.time_embedding.linear_2)
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, timestep: torch.Tensor,
                 image_rotary_emb=None) -> torch.Tensor:
         """video latent bf16 [B, F, C, H, W], text states bf16 [B, N_t, text_dim], timestep [B], rotary table

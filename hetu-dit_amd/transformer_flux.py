@@ -9,6 +9,7 @@ import torch
 from torch import nn
 
 from . import ops
+from ._lib import eager_only
 from .layers.embeddings import conditioning_embedding, norm_out_project, project
 from .layers.modules import (AdaLayerNormContinuous, CombinedTimestepGuidanceTextProjEmbeddings,
                              CombinedTimestepTextProjEmbeddings, FluxPosEmbed)
@@ -60,6 +61,7 @@ class FluxTransformer2DModel(nn.Module):
         return ops.rope_table(ids, self.pos_embed.axes_dim, self.pos_embed.theta)
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, pooled_projections: torch.Tensor,
                 timestep: torch.Tensor, img_ids: torch.Tensor, txt_ids: torch.Tensor,
                 guidance: Optional[torch.Tensor] = None) -> torch.Tensor:

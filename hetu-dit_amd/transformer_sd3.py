@@ -9,6 +9,7 @@ import torch
 from torch import nn
 
 from . import ops
+from ._lib import eager_only
 from .layers.embeddings import conditioning_embedding, hetuDiTPatchEmbedWrapper, norm_out_project, project
 from .layers.modules import AdaLayerNormContinuous, CombinedTimestepTextProjEmbeddings, PatchEmbed
 from .transformer import SD3TransformerBlocks
@@ -36,6 +37,7 @@ class SD3Transformer2DModel(nn.Module):
         return conditioning_embedding(self.time_text_embed, timestep, pooled_projections)
 
     @torch.no_grad()
+    @eager_only
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, pooled_projections: torch.Tensor,
                 timestep: torch.Tensor) -> torch.Tensor:
         """latent bf16 [B, C, H, W], text states bf16 [B, N_t, joint_dim], pooled bf16 [B, pooled_dim], timestep
@@ -50,6 +52,7 @@ class SD3Transformer2DModel(nn.Module):
         return ops.unpatchify(x, self.out_channels, H, W, self.patch_size)
 
     @torch.no_grad()
+    @eager_only
     def denoise_step(self, latents: torch.Tensor, encoder_hidden_states: torch.Tensor, pooled_projections: torch.Tensor,
                      timestep: torch.Tensor, guidance_scale: float, sigma: float, sigma_next: float) -> torch.Tensor:
         """One guided step on one GPU: the CFG pair as a batch of two per latent (unconditional first, as

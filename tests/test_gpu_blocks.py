@@ -79,6 +79,30 @@ def test_sd3_attention_wrapper_reference_api(hdit):
     assert_parity(f, feed_forward(params, "ff", x.float()), what="ff")
 
 
+def test_layer_wrappers_inside_a_compiled_caller(hdit):
+    """A traced block of the caller's own (the reference compiles diffusers' block code around the wrapped layers,
+    ``base_pipeline.py:274-279``) reaches the attention and feed-forward wrappers: Dynamo must break the graph at
+    them, run them as written and resume -- same bits as the uncompiled caller."""
+    from hetu_dit_amd import blocks, synthetic
+
+    B, N, Nt, D, H = 1, 200, 50, 256, 4
+    blk, _ = make(hdit, blocks.JointTransformerBlock, 5, D, H, 64)
+    x, e = synthetic.randn_bf16((B, N, D), 6).to(DEV), synthetic.randn_bf16((B, Nt, D), 7).to(DEV)
+
+    def caller(x, e):
+        a, ca = blk.attn(hidden_states=x * 0.5, encoder_hidden_states=e)
+        return x + a, e + ca, blk.ff(x) * 2.0
+
+    want = caller(x, e)
+    torch.cuda.synchronize()
+    torch._dynamo.reset()
+    got = torch.compile(caller, backend="eager")(x, e)
+    torch.cuda.synchronize()
+    for g_, w_ in zip(got, want):
+        assert torch.equal(g_, w_)
+    torch._dynamo.reset()
+
+
 def test_flux_double_and_single_blocks(hdit):
     from hetu_dit_amd import blocks, synthetic
     from hetu_dit_amd.runtime_state import get_runtime_state

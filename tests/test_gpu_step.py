@@ -149,6 +149,49 @@ def test_sd3_transformer_latent_to_noise(hdit):
     assert_parity(new, want.float(), what="denoise step")
 
 
+@pytest.mark.parametrize("backend", ["eager", "inductor"])
+def test_sd3_transformer_forward_under_torch_compile(hdit, backend):
+    """The reference compiles ``transformer.forward`` when ``use_torch_compile`` is set (``base_pipeline.py:274-279``).
+    The modules here are marked opaque to Dynamo (they reach the C ABI through ctypes), so the compiled callable must
+    run them as written and return the eager result bit for bit, call after call."""
+    import os
+
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.transformer_sd3 import SD3Transformer2DModel
+
+    os.environ.setdefault("TORCHINDUCTOR_COMPILE_THREADS", "1")
+    L, heads = 2, 4
+    model = SD3Transformer2DModel(sample_size=32, patch_size=2, in_channels=16, num_layers=L, attention_head_dim=64,
+                                  num_attention_heads=heads, joint_attention_dim=128, caption_projection_dim=256,
+                                  pooled_projection_dim=64, out_channels=16, pos_embed_max_size=24)
+    synthetic.init_module_(model, 7)
+    model = model.to(DEV)
+    lat = synthetic.randn_bf16((2, 16, 32, 40), 8).to(DEV)
+    enc = synthetic.randn_bf16((2, 77, 128), 9).to(DEV)
+    pooled = synthetic.randn_bf16((2, 64), 10).to(DEV)
+    t = torch.tensor([981.0, 981.0]).to(DEV)
+    want = model(lat, enc, pooled, t)
+    torch.cuda.synchronize()
+    torch._dynamo.reset()
+    compiled = torch.compile(model.forward, backend=backend)
+    for _ in range(2):
+        got = compiled(lat, enc, pooled, t)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+
+    # a compiled caller that does tensor work of its own around the transformer: traced up to the call, resumed after
+    def guided(lat, enc, pooled, t, scale):
+        noise = model(lat, enc, pooled, t)
+        u, c = noise.float().chunk(2)
+        return u + scale * (c - u)
+
+    want2 = guided(lat, enc, pooled, t, 7.0)
+    got2 = torch.compile(guided, backend=backend)(lat, enc, pooled, t, 7.0)
+    torch.cuda.synchronize()
+    assert torch.allclose(got2, want2, rtol=1e-5, atol=1e-5)
+    torch._dynamo.reset()
+
+
 def test_conv2d_wrapper_patch_convolution(hdit):
     """``hetuDiTConv2dWrapper`` (reference layers/conv.py:19-113) on one GPU: the p x p stride-p convolution
     against ``F.conv2d`` in fp32; other geometries are refused."""
