@@ -103,26 +103,42 @@ struct Lds {
 
 // One wave-wide direct-to-LDS copy: lane l's 16 bytes land at LDS byte address lds_addr + 16*l.  Inline
 // assembly, so the compiler's wait-count bookkeeping does not see it; the tile loop waits for it explicitly.
-// Issued at agent scope (sc1), which the CU's L1 never serves: the pipelined kernel waits for "all but the newest
-// n" requests and relies on completion in issue order, and a request that hits in L1 -- the rows of a clamped
-// tile, a tile requested again past the end -- completes ahead of older misses.  From L2, hits and misses
-// complete in issue order.
+// AGENT: issued at agent scope (sc1), which the CU's L1 never serves.  The pipelined kernel waits for "all but the
+// newest n" requests and relies on completion in issue order, and a request that hits in L1 -- the rows of a clamped
+// tile, a tile requested again past the end, a short sequence the previous workgroup on the CU has just read --
+// completes ahead of older misses; from L2, hits and misses complete in issue order.  The kernels that wait for
+// everything (vmcnt(0)) do not care about the order and keep the L1 (2 % faster where two workgroups of a CU read
+// the same keys).
+template <bool AGENT>
 __device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
   // the base is wave-uniform by construction; say so, or a base the compiler keeps in vector registers ends up in
   // the scalar-address operand
   const uint64_t bu = (uint64_t)base_uniform;
   const uint64_t base = ((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(bu >> 32)) << 32) |
                         (unsigned)__builtin_amdgcn_readfirstlane((int)bu);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
-               :
-               : "s"(lds_addr_uniform), "v"(voff), "s"(base)
-               : "m0", "memory");
+  if constexpr (AGENT)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
+                 :
+                 : "s"(lds_addr_uniform), "v"(voff), "s"(base)
+                 : "m0", "memory");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr_uniform), "v"(voff), "s"(base)
+                 : "m0", "memory");
 }
+template <bool AGENT>
 __device__ __forceinline__ void lds_dma16_ptr(const unsigned char* ptr_per_lane, unsigned lds_addr_uniform) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off sc1"
-               :
-               : "s"(lds_addr_uniform), "v"(ptr_per_lane)
-               : "m0", "memory");
+  if constexpr (AGENT)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off sc1"
+                 :
+                 : "s"(lds_addr_uniform), "v"(ptr_per_lane)
+                 : "m0", "memory");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_addr_uniform), "v"(ptr_per_lane)
+                 : "m0", "memory");
 }
 __device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
   return (unsigned)(uintptr_t)((const __attribute__((address_space(3))) unsigned char*)p);
@@ -247,23 +263,23 @@ __device__ __forceinline__ void attn_tracked_body(const AttnParams& P, int q_til
       const unsigned char* vb = vb0 + (int64_t)r0 * P.v.ss0 * 2;
 #pragma unroll
       for (int i = 0; i < NCH; i++) {
-        lds_dma16(kb, koff[0][i], kdst + i * 4096);
-        lds_dma16(vb, voff[0][i], vdst + i * 4096);
+        lds_dma16<false>(kb, koff[0][i], kdst + i * 4096);
+        lds_dma16<false>(vb, voff[0][i], vdst + i * 4096);
       }
     } else if (r0 >= len0 && r0 + BKV <= P.skv) {
       const unsigned char* kb = kb1 + (int64_t)(r0 - len0) * P.k.ss1 * 2;
       const unsigned char* vb = vb1 + (int64_t)(r0 - len0) * P.v.ss1 * 2;
 #pragma unroll
       for (int i = 0; i < NCH; i++) {
-        lds_dma16(kb, koff[1][i], kdst + i * 4096);
-        lds_dma16(vb, voff[1][i], vdst + i * 4096);
+        lds_dma16<false>(kb, koff[1][i], kdst + i * 4096);
+        lds_dma16<false>(vb, voff[1][i], vdst + i * 4096);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < NCH; i++) {
         const int r = min(r0 + dma_row + 4 * RPI * i, P.skv - 1);
-        lds_dma16_ptr((const unsigned char*)(row_ptr(P.k, b, h, r) + dma_kc * 8), kdst + i * 4096);
-        lds_dma16_ptr((const unsigned char*)(row_ptr(P.v, b, h, r) + dma_vc * 8), vdst + i * 4096);
+        lds_dma16_ptr<false>((const unsigned char*)(row_ptr(P.k, b, h, r) + dma_kc * 8), kdst + i * 4096);
+        lds_dma16_ptr<false>((const unsigned char*)(row_ptr(P.v, b, h, r) + dma_vc * 8), vdst + i * 4096);
       }
     }
   };
@@ -647,11 +663,11 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles,
     if (t < full0) {
       const unsigned char* kb = (const unsigned char*)(kb0 + (uint64_t)(unsigned)t * kstep0);
 #pragma unroll
-      for (int i = 0; i < NCH; i++) lds_dma16(kb + i * (4 * RPI) * krow0, koff[0], dst + i * 4096);
+      for (int i = 0; i < NCH; i++) lds_dma16<true>(kb + i * (4 * RPI) * krow0, koff[0], dst + i * 4096);
     } else if ((unsigned)(t - first1) < span1) {
       const unsigned char* kb = (const unsigned char*)(kb1 + (uint64_t)(unsigned)t * kstep1);
 #pragma unroll
-      for (int i = 0; i < NCH; i++) lds_dma16(kb + i * (4 * RPI) * krow1, koff[1], dst + i * 4096);
+      for (int i = 0; i < NCH; i++) lds_dma16<true>(kb + i * (4 * RPI) * krow1, koff[1], dst + i * 4096);
     } else {
       const int r0 = min(t, NT - 1) * BKV;
 #pragma unroll
@@ -659,7 +675,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles,
         const int r = min(r0 + dma_row + 4 * RPI * i, P.skv - 1);
         const bool in0 = r < len0;
         const uint64_t a = (in0 ? kb0 : kb1) + (uint64_t)(unsigned)r * (in0 ? krow0 : krow1) + dma_kc * 16;
-        lds_dma16_ptr((const unsigned char*)a, dst + i * 4096);
+        lds_dma16_ptr<true>((const unsigned char*)a, dst + i * 4096);
       }
     }
   };
@@ -667,11 +683,11 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles,
     if (t < full0) {
       const unsigned char* vb = (const unsigned char*)(vb0 + (uint64_t)(unsigned)t * vstep0);
 #pragma unroll
-      for (int i = 0; i < NCH; i++) lds_dma16(vb + i * (4 * RPI) * vrow0, voff[0], dst + i * 4096);
+      for (int i = 0; i < NCH; i++) lds_dma16<true>(vb + i * (4 * RPI) * vrow0, voff[0], dst + i * 4096);
     } else if ((unsigned)(t - first1) < span1) {
       const unsigned char* vb = (const unsigned char*)(vb1 + (uint64_t)(unsigned)t * vstep1);
 #pragma unroll
-      for (int i = 0; i < NCH; i++) lds_dma16(vb + i * (4 * RPI) * vrow1, voff[1], dst + i * 4096);
+      for (int i = 0; i < NCH; i++) lds_dma16<true>(vb + i * (4 * RPI) * vrow1, voff[1], dst + i * 4096);
     } else {
       const int r0 = min(t, NT - 1) * BKV;
 #pragma unroll
@@ -679,7 +695,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams& P, int q_tiles,
         const int r = min(r0 + dma_row + 4 * RPI * i, P.skv - 1);
         const bool in0 = r < len0;
         const uint64_t a = (in0 ? vb0 : vb1) + (uint64_t)(unsigned)r * (in0 ? vrow0 : vrow1) + dma_vc * 16;
-        lds_dma16_ptr((const unsigned char*)a, dst + i * 4096);
+        lds_dma16_ptr<true>((const unsigned char*)a, dst + i * 4096);
       }
     }
   };
