@@ -271,6 +271,37 @@ __global__ void __launch_bounds__(256) gelu_kernel(const __bf16* __restrict__ x,
 }
 
 // ---------------------------------------------------------------------------
+// The feed-forward activations that are not fused into a GEMM epilogue, applied to the first projection's output
+// (bias already added): exact GELU, GEGLU (value half times exact GELU of the gate half), SiLU.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_erf_f(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f)); }
+
+template <int KIND>
+__global__ void __launch_bounds__(256) ff_activation_kernel(const __bf16* __restrict__ x, __bf16* __restrict__ y,
+                                                            int64_t total_chunks, int chunks_per_row, int64_t ldx,
+                                                            int64_t ldy) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total_chunks) return;
+  int64_t row = i / chunks_per_row;
+  int c = (int)(i - row * chunks_per_row);
+  float f[8];
+  unpack8(*(const i32x4*)(x + row * ldx + c * 8), f);
+  if constexpr (KIND == HDIT_ACT_GEGLU) {
+    float gte[8];
+    unpack8(*(const i32x4*)(x + row * ldx + (int64_t)(chunks_per_row + c) * 8), gte);
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] *= gelu_erf_f(gte[e]);
+  } else if constexpr (KIND == HDIT_ACT_GELU_ERF) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] = gelu_erf_f(f[e]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] = hdit::silu_f(f[e]);
+  }
+  *(i32x4*)(y + row * ldy + c * 8) = pack8(f);
+}
+
+// ---------------------------------------------------------------------------
 // adaLN projection: out[b, n] = W[n, :] . silu(temb[b, :]) + bias[n]
 // One wave per output row; the weight row is streamed once for all batches.
 // ---------------------------------------------------------------------------
@@ -560,6 +591,27 @@ extern "C" __attribute__((visibility("default"))) int hdit_gelu_tanh(const void*
   hipLaunchKernelGGL(gelu_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                      (const __bf16*)x, (const __bf16*)bias, (__bf16*)y, total, dim / 8, ldx, ldy);
   return hdit_host::check_launch("hdit_gelu_tanh");
+}
+
+extern "C" __attribute__((visibility("default"))) int hdit_ff_activation(const void* x, void* y, int64_t rows, int dim, int64_t ldx, int64_t ldy,
+                                  int kind, void* stream) {
+  if (!x || !y || rows < 0 || dim <= 0 || dim % 8 || ldx % 8 || ldy % 8) return HDIT_EINVAL;
+  if (!aligned16(x) || !aligned16(y)) return HDIT_EINVAL;
+  if (kind != HDIT_ACT_GELU_ERF && kind != HDIT_ACT_GEGLU && kind != HDIT_ACT_SILU) return HDIT_EINVAL;
+  if (ldx < (kind == HDIT_ACT_GEGLU ? 2 : 1) * (int64_t)dim || ldy < dim) return HDIT_EINVAL;
+  // in place only where an element is read by the thread that writes it (not GEGLU: other threads read the gate half)
+  if (x == y && kind == HDIT_ACT_GEGLU) return HDIT_EINVAL;
+  const int64_t total = rows * (dim / 8);
+  if (total == 0) return HDIT_OK;
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  if (kind == HDIT_ACT_GELU_ERF)
+    hipLaunchKernelGGL(ff_activation_kernel<HDIT_ACT_GELU_ERF>, grid, block, 0, s, (const __bf16*)x, (__bf16*)y, total, dim / 8, ldx, ldy);
+  else if (kind == HDIT_ACT_GEGLU)
+    hipLaunchKernelGGL(ff_activation_kernel<HDIT_ACT_GEGLU>, grid, block, 0, s, (const __bf16*)x, (__bf16*)y, total, dim / 8, ldx, ldy);
+  else
+    hipLaunchKernelGGL(ff_activation_kernel<HDIT_ACT_SILU>, grid, block, 0, s, (const __bf16*)x, (__bf16*)y, total, dim / 8, ldx, ldy);
+  return hdit_host::check_launch("hdit_ff_activation");
 }
 
 extern "C" __attribute__((visibility("default"))) int hdit_adaln_gemv(const void* temb, const void* w, const void* bias, float* out, int batch, int n, int k,

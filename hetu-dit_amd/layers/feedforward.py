@@ -1,9 +1,12 @@
 """FeedForward wrapper with the interface of the reference's
-``layers/feedforward.py:17-78``: wraps ``net = [GELU(proj), Dropout, Linear]``,
-slices ``net[0].proj`` rows / ``net[2]`` columns by tensor-parallel rank, moves
-``net[2].bias`` to ``self.output_bias`` (added after the reduce).  ``forward``
-is two GEMM launches: bias + GELU-tanh fused into the first epilogue, the
-output bias (and optionally the block's gated residual) into the second."""
+``layers/feedforward.py:17-78``: wraps ``net = [activation(proj), Dropout, Linear]``,
+slices ``net[0].proj`` rows / ``net[2]`` columns by tensor-parallel rank (the two
+halves of a GEGLU projection separately, ``:34-46``), moves ``net[2].bias`` to
+``self.output_bias`` (added after the reduce).  With the tanh GELU every model here
+uses, ``forward`` is two GEMM launches: bias + GELU-tanh fused into the first
+epilogue, the output bias (and optionally the block's gated residual) into the
+second.  The other first layers the reference accepts (exact GELU, GEGLU,
+LinearActivation) take a bias-only first GEMM and one elementwise launch."""
 import torch
 from torch import nn
 
@@ -11,7 +14,7 @@ from .. import ops
 from ..parallel_state import get_tensor_model_parallel_rank, get_tensor_model_parallel_world_size, get_tp_group
 from ..registry import hetuDiTLayerWrappersRegister
 from .base_layer import hetuDiTDiffusionLayerBaseWrapper
-from .modules import GELU, FeedForward
+from .modules import GEGLU, GELU, FeedForward, LinearActivation
 
 
 @hetuDiTLayerWrappersRegister.register(FeedForward)
@@ -21,14 +24,23 @@ class hetuDiTFeedForwardWrapper(hetuDiTDiffusionLayerBaseWrapper):
         tp_degree = get_tensor_model_parallel_world_size()
         tp_rank = get_tensor_model_parallel_rank()
         act = self.module.net[0]
-        if isinstance(act, GELU):
+        if isinstance(act, (GELU, LinearActivation)):
             act.proj.weight.data = act.proj.weight.data.chunk(tp_degree, dim=0)[tp_rank]
             if act.proj.bias is not None:
                 act.proj.bias.data = act.proj.bias.data.chunk(tp_degree, dim=0)[tp_rank]
+        elif isinstance(act, GEGLU):
+            # value half and gate half are sliced separately and joined again
+            act.proj.weight.data = torch.cat([h.chunk(tp_degree, dim=0)[tp_rank] for h in act.proj.weight.data.chunk(2, dim=0)], dim=0)
+            if act.proj.bias is not None:
+                act.proj.bias.data = torch.cat([h.chunk(tp_degree, dim=0)[tp_rank] for h in act.proj.bias.data.chunk(2, dim=0)], dim=0)
         else:
             raise TypeError(f"activation_fn {type(act)} not supported")
-        if getattr(act, "approximate", "tanh") != "tanh":
-            raise TypeError("only GELU(approximate='tanh') is built")
+        if isinstance(act, GELU) and act.approximate not in ("tanh", "none"):
+            raise TypeError(f"GELU(approximate={act.approximate!r}) is not built")
+        # the activation that follows the first projection: None = tanh GELU, fused into that GEMM's epilogue
+        self.activation_kind = (None if isinstance(act, GELU) and act.approximate == "tanh" else
+                                ops.ACT_GELU_ERF if isinstance(act, GELU) else
+                                ops.ACT_GEGLU if isinstance(act, GEGLU) else ops.ACT_SILU)
         self.module.net[2].weight.data = self.module.net[2].weight.chunk(tp_degree, dim=1)[tp_rank]
         self.has_output_bias = False
         if self.module.net[2].bias is not None:
@@ -39,6 +51,8 @@ class hetuDiTFeedForwardWrapper(hetuDiTDiffusionLayerBaseWrapper):
     # -- problems, so that both streams of a joint block share launches ---------
     def in_problem(self, x2: torch.Tensor):
         """x2 [rows, D] -> (problem, h [rows, F]) with bias + GELU-tanh epilogue."""
+        if self.activation_kind is not None:
+            raise TypeError("the blocks fuse the tanh GELU into the first GEMM; other activations go through forward()")
         proj = self.module.net[0].proj
         h = torch.empty(x2.shape[0], proj.weight.shape[0], dtype=torch.bfloat16, device=x2.device)
         bias = proj.bias.data if proj.bias is not None else None
@@ -55,8 +69,15 @@ class hetuDiTFeedForwardWrapper(hetuDiTDiffusionLayerBaseWrapper):
     def forward(self, hidden_states: torch.Tensor, *args, **kwargs) -> torch.Tensor:
         x = hidden_states if hidden_states.is_contiguous() else hidden_states.contiguous()
         x2 = x.view(-1, x.shape[-1])
-        p1, h = self.in_problem(x2)
-        ops.gemm_launch([p1])
+        if self.activation_kind is None:
+            p1, h = self.in_problem(x2)
+            ops.gemm_launch([p1])
+        else:
+            proj = self.module.net[0].proj
+            h = torch.empty(x2.shape[0], proj.weight.shape[0], dtype=torch.bfloat16, device=x2.device)
+            ops.gemm_launch([ops.gemm_problem(x2, proj.weight.data, h, proj.bias.data if proj.bias is not None else None)])
+            # exact GELU and SiLU in place; GEGLU into a buffer of half the width
+            h = ops.ff_activation(h, self.activation_kind, out=None if self.activation_kind == ops.ACT_GEGLU else h)
         out = torch.empty(*x.shape[:-1], self.module.net[2].weight.shape[0], dtype=torch.bfloat16, device=x.device)
         ops.gemm_launch([self.out_problem(h, out.view(-1, out.shape[-1]))])
         get_tp_group().all_reduce(out)

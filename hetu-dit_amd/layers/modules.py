@@ -93,16 +93,45 @@ class GELU(nn.Module):
         self.approximate = approximate
 
 
+class GEGLU(nn.Module):
+    """``proj`` to twice the width; value half times exact GELU of the gate half."""
+
+    def __init__(self, dim_in: int, dim_out: int, bias: bool = True):
+        super().__init__()
+        self.proj = nn.Linear(dim_in, dim_out * 2, bias=bias)
+
+
+class LinearActivation(nn.Module):
+    """``proj`` followed by SiLU."""
+
+    def __init__(self, dim_in: int, dim_out: int, bias: bool = True, activation: str = "silu"):
+        super().__init__()
+        if activation != "silu":
+            raise ValueError("LinearActivation: only 'silu' is built")
+        self.proj = nn.Linear(dim_in, dim_out, bias=bias)
+        self.activation = activation
+
+
 class FeedForward(nn.Module):
-    """``net = [GELU(proj), Dropout, Linear]`` (activation_fn="gelu-approximate")."""
+    """``net = [activation(proj), Dropout, Linear]``; ``activation_fn`` as in diffusers: "gelu-approximate" (what
+    every model here uses), "gelu", "geglu", "linear-silu"."""
 
     def __init__(self, dim: int, dim_out: Optional[int] = None, mult: int = 4, inner_dim: Optional[int] = None,
-                 bias: bool = True):
+                 bias: bool = True, activation_fn: str = "gelu-approximate"):
         super().__init__()
         inner_dim = inner_dim or dim * mult
         dim_out = dim_out or dim
-        self.net = nn.ModuleList([GELU(dim, inner_dim, approximate="tanh", bias=bias), nn.Dropout(0.0),
-                                  nn.Linear(inner_dim, dim_out, bias=bias)])
+        if activation_fn == "gelu-approximate":
+            act = GELU(dim, inner_dim, approximate="tanh", bias=bias)
+        elif activation_fn == "gelu":
+            act = GELU(dim, inner_dim, approximate="none", bias=bias)
+        elif activation_fn == "geglu":
+            act = GEGLU(dim, inner_dim, bias=bias)
+        elif activation_fn == "linear-silu":
+            act = LinearActivation(dim, inner_dim, bias=bias)
+        else:
+            raise ValueError(f"activation_fn {activation_fn!r} is not built")
+        self.net = nn.ModuleList([act, nn.Dropout(0.0), nn.Linear(inner_dim, dim_out, bias=bias)])
 
 
 class AdaLayerNormZero(nn.Module):

@@ -814,6 +814,28 @@ def adaln_gemv(temb: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
     return out
 
 
+ACT_GELU_ERF, ACT_GEGLU, ACT_SILU = 0, 1, 2
+
+
+def ff_activation(x: torch.Tensor, kind: int, out=None) -> torch.Tensor:
+    """The feed-forward activations without a fused GEMM epilogue, on the first projection's output ``x [..., n]``
+    (bias already added): exact GELU and SiLU keep the width (and may run in place, ``out=x``), GEGLU halves it."""
+    _need(x, bf16, "x")
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(1) != 1:
+        raise ValueError("x needs a unit inner stride")
+    dim = x2.shape[1] // 2 if kind == ACT_GEGLU else x2.shape[1]
+    if kind == ACT_GEGLU and x2.shape[1] % 2:
+        raise ValueError("GEGLU needs an even width")
+    if out is None:
+        out = torch.empty(*x.shape[:-1], dim, dtype=bf16, device=x.device)
+    o2 = out.view(-1, dim)
+    rows = x2.shape[0]
+    check(_lib.lib().hdit_ff_activation(x2.data_ptr(), o2.data_ptr(), rows, dim, x2.stride(0) if rows > 1 else x2.shape[1],
+                                        o2.stride(0) if rows > 1 else dim, kind, _stream()), "hdit_ff_activation")
+    return out
+
+
 def gelu_tanh(x: torch.Tensor, bias: Optional[torch.Tensor] = None, out=None) -> torch.Tensor:
     _need(x, bf16, "x")
     x2 = x.reshape(-1, x.shape[-1])

@@ -243,6 +243,19 @@ int hdit_adaln_gemv(const void* temb, const void* w, const void* bias, float* ou
 int hdit_gelu_tanh(const void* x, const void* bias, void* y, int64_t rows, int dim, int64_t ldx,
                    int64_t ldy, void* stream);
 
+/* The feed-forward activations that have no fused GEMM epilogue, applied to the first projection's output
+ * x [rows, ldx] (bias already added) -> y [rows, dim] (bf16):
+ *   HDIT_ACT_GELU_ERF  y = gelu(x), exact          diffusers GELU(approximate="none")
+ *   HDIT_ACT_GEGLU     y = x[:, :dim] * gelu(x[:, dim:2*dim])   diffusers GEGLU
+ *   HDIT_ACT_SILU      y = silu(x)                 diffusers LinearActivation
+ * the first-layer classes layers/feedforward.py:25-57 accepts besides the tanh GELU.  In place (y == x) except
+ * for GEGLU. */
+#define HDIT_ACT_GELU_ERF 0
+#define HDIT_ACT_GEGLU 1
+#define HDIT_ACT_SILU 2
+int hdit_ff_activation(const void* x, void* y, int64_t rows, int dim, int64_t ldx, int64_t ldy, int kind,
+                       void* stream);
+
 /* In-place per-head QK normalisation + rotary embedding on x[b, s, h, :]
  * (bf16, strides as in hdit_seq_segment, head_dim 64 or 128):
  *   norm_kind 0: none; 1: RMSNorm(eps, weight); 2: LayerNorm(eps, weight, bias)

@@ -27,6 +27,9 @@ therefore pinned by what mathematics and PyTorch's own library routines fix
 * ``layer_norm``        -- ``F.layer_norm``; zero-mean / unit-variance invariant
 * ``rms_norm``          -- ``F.rms_norm``; scale invariance
 * ``gelu_tanh``         -- ``F.gelu(approximate="tanh")``; values at 0, +-1, large |x|
+* ``gelu_erf``          -- ``F.gelu``, ``math.erf`` point by point, the identity gelu(x) - gelu(-x) = x;
+                           ``feed_forward`` with "gelu" / "geglu" / "linear-silu" against a chain of
+                           ``F.linear`` / ``F.gelu`` / ``F.silu`` with mutations (swapped halves, tanh for erf)
 * ``silu``              -- ``F.silu``
 * ``attention``         -- ``F.scaled_dot_product_attention`` (math backend), numpy
                            brute force, rows-sum-to-one, constant-V, KV permutation
@@ -68,6 +71,7 @@ therefore pinned by what mathematics and PyTorch's own library routines fix
 
 from .ops import (  # noqa: F401
     silu,
+    gelu_erf,
     gelu_tanh,
     linear,
     layer_norm,

@@ -22,11 +22,13 @@ from .ops import (
     adaln_modulation,
     apply_rotary_emb,
     attention,
+    gelu_erf,
     gelu_tanh,
     layer_norm,
     linear,
     modulate,
     rms_norm,
+    silu,
 )
 
 P = Dict[str, torch.Tensor]
@@ -48,11 +50,23 @@ def _unheads(x: torch.Tensor) -> torch.Tensor:
     return x.transpose(1, 2).reshape(b, s, h * d)
 
 
-def feed_forward(p: P, prefix: str, x: torch.Tensor) -> torch.Tensor:
-    """``net = [GELU(proj, approximate="tanh"), Dropout, Linear]`` -- the
-    module ``hetuDiTFeedForwardWrapper`` wraps (``layers/feedforward.py:17-78``);
-    at one GPU the detached output bias is simply added back (``:75-77``)."""
-    h = gelu_tanh(_lin(p, prefix + ".net.0.proj", x))
+def feed_forward(p: P, prefix: str, x: torch.Tensor, activation_fn: str = "gelu-approximate") -> torch.Tensor:
+    """``net = [activation(proj), Dropout, Linear]`` -- the module ``hetuDiTFeedForwardWrapper`` wraps
+    (``layers/feedforward.py:17-78``); at one GPU the detached output bias is simply added back (``:75-77``).
+    ``activation_fn`` as diffusers names the first-layer classes the wrapper accepts (``:25-57``): tanh GELU (every
+    model on this path), exact GELU, GEGLU (value half times exact GELU of the gate half), LinearActivation (SiLU)."""
+    h = _lin(p, prefix + ".net.0.proj", x)
+    if activation_fn == "gelu-approximate":
+        h = gelu_tanh(h)
+    elif activation_fn == "gelu":
+        h = gelu_erf(h)
+    elif activation_fn == "geglu":
+        value, gate_half = h.chunk(2, dim=-1)
+        h = value * gelu_erf(gate_half)
+    elif activation_fn == "linear-silu":
+        h = silu(h)
+    else:
+        raise ValueError(activation_fn)
     return _lin(p, prefix + ".net.2", h)
 
 

@@ -33,6 +33,14 @@ def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
     return 0.5 * x * (1.0 + torch.tanh(c * (x + 0.044715 * x * x * x)))
 
 
+def gelu_erf(x: torch.Tensor) -> torch.Tensor:
+    """x Phi(x) = 0.5 x (1 + erf(x / sqrt 2)): ``F.gelu`` without approximation, what diffusers' ``GELU(approximate=
+    "none")`` and the gate of ``GEGLU`` compute -- first-layer classes the reference's FeedForward wrapper accepts
+    (``layers/feedforward.py:25-46``)."""
+    x = _f32(x)
+    return 0.5 * x * (1.0 + torch.erf(x * (1.0 / math.sqrt(2.0))))
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x W^T + b (``nn.Linear``; the projections at
     ``layers/attention_processor.py:688-695,:844-846,:1054-1056``)."""

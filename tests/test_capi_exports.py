@@ -30,7 +30,7 @@ def library():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for name in ("hdit_gemm_bf16", "hdit_attn_fwd_bf16", "hdit_attn_fwd_fp8", "hdit_attn_absmax",
-                 "hdit_layernorm_modulate", "hdit_layernorm_modulate_jobs", "hdit_gate_residual", "hdit_adaln_gemv", "hdit_gelu_tanh",
+                 "hdit_layernorm_modulate", "hdit_layernorm_modulate_jobs", "hdit_gate_residual", "hdit_adaln_gemv", "hdit_gelu_tanh", "hdit_ff_activation",
                  "hdit_qk_norm_rope", "hdit_copy_rows", "hdit_patchify", "hdit_unpatchify", "hdit_timestep_embedding",
                  "hdit_silu", "hdit_cfg_euler_step",
     "hdit_rope_table", "hdit_clock_sample", "hdit_gemm_force_config", "hdit_abi_version", "hdit_last_error"):

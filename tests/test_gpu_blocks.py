@@ -103,6 +103,48 @@ def test_layer_wrappers_inside_a_compiled_caller(hdit):
     torch._dynamo.reset()
 
 
+@pytest.mark.parametrize("activation_fn", ["gelu", "geglu", "linear-silu", "gelu-approximate"])
+def test_feed_forward_wrapper_other_first_layers(hdit, activation_fn):
+    """hetuDiTFeedForwardWrapper over the first-layer classes the reference's wrapper accepts
+    (``layers/feedforward.py:25-57``): exact GELU, GEGLU, LinearActivation, beside the tanh GELU of the models."""
+    from hetu_dit_amd import synthetic
+    from hetu_dit_amd.base_model import wrap_layer
+    from hetu_dit_amd.layers.modules import FeedForward
+    from oracle.blocks import feed_forward
+
+    print(f"ff wrapper activation_fn={activation_fn}", flush=True)
+    D, Fi = 256, 640
+    ff = FeedForward(D, inner_dim=Fi, activation_fn=activation_fn)
+    synthetic.init_module_(ff, 31, std=0.1)
+    params = {"ff." + k: v.detach().float() for k, v in ff.state_dict().items()}
+    wrapped = wrap_layer(ff).to(DEV)
+    x = synthetic.randn_bf16((2, 333, D), 32)
+    got = wrapped(x.to(DEV))
+    torch.cuda.synchronize()
+    assert got.shape == x.shape
+    assert_parity(got, feed_forward(params, "ff", x.float(), activation_fn=activation_fn), what=f"ff {activation_fn}")
+    if activation_fn != "gelu-approximate":
+        with pytest.raises(TypeError):
+            wrapped.in_problem(x.to(DEV).view(-1, D))
+
+
+def test_ff_activation_entry_point_refusals(hdit):
+    import ctypes as C
+
+    lib = hdit._lib.lib()
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device=DEV)
+    y = torch.zeros(4, 32, dtype=torch.bfloat16, device=DEV)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ok = lib.hdit_ff_activation(x.data_ptr(), y.data_ptr(), 4, 32, 64, 32, hdit.ops.ACT_GEGLU, st)
+    assert ok == 0
+    assert lib.hdit_ff_activation(x.data_ptr(), x.data_ptr(), 4, 32, 64, 64, hdit.ops.ACT_GEGLU, st) != 0  # in place
+    assert lib.hdit_ff_activation(x.data_ptr(), y.data_ptr(), 4, 32, 32, 32, hdit.ops.ACT_GEGLU, st) != 0  # no gate half
+    assert lib.hdit_ff_activation(x.data_ptr(), y.data_ptr(), 4, 32, 64, 32, 7, st) != 0                  # unknown kind
+    assert lib.hdit_ff_activation(x.data_ptr(), y.data_ptr(), 4, 30, 64, 32, hdit.ops.ACT_SILU, st) != 0    # width % 8
+    assert lib.hdit_ff_activation(x.data_ptr(), x.data_ptr(), 4, 64, 64, 64, hdit.ops.ACT_SILU, st) == 0    # in place ok
+    torch.cuda.synchronize()
+
+
 def test_flux_double_and_single_blocks(hdit):
     from hetu_dit_amd import blocks, synthetic
     from hetu_dit_amd.runtime_state import get_runtime_state

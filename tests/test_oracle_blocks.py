@@ -1,6 +1,7 @@
 """Pins on the oracle's block wiring that do not need the reference: adaLN-"Zero" identity, call-site
 conventions the reference fixes (joint order, return order, split points), reduction of the stale-KV
 patch path to the full-sequence path, and cross-checks between block families."""
+import pytest
 import torch
 
 import oracle
@@ -164,3 +165,30 @@ def test_feed_forward_against_library():
     want = F.linear(F.gelu(F.linear(x, p["ff.net.0.proj.weight"], p["ff.net.0.proj.bias"]), approximate="tanh"),
                     p["ff.net.2.weight"], p["ff.net.2.bias"])
     torch.testing.assert_close(oracle.feed_forward(p, "ff", x), want, rtol=1e-5, atol=1e-5)
+
+
+def test_feed_forward_other_first_layers_against_library():
+    """The first-layer classes the reference's wrapper accepts besides the tanh GELU (``layers/feedforward.py:25-57``),
+    each against a chain of library calls, and each mutation of that chain (tanh for erf, halves swapped, gate not
+    activated) must break the agreement."""
+    D, Fi = 16, 48
+    F = torch.nn.functional
+    x = torch.randn(2, 5, D)
+    for name, width in (("gelu", Fi), ("geglu", 2 * Fi), ("linear-silu", Fi)):
+        p = _params({"ff.net.0.proj.weight": (width, D), "ff.net.0.proj.bias": (width,), "ff.net.2.weight": (D, Fi),
+                     "ff.net.2.bias": (D,)}, seed=17, std=0.5)
+        h = F.linear(x, p["ff.net.0.proj.weight"], p["ff.net.0.proj.bias"])
+        if name == "gelu":
+            good, bad = F.gelu(h), [F.gelu(h, approximate="tanh"), F.silu(h)]
+        elif name == "geglu":
+            a, g = h.chunk(2, dim=-1)
+            good, bad = a * F.gelu(g), [g * F.gelu(a), a * g, a * F.gelu(g, approximate="tanh"), F.gelu(a) * g]
+        else:
+            good, bad = F.silu(h), [F.gelu(h), h]
+        out = lambda hh: F.linear(hh, p["ff.net.2.weight"], p["ff.net.2.bias"])  # noqa: E731
+        got = oracle.feed_forward(p, "ff", x, activation_fn=name)
+        torch.testing.assert_close(got, out(good), rtol=1e-5, atol=1e-5)
+        for b in bad:
+            assert (got - out(b)).abs().max().item() > 1e-4, name
+    with pytest.raises(ValueError):
+        oracle.feed_forward(p, "ff", x, activation_fn="swiglu")

@@ -49,6 +49,19 @@ def test_rms_norm_matches_library():
     close(ops.rms_norm(x * 5.0, 0.0), ops.rms_norm(x, 0.0), 1e-5)
 
 
+def test_gelu_erf_pinned_by_library_erf_and_symmetry():
+    import math
+
+    x = torch.linspace(-6, 6, 101)
+    close(ops.gelu_erf(x), F.gelu(x), 1e-6)
+    for v in (-3.0, -1.0, -0.25, 0.0, 0.5, 1.0, 2.5):
+        want = 0.5 * v * (1.0 + math.erf(v / math.sqrt(2.0)))
+        assert abs(ops.gelu_erf(torch.tensor([v])).item() - want) < 1e-6
+    close(ops.gelu_erf(x) - ops.gelu_erf(-x), x, 1e-5)  # x Phi(x) + x Phi(-x) = x
+    # it is not the tanh form: the two differ by up to 2e-4 around |x| = 2
+    assert (ops.gelu_erf(x) - ops.gelu_tanh(x)).abs().max().item() > 1e-4
+
+
 def test_gelu_tanh_and_silu():
     x = torch.linspace(-6, 6, 101)
     close(ops.gelu_tanh(x), F.gelu(x, approximate="tanh"), 1e-6)
