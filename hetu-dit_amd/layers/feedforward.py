@@ -24,23 +24,33 @@ class hetuDiTFeedForwardWrapper(hetuDiTDiffusionLayerBaseWrapper):
         tp_degree = get_tensor_model_parallel_world_size()
         tp_rank = get_tensor_model_parallel_rank()
         act = self.module.net[0]
-        if isinstance(act, (GELU, LinearActivation)):
+        # The first layer is recognised by class or, for diffusers' own instances, by class name: what is used of
+        # it is ``proj`` and, for GELU, ``approximate`` (diffusers' default there is "none").
+        name = type(act).__name__
+        is_gelu = isinstance(act, GELU) or name == "GELU"
+        is_geglu = isinstance(act, GEGLU) or name == "GEGLU"
+        is_linear_act = isinstance(act, LinearActivation) or name == "LinearActivation"
+        if is_gelu or is_linear_act:
             act.proj.weight.data = act.proj.weight.data.chunk(tp_degree, dim=0)[tp_rank]
             if act.proj.bias is not None:
                 act.proj.bias.data = act.proj.bias.data.chunk(tp_degree, dim=0)[tp_rank]
-        elif isinstance(act, GEGLU):
+        elif is_geglu:
             # value half and gate half are sliced separately and joined again
             act.proj.weight.data = torch.cat([h.chunk(tp_degree, dim=0)[tp_rank] for h in act.proj.weight.data.chunk(2, dim=0)], dim=0)
             if act.proj.bias is not None:
                 act.proj.bias.data = torch.cat([h.chunk(tp_degree, dim=0)[tp_rank] for h in act.proj.bias.data.chunk(2, dim=0)], dim=0)
         else:
             raise TypeError(f"activation_fn {type(act)} not supported")
-        if isinstance(act, GELU) and act.approximate not in ("tanh", "none"):
-            raise TypeError(f"GELU(approximate={act.approximate!r}) is not built")
+        approximate = getattr(act, "approximate", "none") if is_gelu else None
+        if is_gelu and approximate not in ("tanh", "none"):
+            raise TypeError(f"GELU(approximate={approximate!r}) is not built")
+        if is_linear_act:
+            fn = getattr(act, "activation", "silu")
+            if not (fn == "silu" or isinstance(fn, nn.SiLU)):
+                raise TypeError(f"LinearActivation({fn!r}): only SiLU is built")
         # the activation that follows the first projection: None = tanh GELU, fused into that GEMM's epilogue
-        self.activation_kind = (None if isinstance(act, GELU) and act.approximate == "tanh" else
-                                ops.ACT_GELU_ERF if isinstance(act, GELU) else
-                                ops.ACT_GEGLU if isinstance(act, GEGLU) else ops.ACT_SILU)
+        self.activation_kind = (None if approximate == "tanh" else ops.ACT_GELU_ERF if is_gelu else
+                                ops.ACT_GEGLU if is_geglu else ops.ACT_SILU)
         self.module.net[2].weight.data = self.module.net[2].weight.chunk(tp_degree, dim=1)[tp_rank]
         self.has_output_bias = False
         if self.module.net[2].bias is not None:

@@ -295,3 +295,51 @@ def test_torch_library_ops_have_fake_kernels():
         cos, sin = torch.ops.hdit.rope_table(torch.empty(9, 3, dtype=torch.float32, device="cuda"), [16, 56, 56])
         assert cos.shape == sin.shape == (9, 128) and cos.dtype == torch.float32
         assert torch.ops.hdit.cfg_euler_step(lat, lat, lat, 7.0, 1.0, 0.9).shape == lat.shape
+
+
+def test_feed_forward_wrapper_recognises_foreign_first_layers_and_slices_geglu_per_half(monkeypatch):
+    """The wrapper reads a first layer by class name as well as by class (an instance of diffusers' own ``GELU`` /
+    ``GEGLU`` / ``LinearActivation`` is not an instance of the classes here), takes diffusers' ``approximate="none"``
+    default, slices the value and gate halves of a GEGLU projection separately per tensor-parallel rank
+    (reference ``layers/feedforward.py:34-46``) and refuses what it has no kernel for."""
+    from hetu_dit_amd import ops
+    from hetu_dit_amd.layers import feedforward as ffmod
+    from hetu_dit_amd.layers.feedforward import hetuDiTFeedForwardWrapper
+
+    def foreign(name, width, **attrs):
+        cls = type(name, (nn.Module,), {})
+        m = cls()
+        m.proj = nn.Linear(8, width)
+        for k, v in attrs.items():
+            setattr(m, k, v)
+        return m
+
+    def ff_with(first, inner):
+        ff = nn.Module()
+        ff.net = nn.ModuleList([first, nn.Dropout(0.0), nn.Linear(inner, 8)])
+        return ff
+
+    assert hetuDiTFeedForwardWrapper(ff_with(foreign("GELU", 16, approximate="tanh"), 16)).activation_kind is None
+    assert hetuDiTFeedForwardWrapper(ff_with(foreign("GELU", 16, approximate="none"), 16)).activation_kind == ops.ACT_GELU_ERF
+    assert hetuDiTFeedForwardWrapper(ff_with(foreign("GELU", 16), 16)).activation_kind == ops.ACT_GELU_ERF
+    assert hetuDiTFeedForwardWrapper(ff_with(foreign("GEGLU", 32), 16)).activation_kind == ops.ACT_GEGLU
+    assert hetuDiTFeedForwardWrapper(ff_with(foreign("LinearActivation", 16, activation=nn.SiLU()), 16)).activation_kind == ops.ACT_SILU
+    with pytest.raises(TypeError):
+        hetuDiTFeedForwardWrapper(ff_with(foreign("LinearActivation", 16, activation=nn.ReLU()), 16))
+    with pytest.raises(TypeError):
+        hetuDiTFeedForwardWrapper(ff_with(foreign("SwiGLU", 32), 16))
+    with pytest.raises(TypeError):
+        hetuDiTFeedForwardWrapper(ff_with(foreign("GELU", 16, approximate="sigmoid"), 16))
+
+    # rank 1 of 2: rows [4, 8) of the value half followed by rows [4, 8) of the gate half; net[2] keeps columns [4, 8)
+    monkeypatch.setattr(ffmod, "get_tensor_model_parallel_world_size", lambda: 2)
+    monkeypatch.setattr(ffmod, "get_tensor_model_parallel_rank", lambda: 1)
+    first = foreign("GEGLU", 16)
+    w, b = first.proj.weight.data.clone(), first.proj.bias.data.clone()
+    ff = ff_with(first, 8)
+    w2 = ff.net[2].weight.data.clone()
+    wrapped = hetuDiTFeedForwardWrapper(ff)
+    assert torch.equal(wrapped.module.net[0].proj.weight.data, torch.cat([w[4:8], w[12:16]]))
+    assert torch.equal(wrapped.module.net[0].proj.bias.data, torch.cat([b[4:8], b[12:16]]))
+    assert torch.equal(wrapped.module.net[2].weight.data, w2[:, 4:8])
+    assert wrapped.has_output_bias and wrapped.module.net[2].bias is None
