@@ -452,16 +452,18 @@ def test_gemm_more_problems_than_one_call_takes(hdit):
 
 def test_gemm_random_shapes_and_epilogues(hdit):
     """Seeded sweep over ragged m / n, short and long k, every tile shape and epilogue, one to three problems
-    per call."""
+    per call; the caches are flushed before every launch, so that operands arrive with HBM latency and the
+    slab pipelines' waits are what keeps a tile from running ahead of its data."""
     import random
 
     rng = random.Random(7)
     ops = hdit.ops
     lib = hdit._lib.lib()
+    flush = torch.empty(1 << 28, dtype=torch.int32, device=DEV)  # 1 GiB: four times the last-level cache
     try:
-        for it in range(40):
-            cfg = rng.choice([-1, 0, 1, 2, 3, 4, 0, 3])
-            k = 64 * rng.randint(1, 7)
+        for it in range(48):
+            cfg = rng.choice([-1, 0, 1, 2, 3, 4, 0, 3, 2])
+            k = 1536 if rng.random() < 0.25 else 64 * rng.randint(1, 7)
             probs, checks = [], []
             for j in range(rng.choice([1, 1, 2, 3])):
                 m = rng.choice([1, 7, 130, 255, 257, 600, 1000])
@@ -485,6 +487,8 @@ def test_gemm_random_shapes_and_epilogues(hdit):
                 checks.append((out, want, f"case {it} cfg {cfg} m={m} n={n} k={k} {epi}"))
             print(f"gemm random case {it}: cfg={cfg} k={k} problems={len(probs)}", flush=True)
             lib.hdit_gemm_force_config(cfg)
+            flush.fill_(it)
+            torch.cuda.synchronize()
             ops.gemm_launch(probs)
             torch.cuda.synchronize()
             for out, want, what in checks:
@@ -499,6 +503,7 @@ def test_attention_random_shapes(hdit):
     import random
 
     rng = random.Random(11)
+    flush = torch.empty(1 << 28, dtype=torch.int32, device=DEV)  # operands from HBM, as in the GEMM sweep
     for it in range(30):
         hd = rng.choice([64, 128])
         B, H = rng.choice([1, 2]), rng.choice([1, 3, 4, 8])
@@ -512,7 +517,10 @@ def test_attention_random_shapes(hdit):
             ks, vs = [kd[:, :c], kd[:, c:]], [vd[:, :c], vd[:, c:]]
         else:
             ks, vs = [kd], [vd]
-        (o,) = hdit.ops.attention([g(q)], ks, vs)
+        gq = g(q)
+        flush.fill_(it)
+        torch.cuda.synchronize()
+        (o,) = hdit.ops.attention([gq], ks, vs)
         torch.cuda.synchronize()
         want = O.attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
         assert_parity(o, want, what=f"attention random case {it}")
