@@ -76,7 +76,7 @@ struct Cfg {
   // DMA: the 256-row shapes take their operand slabs straight from global memory into LDS
   // (global_load_lds_dwordx4: no staging registers, no ds_write).  A has three slots (requested two slabs
   // ahead), B two (requested one slab ahead, first in the queue); the epilogue windows alias the A slot the
-  // tile's last slab vacated, which is exactly as large.  The bias slots exist when they still fit.
+  // tile's last slab vacated, which is exactly as large.
   static constexpr bool DMA = TM == 4;
   static constexpr int A_SLOTS = 3, B_SLOTS = 2;
   static constexpr int B_OFF = A_SLOTS * A_BYTES;
@@ -88,9 +88,7 @@ struct Cfg {
   static constexpr bool RING = TM == 2 && TN == 2;
   static constexpr int NS = RING ? 4 : 2;
   static constexpr bool DIRECT = DMA || RING;
-  static constexpr bool BIAS_IN_LDS = !DMA || DMA_BYTES + NW * 1024 <= 160 * 1024;
-  static constexpr int BIAS_OFF = DMA ? DMA_BYTES : NS * STAGE_BYTES;  // one 1 KiB bias slot per wave
-  static constexpr int LDS_BYTES = BIAS_OFF + (BIAS_IN_LDS ? NW * 1024 : 0);
+  static constexpr int LDS_BYTES = DMA ? DMA_BYTES : NS * STAGE_BYTES;
   static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
   static_assert(DMA ? NW * EPI_WAVE_BYTES <= A_BYTES : NW * EPI_WAVE_BYTES <= STAGE_BYTES,
                 "the epilogue windows live inside one stage (one A slot)");
@@ -120,22 +118,14 @@ __device__ __forceinline__ TileCoord locate(const GemmTable& tab, int lid) {
 }
 
 // One wave-wide direct-to-LDS copy: lane l's 16 bytes at base + voff land at LDS byte address
-// lds_addr + 16*l.  Only used for the bias slots.  Inline assembly, so the compiler's wait-count
+// lds_addr + lds_off + 16*l; the sum is formed in M0 itself (one scalar instruction less per request than adding
+// first and moving the result: a slab is 16 requests per wave).  Inline assembly, so the compiler's wait-count
 // insertion does not see it: an extra operation in flight only makes the waits it computes for its own
 // loads stricter than needed.
 // Every direct-to-LDS request is issued at agent scope (sc1), which the CU's L1 never serves.  The kernels wait
 // for "all but the newest n" requests and rely on completion in issue order; a request that hits in L1 completes
 // ahead of older misses (measured: a ragged tile, whose out-of-range lanes all read the problem's last row, then
 // multiplied a slab that had not landed).  From L2, hits and misses complete in issue order.
-__device__ __forceinline__ void lds_dma16(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
-               :
-               : "s"(lds_addr_uniform), "v"(voff), "s"(base_uniform)
-               : "m0");
-}
-
-// The same with the LDS address given as a uniform base plus a uniform offset: the sum is formed in M0 itself, one
-// scalar instruction less per request than adding first and moving the result (a slab is 16 requests per wave).
 __device__ __forceinline__ void lds_dma16_sum(const unsigned char* base_uniform, unsigned voff, unsigned lds_addr_uniform,
                                               unsigned lds_off_uniform) {
   asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
@@ -263,18 +253,23 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
   };
   auto read_frags = [&](const unsigned char* sbase, int ks, int buf) { read_frags2(sbase, sbase + C::A_BYTES, ks, buf); };
 
-  // Bias of a tile: every wave copies the 32*TN bias values of its own columns (8 per lane, lanes past the
-  // end clamped) into a private LDS slot when it starts the tile; the copy is older than the loads of the
-  // tile's second slab, so the waits for those cover it.  A problem without bias copies from its B
-  // operand and ignores the result.
-  const unsigned char* bias_slot = lds + C::BIAS_OFF + wave * 1024;
-  const unsigned bias_lds = __builtin_amdgcn_readfirstlane(lds_address(lds)) + C::BIAS_OFF + wave * 1024;
-  auto issue_bias = [&](const TileCoord& tc) {
+  // The bias enters through the accumulators: a tile's accumulators start as bias (x) ones -- one MFMA per 32-column
+  // block, whose A operand holds bias[n] at k = 0 and whose B operand holds 1 at k = 0 -- instead of zero.  The
+  // epilogue then needs neither bias registers (the 256 x 256 shape could only find its 32 by spilling accumulators)
+  // nor an LDS slot, and every shape forms bias + sum of products in the same order, so results do not depend on the
+  // shape a problem is given.  Lane l < 32 fetches the bias of column l of each of the wave's column blocks; the
+  // values of the next tile are requested at the start of the current tile's epilogue, in front of its stores.
+  unsigned short bnext[TN];
+  auto fetch_bias = [&](const TileCoord& tc) {
     const hdit_gemm_problem& pr = tab.p[tc.pi];
-    const unsigned char* src = pr.bias ? (const unsigned char*)pr.bias : (const unsigned char*)pr.b;
-    if constexpr (C::BIAS_IN_LDS) lds_dma16(src, (unsigned)(min(tc.n0 + wn0 + lane * 8, pr.n - 8) * 2), bias_lds);
+    const unsigned short* bsrc = (const unsigned short*)pr.bias;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      bnext[j] = 0;
+      if (bsrc) bnext[j] = bsrc[min(tc.n0 + wn0 + j * 32 + l32, pr.n - 1)];
+    }
   };
-  issue_bias(locate<C>(tab, lid));
+  fetch_bias(locate<C>(tab, lid));
 
   // prologue: slab 0 into stage 0, slab 1 into the registers
   p_setup();
@@ -333,17 +328,24 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
     const int KT = pr.k / BK;
     if (!first_tile) {
       __syncthreads();  // every wave has left the previous epilogue, whose staging windows the next writes reuse
-      issue_bias(tc);
     }
     first_tile = false;
 
     f32x16 acc[TM][TN];
+    {
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      i32x4 ones_bits = {lh == 0 ? 0x3f80 : 0, 0, 0, 0};  // bf16 1.0 at k = 0 (lanes < 32 hold k = 0..7)
+      bf16x8 ones;
+      __builtin_memcpy(&ones, &ones_bits, 16);
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+      for (int j = 0; j < TN; j++) {
+        i32x4 bb = {lh == 0 ? (int)bnext[j] : 0, 0, 0, 0};
+        bf16x8 bfr;
+        __builtin_memcpy(&bfr, &bb, 16);
 #pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+        for (int i = 0; i < TM; i++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr, ones, zero, 0, 0, 0);
+      }
+    }
 
     // One k-step: the MFMAs on fragment buffer `buf`.  Under them, pinned in this order: two reads per MFMA
     // of the fragments the next k-step needs (an MFMA goes first, so that its wait for its own fragments
@@ -469,9 +471,6 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
                                     : (stage ^ 1) * C::STAGE_BYTES);
 
     // ---- epilogue ---------------------------------------------------------
-    // register-staged shapes: the bias copy is only known to have landed after the second slab's loads
-    // (direct-to-LDS shapes: the wait before every slab's barrier covers it)
-    if (!C::DMA && KT < 2) __builtin_amdgcn_s_waitcnt(0x0f70);
     auto epilogue = [&](auto mode_tag) {
       constexpr int MODE = decltype(mode_tag)::value;
       constexpr bool GATED = MODE == HDIT_EPI_GATE_RESIDUAL;
@@ -488,7 +487,6 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
       const int M = pr.m, N = pr.n;
       const int ldc = (int)pr.ldc, ldr = (int)pr.ldr;
       const int ncol0 = tc.n0 + wn0;
-      const int bias_mask = pr.bias ? -1 : 0;  // the slot holds unrelated data when the problem has no bias
 
       // Write-back layout: 16 lanes cover one 256-byte row segment, a wave covers 4 rows per pass, 8 passes
       // per 32-row block, done as two halves of 4.  The residual rows and the gate columns are requested one
@@ -528,14 +526,10 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
         gte0 = *(const f32x4*)g;
         gte1 = *(const f32x4*)(g + 4);
       };
-      i32x4 breg[C::BIAS_IN_LDS ? 1 : 2 * TN];  // the bias of this lane's columns when it has no LDS slot
-      if constexpr (!C::BIAS_IN_LDS) {
-#pragma unroll
-        for (int c = 0; c < 2 * TN; c++) {
-          const int col = min(ncol0 + ((c >> 1) * 4 + 2 * (c & 1) + lh) * 8, N - 8);
-          breg[c] = i32x4{0, 0, 0, 0};
-          if (pr.bias) breg[c] = *(const i32x4*)((const unsigned char*)pr.bias + (unsigned)(col * 2));
-        }
+      {
+        // bias of the next tile of this workgroup (this tile's is inside its accumulators: see the tile start)
+        const int next_lid = lid + wgs_per_xcd;
+        if (next_lid < xcd_end) fetch_bias(locate<C>(tab, next_lid));
       }
       if (GATED) {
         prefetch_rows(0, 0);
@@ -560,7 +554,7 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
           for (int gp = 0; gp < 2; gp++) {
             // accumulator groups g = 2gp (even) and 2gp+1 (odd) hold columns 8g + 4*lh + e.  After the swap
             // lanes < 32 own the 8 columns of the even group, lanes >= 32 those of the odd group.
-            float v[8], bf[8];
+            float v[8];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
               auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(acc[i][j][(2 * gp) * 4 + e]),
@@ -569,10 +563,6 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
               v[4 + e] = __int_as_float(sw[1]);
             }
             const int chunk = j * 4 + 2 * gp + lh;  // 16-byte chunk inside the wave's 256-byte row
-            if constexpr (C::BIAS_IN_LDS) hdit::unpack8(*(const i32x4*)(bias_slot + (chunk << 4)) & bias_mask, bf);
-            else hdit::unpack8(breg[j * 2 + gp], bf);
-#pragma unroll
-            for (int e = 0; e < 8; e++) v[e] += bf[e];
             if (MODE == HDIT_EPI_BIAS_GELU) {
 #pragma unroll
               for (int e = 0; e < 8; e++) v[e] = hdit::gelu_tanh_f(v[e]);

@@ -60,6 +60,31 @@ def test_gemm_ragged_tile_with_operands_out_of_the_caches(hdit, m, cfg):
         lib.hdit_gemm_force_config(-1)
 
 
+@pytest.mark.parametrize("epi", ["bias", "gelu", "nobias"])
+def test_gemm_result_does_not_depend_on_the_tile_shape(hdit, epi):
+    """Every tile shape forms bias + sum of products in the same order (the bias initialises the accumulators, the
+    k-steps follow), so the shape the planner gives a problem does not change a single bit of its result: launch
+    forms that split or group problems differently (one stream, two streams, merged fronts) can be compared for
+    equality."""
+    print(f"gemm shape independence epi={epi}", flush=True)
+    lib = hdit._lib.lib()
+    m, n, k = 777, 1536, 1536
+    a, w, b = g(rnd(m, k, seed=1)), g(rnd(n, k, scale=0.05, seed=2)), g(rnd(n, seed=3))
+    outs = []
+    try:
+        for cfg in (0, 1, 2, 3, 4):
+            lib.hdit_gemm_force_config(cfg)
+            out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+            hdit.ops.gemm_launch([hdit.ops.gemm_problem(a, w, out, None if epi == "nobias" else b,
+                                                        hdit.ops.EPI_BIAS_GELU if epi == "gelu" else hdit.ops.EPI_BIAS)])
+            torch.cuda.synchronize()
+            outs.append(out)
+    finally:
+        lib.hdit_gemm_force_config(-1)
+    for cfg, out in enumerate(outs[1:], start=1):
+        assert torch.equal(out, outs[0]), f"shape {cfg} differs from shape 0"
+
+
 def test_gemm_gelu_and_gate_residual_grouped(hdit):
     B, T1, T2, D, F = 2, 320, 77, 256, 512
     x1, x2 = rnd(B, T1, D), rnd(B, T2, D)
