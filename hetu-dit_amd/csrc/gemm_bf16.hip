@@ -192,12 +192,17 @@ __device__ __forceinline__ void run_tiles(const GemmTable& tab, int total_tiles,
 #pragma unroll
     for (int i = 0; i < C::A_LOADS; i++) {
       const int gr = min(tc.m0 + (wave + i * NW) * 8 + ld_row, pr.m - 1);
-      p_off[i] = (unsigned)(((int64_t)gr * pr.lda + src_chunk * 8) * 2);
+      unsigned row_off = (unsigned)gr * (unsigned)pr.lda;  // byte offsets stay below 2^32: checked on the host
+      asm volatile("" : "+v"(row_off));  // a product of its own: fused with the addition it is a 64-bit multiply-add,
+                                         // and the offsets then occupy register pairs for the whole kernel
+      p_off[i] = (row_off + (unsigned)(src_chunk * 8)) * 2u;
     }
 #pragma unroll
     for (int i = 0; i < C::B_LOADS; i++) {
       const int gr = min(tc.n0 + (wave + i * NW) * 8 + ld_row, pr.n - 1);
-      p_off[C::A_LOADS + i] = (unsigned)(((int64_t)gr * pr.ldb + src_chunk * 8) * 2);
+      unsigned row_off = (unsigned)gr * (unsigned)pr.ldb;
+      asm volatile("" : "+v"(row_off));
+      p_off[C::A_LOADS + i] = (row_off + (unsigned)(src_chunk * 8)) * 2u;
     }
   };
   // Once the stream is exhausted the last slab is simply loaded again and written to a stage nobody
