@@ -364,6 +364,12 @@ __device__ __forceinline__ void attn_tracked_body(const AttnParams& P, int q_til
     };
     if constexpr (L::Q_IN_LDS) mask_scores();
     else scores_from_registers();
+    if constexpr (FOLD) {
+      // Both key blocks start from the reference vectors.  Reading them once more here keeps them alive past the
+      // second block's first MFMA, which the compiler otherwise ties to a copy of them (16 v_mov_b64 per tile)
+      // instead of naming them as its addend the way the first block's does.
+      asm volatile("" : : "v"(negm[0]), "v"(negm[1]));
+    }
 
     // ---- online softmax in the log2 domain.  A lane owns one query column per qb and 32 of its 64 keys;
     // the other 32 live in lane^32.
