@@ -38,13 +38,17 @@ def sample_rows(m, count, seed):
     return idx
 
 
-# (image rows, text rows, n, k, epilogue): the four GEMM calls of an SD3 joint block at configs[1], the QKV+MLP
-# call of a Flux single block at configs[2], the FF1 call of a CogVideoX block at configs[4]
+# (image rows, text rows, n, k, epilogue): the four GEMM calls of an SD3 joint block at configs[1], the
+# out-projection and second MLP call of a PipeFusion patch at configs[3] (2048 image rows: the planner gives them the
+# 128x128 ring alone, with 24 and 96 slabs per tile), the QKV+MLP call of a Flux single block at configs[2], the FF1
+# call of a CogVideoX block at configs[4]
 GEMM_CASES = [
     (8192, 666, 4608, 1536, "bias"),
     (8192, 666, 1536, 1536, "gate"),
     (8192, 666, 6144, 1536, "gelu"),
     (8192, 666, 1536, 6144, "gate"),
+    (2048, 0, 1536, 1536, "gate"),
+    (2048, 0, 1536, 6144, "gate"),
     (4608, 0, 9216, 3072, "bias"),
     (17776, 0, 12288, 3072, "gelu"),
 ]
